@@ -1,0 +1,178 @@
+/*
+ * omni_dit.h — flat C ABI of libomni_dit_hip.so: the MI355X (gfx950) kernels under the per-step
+ * DiT transformer-block forward of vLLM-Omni's diffusion stack.
+ *
+ * Conventions
+ *   - Every pointer except `stream` is a DEVICE pointer owned by the caller. No entry point
+ *     allocates, frees or synchronises; all work is enqueued on `stream` (a hipStream_t; NULL = the
+ *     legacy default stream).
+ *   - Tensors are row-major with the innermost dimension contiguous. Strides are in ELEMENTS.
+ *   - `dtype` is one of ODIT_BF16 / ODIT_F16 / ODIT_F32 and names the element type of the activation
+ *     tensors. Arithmetic inside every kernel is fp32.
+ *   - Return value: 0 on success, a negative ODIT_E* code on failure; odit_last_error() then returns a
+ *     thread-local, NUL-terminated description. Argument errors are detected on the host BEFORE any
+ *     launch, so a failing call enqueues nothing.
+ *   - Re-entrant; no global mutable state apart from the thread-local error string.
+ *
+ * The reference (Flink-ddd/vllm-omni) is pure Python and has no FFI of its own for this path; each
+ * entry point below replaces the third-party kernel call(s) made at the cited reference lines.
+ */
+#ifndef OMNI_DIT_H_
+#define OMNI_DIT_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ODIT_VERSION 100 /* major*10000 + minor*100 + patch */
+
+enum odit_dtype { ODIT_BF16 = 0, ODIT_F16 = 1, ODIT_F32 = 2 };
+
+enum odit_status {
+  ODIT_OK = 0,
+  ODIT_EINVAL = -1,   /* bad shape / stride / alignment / null pointer            */
+  ODIT_ENOTSUP = -2,  /* valid request this build has no kernel for               */
+  ODIT_ELAUNCH = -3,  /* hipLaunchKernel / hipGetLastError reported a failure     */
+  ODIT_EWORKSPACE = -4 /* caller workspace too small                              */
+};
+
+/* Flag bits shared by the elementwise entry points. */
+#define ODIT_FLAG_REF_ROUNDING 1u /* round intermediates to `dtype` at the points where the reference's
+                                     op-by-op torch path does (makes bf16 results track the reference
+                                     bit-for-bit up to reduction order); default is one final rounding */
+#define ODIT_FLAG_NEOX 2u         /* rotary: rotate (i, i+rot/2) pairs instead of (2i, 2i+1)            */
+
+int odit_version(void);
+const char* odit_last_error(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * K1  joint (text+image) non-causal flash attention:  o = softmax(q k^T * scale [+ key mask]) v
+ *
+ * Replaces torch.nn.functional.scaled_dot_product_attention at
+ *   vllm_omni/diffusion/attention/backends/sdpa.py:82-90
+ * and aiter/flash-attn `flash_attn_func` at
+ *   vllm_omni/diffusion/attention/backends/flash_attn.py:105-111, utils/fa.py:24-32
+ * behind AttentionImpl.forward_hip (backends/abstract.py:132-140).
+ *
+ * q [B,Sq,H,D], k,v [B,Sk,Hkv,D], o [B,Sq,H,D]; layout BSHD as the reference passes them; each
+ * tensor gives strides for (batch, seq, head); the D axis must be contiguous, every stride a
+ * multiple of 8 elements and every base pointer 16-byte aligned. H % Hkv == 0 (grouped KV).
+ * key_mask: NULL, or uint8 [B,Sk] (row stride Sk); keys with mask == 0 are excluded, matching the
+ *   [B,Sk] boolean key-padding mask of flash_attn.py:80-102. A row whose keys are all excluded
+ *   returns zeros.
+ * lse: NULL, or float [B,H,Sq] receiving log(sum exp(scale*q.k)) per row (natural log).
+ * dtype: ODIT_BF16 or ODIT_F16 (fp32 never reaches a backend: attention/layer.py:134-140).
+ * D in {64, 128}.
+ */
+int odit_attn_fwd(const void* q, const void* k, const void* v, void* o, const uint8_t* key_mask,
+                  float* lse, int B, int Sq, int Sk, int H, int Hkv, int D,
+                  const int64_t q_strides[3], const int64_t k_strides[3],
+                  const int64_t v_strides[3], const int64_t o_strides[3], float scale, int dtype,
+                  void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * K2  fused QK-RMSNorm + rotary embedding + scatter into the joint [txt;img] sequence.
+ *
+ * Replaces, in one pass over a fused-QKV projection output:
+ *   vLLM RMSNorm(head_dim) x2       vllm_omni/diffusion/models/qwen_image/qwen_image_transformer.py:588-591
+ *   RotaryEmbedding.forward x2      vllm_omni/diffusion/layers/rope.py:108-159 (interleaved: rope.py:12-36)
+ *   torch.cat([txt, img], dim=1) x3 qwen_image_transformer.py:603-606
+ * and, with norm_mode = ODIT_NORM_ROW, Wan's whole-row fp32 RMSNorm + apply_rotary_emb_wan
+ *   vllm_omni/diffusion/models/wan2_2/wan2_2_transformer.py:34-56, 59-89, 406-420.
+ *
+ * q_in/k_in/v_in: [B,S,H,D] views (typically slices of one [B,S,3*H*D] GEMM output) addressed by
+ *   in_strides = (batch, seq) strides in elements, shared by the three; heads are D apart.
+ *   k_in and v_in may be NULL (then only q is processed); v is copied unchanged.
+ * q_out/k_out/v_out: [B,S_total,H,D] dense joint buffers; row s of the input lands in row
+ *   out_seq_offset + s. May alias the inputs only if layouts coincide exactly.
+ * wq, wk: RMSNorm weights, float32 or `dtype` per w_dtype; [D] for ODIT_NORM_HEAD, [H*D] for
+ *   ODIT_NORM_ROW; NULL = weight of ones. Ignored for ODIT_NORM_NONE.
+ * cos, sin: float32 [S, rot/2] tables (row stride rot/2), NULL = no rotation (identity).
+ *   rot <= D, rot % 8 == 0. Pair (x[2i], x[2i+1]) -> (x0*c - x1*s, x1*c + x0*s); with
+ *   ODIT_FLAG_NEOX pair (x[i], x[i+rot/2]).
+ * With ODIT_FLAG_REF_ROUNDING: normalised value rounded to `dtype` before the weight multiply
+ *   (vLLM RMSNorm order; skipped for ODIT_NORM_ROW whose reference keeps fp32), cos/sin rounded to
+ *   `dtype` (qwen_image_transformer.py:593-596) and the rotation evaluated in `dtype` steps.
+ */
+enum odit_norm_mode { ODIT_NORM_NONE = 0, ODIT_NORM_HEAD = 1, ODIT_NORM_ROW = 2 };
+
+int odit_qknorm_rope(const void* q_in, const void* k_in, const void* v_in, void* q_out, void* k_out,
+                     void* v_out, const void* wq, const void* wk, const float* cos, const float* sin,
+                     int B, int S, int H, int D, int rot, const int64_t in_strides[2],
+                     int out_seq_offset, int S_total, float eps, int norm_mode, int w_dtype,
+                     int dtype, unsigned flags, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * K3  fused LayerNorm (no affine, or fp32 affine) + adaLN shift/scale modulation:
+ *        out = LN(x) * (1 + scale) + shift
+ *
+ * Replaces nn.LayerNorm + mul + add in AdaLayerNorm.forward_native
+ *   vllm_omni/diffusion/layers/adalayernorm.py:23-60, 102-110
+ * (same arithmetic: QwenImageTransformerBlock._modulate qwen_image_transformer.py:710-744;
+ *  Flux norm2 + inline modulate flux_transformer.py:292-293; Wan FP32LayerNorm + modulate
+ *  wan2_2_transformer.py:659, 668-670).
+ *
+ * x, out: [B,S,C], x_strides/out_strides = (batch, seq) strides; C contiguous.
+ * shift, scale: element (b, c) at ptr[b*mod_stride_b + c]; NULL = 0. Type per mod_dtype (`dtype` or
+ *   ODIT_F32). `gate` is not touched here: the caller returns it as a view.
+ * index: NULL, or int32 [B,S] (row stride S): token (b,s) uses modulation row b when index == 0 and
+ *   row b + B otherwise (adalayernorm.py:31-54).
+ * ln_weight, ln_bias: NULL or float32 [C] (elementwise-affine LayerNorm, applied before modulation).
+ */
+int odit_adaln_modulate(const void* x, void* out, const void* shift, const void* scale,
+                        const int32_t* index, const float* ln_weight, const float* ln_bias, int B,
+                        int S, int C, const int64_t x_strides[2], const int64_t out_strides[2],
+                        int64_t mod_stride_b, float eps, int mod_dtype, int dtype, unsigned flags,
+                        void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * K4  gated residual:  out = h + gate * y     (gate broadcast over the sequence, or per token)
+ *
+ * Replaces the torch mul + add at qwen_image_transformer.py:794-795, 801, 806
+ * (Flux flux_transformer.py:289-290, 299-300, 362-364; Wan wan2_2_transformer.py:661, 673 with
+ *  fp32 gate). gate == NULL means gate of ones (plain residual, wan2_2_transformer.py:666).
+ *
+ * h, y, out: [B,S,C] with (batch, seq) strides; out may alias h.
+ * gate element (b,s,c) at gate[b*gate_strides[0] + s*gate_strides[1] + c]; type per gate_dtype.
+ */
+int odit_gated_residual(const void* h, const void* y, const void* gate, void* out, int B, int S,
+                        int C, const int64_t h_strides[2], const int64_t y_strides[2],
+                        const int64_t out_strides[2], const int64_t gate_strides[2], int gate_dtype,
+                        int dtype, unsigned flags, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * K5  TeaCache relative-L1 reduction, per batch row:
+ *        sums[b] = ( sum_i |cur[b,i] - prev[b,i]| , sum_i |prev[b,i]| )
+ *
+ * Replaces the six torch kernels of
+ *   vllm_omni/diffusion/cache/teacache/hook.py:214-221
+ * ((cur-prev).abs().mean() / (prev.abs().mean() + 1e-8)); the host divides and applies the
+ * polynomial. With ODIT_FLAG_REF_ROUNDING the difference is rounded to `dtype` before abs(), as
+ * torch does for a bf16 subtraction. Deterministic: fixed-shape two-stage tree, fp64 final stage.
+ *
+ * cur, prev: [B, n] with row strides cur_stride / prev_stride (elements); n % 8 == 0 not required.
+ * sums: double [B,2] on the device.
+ * workspace: device scratch of at least odit_rel_l1_workspace_bytes(B, n) bytes, 16-byte aligned.
+ */
+size_t odit_rel_l1_workspace_bytes(int B, int64_t n);
+int odit_rel_l1(const void* cur, const void* prev, double* sums, void* workspace,
+                size_t workspace_bytes, int B, int64_t n, int64_t cur_stride, int64_t prev_stride,
+                int dtype, unsigned flags, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Pointwise helpers on the block path.
+ *
+ * odit_gelu_tanh: out = 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) over n contiguous elements;
+ *   replaces F.gelu(approximate="tanh") at qwen_image_transformer.py:424.
+ * odit_silu: out = x * sigmoid(x); replaces nn.SiLU at qwen_image_transformer.py:682-685, 699-702.
+ */
+int odit_gelu_tanh(const void* x, void* out, int64_t n, int dtype, void* stream);
+int odit_silu(const void* x, void* out, int64_t n, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OMNI_DIT_H_ */

@@ -1,0 +1,22 @@
+"""CPU oracle for the DiT transformer-block hot path — TEST INFRASTRUCTURE ONLY.
+
+A clean-room, plain-PyTorch restatement (CPU, fp32 or the tensor dtype, one torch op per reference op,
+same dtype casts) of the reference's torch path for the per-step DiT block forward. Only ``tests/``,
+``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may import this package, and
+only as the checker or the timed CPU baseline; the product package never does.
+
+The reference (Flink-ddd/vllm-omni) is pure Python and cannot be imported where this runs (vllm and
+diffusers are absent), so there is no compiled ``oracle/_ref``. Each function cites the reference
+lines it follows. How each function is pinned independently of its own formula (closed forms,
+library routines, brute force, invariants) is listed in ``tests/test_oracle_*.py``.
+
+Parity status of arithmetic that lives in third-party wheels absent from the reference tree
+(**parity unpinned** at that boundary — upstream conventions adopted, not verifiable here):
+  * ``rms_norm_head``      vllm RMSNorm cast order (fp32 normalise -> cast -> x weight); vllm==0.16.0 / 0.14.0+rocm700
+  * ``ada_layer_norm_continuous``, ``timestep_embedding`` + ``TimestepEmbedding`` MLP,
+    ``flow_match_euler_step`` / sigma shifting    diffusers>=0.36.0 (AdaLayerNormContinuous chunk
+    order scale,shift; FlowMatchEulerDiscreteScheduler). ``timestep_embedding`` itself IS pinned by the
+    in-tree duplicate at pipeline_qwen_image.py:141-190.
+Everything else (attention, interleaved/NeoX rotary, AdaLayerNorm, gated residual, rel-L1, TeaCache
+decision logic, Qwen rope tables, block wiring, CFG combine) follows code present in the reference.
+"""

@@ -1,0 +1,82 @@
+"""The C-ABI library loads and exports exactly what include/omni_dit.h declares; argument errors are
+reported on the host before any launch (so these run without a GPU)."""
+
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from vllm_omni_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "omni_dit.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(odit_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    assert _declared_functions() == sorted(_lib.EXPORTED_SYMBOLS)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    for name in _declared_functions():
+        assert hasattr(lib, name), name
+    assert lib.odit_version() == 100
+
+
+def _strides(*v):
+    return _lib.i64_array(v)
+
+
+def test_argument_errors_are_caught_before_launch():
+    lib = _lib.load()
+    buf = C.create_string_buffer(4096)
+    p = C.addressof(buf)
+    p16 = (p + 15) & ~15
+    s3 = _strides(1024, 128, 128)
+    # unsupported head size
+    rc = lib.odit_attn_fwd(p16, p16, p16, p16, None, None, 1, 4, 4, 1, 1, 48, s3, s3, s3, s3, 0.1, 0, None)
+    assert rc == -2 and b"head size" in lib.odit_last_error()
+    # fp32 attention is not offered (the reference routes fp32 to SDPA)
+    rc = lib.odit_attn_fwd(p16, p16, p16, p16, None, None, 1, 4, 4, 1, 1, 64, s3, s3, s3, s3, 0.1, 2, None)
+    assert rc == -2
+    # misaligned pointer
+    rc = lib.odit_attn_fwd(p16 + 2, p16, p16, p16, None, None, 1, 4, 4, 1, 1, 64, s3, s3, s3, s3, 0.1, 0, None)
+    assert rc == -1 and b"aligned" in lib.odit_last_error()
+    # heads not divisible by kv heads
+    rc = lib.odit_attn_fwd(p16, p16, p16, p16, None, None, 1, 4, 4, 3, 2, 64, s3, s3, s3, s3, 0.1, 0, None)
+    assert rc == -1
+    # null pointers
+    rc = lib.odit_adaln_modulate(None, p16, None, None, None, None, None, 1, 1, 8, _strides(8, 8), _strides(8, 8),
+                                 8, 1e-6, 0, 0, 0, None)
+    assert rc == -1
+    # joint rows out of range
+    rc = lib.odit_qknorm_rope(p16, None, None, p16, None, None, None, None, None, None, 1, 4, 1, 64, 0,
+                              _strides(256, 64), 2, 4, 1e-6, 1, 0, 0, 0, None)
+    assert rc == -1 and b"do not fit" in lib.odit_last_error()
+    # workspace too small
+    assert lib.odit_rel_l1_workspace_bytes(2, 1 << 20) == 2 * 128 * 8
+    rc = lib.odit_rel_l1(p16, p16, p16, p16, 8, 2, 1 << 20, 1 << 20, 1 << 20, 0, 0, None)
+    assert rc == -4
+    # empty problems succeed without touching the device
+    assert lib.odit_gelu_tanh(None, None, 0, 0, None) == 0
+    assert lib.odit_gated_residual(p16, p16, None, p16, 0, 4, 8, _strides(32, 8), _strides(32, 8), _strides(32, 8),
+                                   None, 0, 0, 0, None) == 0
+
+
+def test_wrappers_refuse_cpu_tensors():
+    import torch
+
+    from vllm_omni_amd import kernels
+
+    x = torch.zeros(1, 4, 8, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        kernels.adaln_modulate(x, None, None)
+    with pytest.raises(RuntimeError, match="GPU"):
+        kernels.gelu_tanh(x)

@@ -1,0 +1,190 @@
+"""Host-side logic of the product package against the oracle and against closed forms (CPU only)."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from oracle import denoise as odn
+from oracle import teacache as otc
+from vllm_omni_amd import denoise
+from vllm_omni_amd.attention.backends.registry import DiffusionAttentionBackendEnum, register_diffusion_backend
+from vllm_omni_amd.attention.selector import get_attn_backend
+from vllm_omni_amd.cache.teacache.config import _MODEL_COEFFICIENTS, TeaCacheConfig
+from vllm_omni_amd.cache.teacache.hook import TeaCacheHook, rel_l1_from_sums
+from vllm_omni_amd.cache.teacache.state import TeaCacheState
+from vllm_omni_amd.hooks.base import HookRegistry, ModelHook, StateManager
+
+
+# ----------------------------------------------------------------------------------- TeaCache
+def test_coefficients_are_the_references():
+    for k, v in otc.COEFFICIENTS.items():
+        assert _MODEL_COEFFICIENTS[k] == v
+    assert TeaCacheConfig().rel_l1_thresh == 0.2
+    with pytest.raises(ValueError):
+        TeaCacheConfig(rel_l1_thresh=0.0)
+    with pytest.raises(KeyError):
+        TeaCacheConfig(transformer_type="Nope")
+    with pytest.raises(ValueError):
+        TeaCacheConfig(coefficients=[1.0, 2.0])
+
+
+def _run_decider(rels, coeffs, thresh):
+    hook = TeaCacheHook(TeaCacheConfig(rel_l1_thresh=thresh, coefficients=coeffs))
+    st = TeaCacheState()
+    out = []
+    for r in rels:
+        out.append(hook._decide(st, r))
+        st.cnt += 1
+    return out
+
+
+def test_decision_sequence_hand_built():
+    # |p(r)| = 0.1 per step with p(x) = x, threshold 0.25: compute, skip, skip, compute(reset), skip, skip, compute
+    coeffs = [0.0, 0.0, 0.0, 1.0, 0.0]
+    got = _run_decider([None] + [0.1] * 6, coeffs, 0.25)
+    assert got == [True, False, False, True, False, False, True]
+    # exact threshold hit computes (strict <)
+    assert _run_decider([None, 0.25], coeffs, 0.25) == [True, True]
+
+
+def test_decision_matches_oracle_on_random_trajectories():
+    rng = np.random.default_rng(0)
+    for name in ("QwenImageTransformer2DModel", "FluxTransformer2DModel"):
+        coeffs = otc.COEFFICIENTS[name]
+        for thresh in (0.1, 0.25, 0.6):
+            rels = [None] + list(rng.uniform(0.0, 0.35, size=40))
+            st = otc.BranchState()
+            ref = []
+            for r in rels:
+                ref.append(otc.decide(st, r, coeffs, thresh))
+                st.cnt += 1
+            assert _run_decider(rels, coeffs, thresh) == ref
+
+
+def test_rel_l1_from_sums_reproduces_torch_rounding():
+    g = torch.Generator().manual_seed(3)
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        prev = torch.randn(2048, generator=g).to(dtype)
+        cur = (prev.float() * 1.05 + 0.02 * torch.randn(2048, generator=g)).to(dtype)
+        want = ((cur - prev).abs().mean() / (prev.abs().mean() + 1e-8)).item()
+        sd = (cur - prev).abs().double().sum().item()
+        sp = prev.abs().double().sum().item()
+        got = rel_l1_from_sums(sd, sp, 2048, dtype)
+        assert got == pytest.approx(want, rel=1e-6 if dtype == torch.float32 else 0)
+
+
+# ----------------------------------------------------------------------------------- hooks
+class _Toy(nn.Module):
+    def forward(self, x, k=1):
+        return x * 2 + k
+
+
+def test_hook_registry_dispatch_rules():
+    m = _Toy()
+    reg = HookRegistry.get_or_create(m)
+    assert HookRegistry.get_or_create(m) is reg
+    assert m(3) == 7  # no hooks: original forward
+
+    class AddOne(ModelHook):
+        def post_forward(self, module, output):
+            return output + 1
+
+    class TimesTen(ModelHook):
+        def pre_forward(self, module, *args, **kwargs):
+            return (args[0] * 10,), kwargs
+
+    reg.register_hook("a", AddOne())
+    assert m(3) == 8
+    reg.register_hook("b", TimesTen())
+    assert m(3, k=0) == 61  # pre hooks in name order, post hooks reversed
+    reg.remove_hook("a")
+    reg.remove_hook("b")
+    assert m(3) == 7
+
+    class Replace(ModelHook):
+        def new_forward(self, module, *args, **kwargs):
+            return "replaced"
+
+    reg.register_hook("r", Replace())
+    assert m(1) == "replaced"
+
+
+def test_state_manager_contexts():
+    sm = StateManager(TeaCacheState)
+    sm.set_context("teacache_positive")
+    a = sm.get_state()
+    a.cnt = 5
+    sm.set_context("teacache_negative")
+    assert sm.get_state().cnt == 0
+    sm.set_context("teacache_positive")
+    assert sm.get_state() is a
+    sm.reset()
+    assert sm.get_state().cnt == 0
+
+
+# ----------------------------------------------------------------------------------- registry / selector
+def test_backend_registry_and_selector(monkeypatch):
+    E = DiffusionAttentionBackendEnum
+    with pytest.raises(ValueError, match="Unknown diffusion attention backend"):
+        E["NOPE"]
+    with pytest.raises(ValueError, match="must be registered"):
+        E.SAGE_ATTN.get_path()
+    assert E.FLASH_ATTN.get_class().get_name() == "HIP_FLASH_ATTN"
+    assert E.TORCH_SDPA.get_class().get_name() == "SDPA"
+    register_diffusion_backend(E.TORCH_SDPA, E.FLASH_ATTN.value)
+    try:
+        assert E.TORCH_SDPA.is_overridden() and E.TORCH_SDPA.get_class().get_name() == "HIP_FLASH_ATTN"
+    finally:
+        E.TORCH_SDPA.clear_override()
+    get_attn_backend.cache_clear()
+    assert get_attn_backend(-1).get_name() == "HIP_FLASH_ATTN"
+    get_attn_backend.cache_clear()
+    monkeypatch.setenv("DIFFUSION_ATTENTION_BACKEND", "TORCH_SDPA")
+    assert get_attn_backend(-1).get_name() == "SDPA"
+    get_attn_backend.cache_clear()
+    cls = get_attn_backend.__wrapped__(-1).get_impl_cls()
+    with pytest.raises(NotImplementedError):
+        from vllm_omni_amd.attention.backends.hip_flash import HipFlashAttentionImpl
+
+        HipFlashAttentionImpl(4, 64, 0.125, causal=True)
+    assert cls is not None
+
+
+# ----------------------------------------------------------------------------------- denoise harness
+def test_schedule_matches_oracle_and_closed_form():
+    for n, s in ((4, 256), (20, 4096), (28, 1024)):
+        a, b = denoise.flow_match_sigmas(n, s), odn.shifted_sigmas(n, s)
+        assert np.array_equal(a, b) and a[-1] == 0.0 and len(a) == n + 1
+        assert np.all(np.diff(a) < 0)
+    # mu endpoints: 0.5 at 256 tokens, 1.15 at 4096; sigma=1 is a fixed point of the shift
+    assert math.isclose(denoise.calculate_shift(256), 0.5) and math.isclose(denoise.calculate_shift(4096), 1.15)
+    assert denoise.flow_match_sigmas(10, 4096)[0] == 1.0
+    # shift formula at one interior point, by hand: s = 0.5, mu = 1.15 -> e/(e+1)
+    sig = denoise.flow_match_sigmas(2, 4096)
+    e = math.exp(1.15)
+    assert math.isclose(float(sig[1]), e / (e + 1.0), rel_tol=1e-6)
+
+
+def test_cfg_combine_and_euler_closed_forms():
+    g = torch.Generator().manual_seed(0)
+    pos, neg = torch.randn(1, 8, 4, generator=g), torch.randn(1, 8, 4, generator=g)
+    assert torch.allclose(denoise.combine_cfg_noise(pos, neg, 1.0), pos, atol=1e-6)
+    assert torch.allclose(denoise.combine_cfg_noise(pos, neg, 0.0), neg)
+    out = denoise.combine_cfg_noise(pos, neg, 4.0, cfg_normalize=True)
+    assert torch.allclose(out.norm(dim=-1), pos.norm(dim=-1), atol=1e-5)
+    assert torch.allclose(out, odn.combine_cfg(pos, neg, 4.0, True))
+    # Euler on a constant velocity field integrates exactly: x_end = x0 - v (sigma goes 1 -> 0)
+    sig = denoise.flow_match_sigmas(7, 1024)
+    x = torch.zeros(1, 3, 2)
+    v = torch.full((1, 3, 2), 2.5)
+    for i in range(7):
+        x = denoise.euler_step(x, v, float(sig[i]), float(sig[i + 1]))
+    assert torch.allclose(x, -v, atol=1e-5)
+    # Euler on the linear field v = x / sigma keeps x / sigma constant: x_i = x_0 * sigma_i
+    x = torch.ones(1, 2, 2)
+    for i in range(6):
+        x = denoise.euler_step(x, x / float(sig[i]), float(sig[i]), float(sig[i + 1]))
+        assert torch.allclose(x, torch.full_like(x, float(sig[i + 1])), atol=1e-5)

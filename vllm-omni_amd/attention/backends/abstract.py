@@ -1,0 +1,96 @@
+"""Attention backend ABI: same classes, method names and argument meaning as the reference's
+vllm_omni/diffusion/attention/backends/abstract.py:13-140."""
+
+from __future__ import annotations
+
+from abc import ABC, abstractmethod
+from dataclasses import dataclass
+from typing import Generic, TypeVar
+
+import torch
+
+from ...platforms import current_omni_platform
+
+
+class AttentionBackend(ABC):
+    """Class-level description of a backend; never instantiated (abstract.py:13-51)."""
+
+    accept_output_buffer: bool = False
+
+    @classmethod
+    def supports_attention_mask(cls) -> bool:
+        return False
+
+    @staticmethod
+    @abstractmethod
+    def get_name() -> str: ...
+
+    @staticmethod
+    @abstractmethod
+    def get_impl_cls() -> type["AttentionImpl"]: ...
+
+    @staticmethod
+    def get_metadata_cls() -> type["AttentionMetadata"]:
+        return AttentionMetadata
+
+    @staticmethod
+    def get_builder_cls():
+        raise NotImplementedError
+
+    @staticmethod
+    @abstractmethod
+    def get_supported_head_sizes() -> list[int]: ...
+
+    @classmethod
+    def supports_head_size(cls, head_size: int) -> bool:
+        sizes = cls.get_supported_head_sizes()
+        return (not sizes) or head_size in sizes
+
+
+@dataclass
+class AttentionMetadata:
+    """Per-call extras (abstract.py:54-66). ``attn_mask`` is a [B,Sk] key-padding mask; the joint_*
+    fields carry a replicated text segment for sequence-parallel strategies and are unused on one GPU."""
+
+    attn_mask: torch.Tensor | None = None
+    joint_attn_mask: torch.Tensor | None = None
+    joint_query: torch.Tensor | None = None
+    joint_key: torch.Tensor | None = None
+    joint_value: torch.Tensor | None = None
+    joint_strategy: str = "front"
+
+
+T = TypeVar("T", bound=AttentionMetadata)
+
+
+class AttentionImpl(ABC, Generic[T]):
+    """abstract.py:69-140: ``forward`` dispatches on the platform; on ROCm that is ``forward_hip``."""
+
+    @abstractmethod
+    def __init__(self, num_heads: int, head_size: int, softmax_scale: float, causal: bool = False,
+                 num_kv_heads: int | None = None, prefix: str = "", **extra_impl_args) -> None: ...
+
+    def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                attn_metadata: T | None = None) -> torch.Tensor:
+        plat = current_omni_platform
+        if plat.is_rocm():
+            return self.forward_hip(query, key, value, attn_metadata)
+        if plat.is_cuda():
+            return self.forward_cuda(query, key, value, attn_metadata)
+        if plat.is_npu():
+            return self.forward_npu(query, key, value, attn_metadata)
+        if plat.is_xpu():
+            return self.forward_xpu(query, key, value, attn_metadata)
+        raise NotImplementedError(f"No forward implementation for platform: {plat}")
+
+    def forward_cuda(self, query, key, value, attn_metadata=None):
+        raise NotImplementedError
+
+    def forward_npu(self, query, key, value, attn_metadata=None):
+        raise NotImplementedError
+
+    def forward_xpu(self, query, key, value, attn_metadata=None):
+        raise NotImplementedError
+
+    def forward_hip(self, query, key, value, attn_metadata=None):
+        return self.forward_cuda(query, key, value, attn_metadata)

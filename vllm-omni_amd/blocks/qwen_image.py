@@ -1,0 +1,374 @@
+"""Qwen-Image dual-stream MMDiT composed from the gfx950 kernels.
+
+Module tree, parameter names and call signatures follow
+vllm_omni/diffusion/models/qwen_image/qwen_image_transformer.py (``qit.py`` below) so a reference
+state dict loads unchanged (fused ``to_qkv`` / ``add_kv_proj`` as after its ``load_weights`` stacking,
+qit.py:1073-1113). Differences are all below the module interfaces:
+
+  * QK-RMSNorm + rotary + the three ``torch.cat([txt, img])`` copies are one fused pass per stream that
+    writes straight into the joint [B, S_txt+S_img, H, D] buffers (qit.py:588-606);
+  * adaLN LayerNorm+modulate and the gated residual are one pass each (qit.py:770-773, 794-806);
+  * GELU(tanh) runs in place on the MLP-up output (qit.py:424);
+  * dense projections are ``torch.nn.functional.linear`` (hipBLASLt MFMA GEMMs).
+"""
+
+from __future__ import annotations
+
+from functools import lru_cache
+from typing import Any
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .. import kernels
+from .._lib import ODIT_NORM_HEAD
+from ..attention.backends.abstract import AttentionMetadata
+from ..attention.layer import Attention
+from ..layers.adalayernorm import AdaLayerNorm
+from ..layers.rmsnorm import RMSNorm
+from ..layers.rope import RotaryEmbedding
+
+
+class Transformer2DModelOutput:
+    """Minimal stand-in for diffusers' output object: ``.sample`` and ``[0]`` both work."""
+
+    def __init__(self, sample: torch.Tensor):
+        self.sample = sample
+
+    def __getitem__(self, i: int):
+        return (self.sample,)[i]
+
+
+class SiLU(nn.Module):
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return kernels.silu(x)
+
+
+class ApproxGELU(nn.Module):
+    """Linear + GELU(tanh) (qit.py:399-424); the activation overwrites the projection output."""
+
+    def __init__(self, dim_in: int, dim_out: int, bias: bool = True):
+        super().__init__()
+        self.proj = nn.Linear(dim_in, dim_out, bias=bias)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        y = self.proj(x)
+        return kernels.gelu_tanh(y, out=y)
+
+
+class FeedForward(nn.Module):
+    """net.0 = Linear+GELU(tanh), net.1 = placeholder, net.2 = Linear (qit.py:427-466)."""
+
+    def __init__(self, dim: int, dim_out: int | None = None, mult: int = 4, inner_dim: int | None = None,
+                 bias: bool = True):
+        super().__init__()
+        inner = inner_dim or dim * mult
+        self.net = nn.ModuleList([ApproxGELU(dim, inner, bias=bias), nn.Identity(),
+                                  nn.Linear(inner, dim_out or dim, bias=bias)])
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        for m in self.net:
+            x = m(x)
+        return x
+
+
+class QwenEmbedRope(nn.Module):
+    """3-axis rotary tables with centred rows/columns (``scale_rope=True``), qit.py:298-396.
+    ``forward`` returns complex64 (vid_freqs, txt_freqs) like the reference; ``cos_sin`` returns the
+    float32 [S, D/2] tables the fused kernel reads, cached per (shape, device)."""
+
+    def __init__(self, theta: int, axes_dim: list[int], scale_rope: bool = True):
+        super().__init__()
+        self.theta, self.axes_dim, self.scale_rope = theta, list(axes_dim), scale_rope
+        pos = torch.arange(4096)
+        neg = torch.arange(4096).flip(0) * -1 - 1
+        self.pos_freqs = torch.cat([self.rope_params(pos, d, theta) for d in self.axes_dim], dim=1)
+        self.neg_freqs = torch.cat([self.rope_params(neg, d, theta) for d in self.axes_dim], dim=1)
+        self._tables = lru_cache(maxsize=16)(self._build)
+
+    @staticmethod
+    def rope_params(index: torch.Tensor, dim: int, theta: int = 10000) -> torch.Tensor:
+        assert dim % 2 == 0
+        inv = 1.0 / torch.pow(theta, torch.arange(0, dim, 2).to(torch.float32).div(dim))
+        ang = torch.outer(index.to(torch.float32), inv)
+        return torch.polar(torch.ones_like(ang), ang)
+
+    def _video_freqs(self, frame: int, height: int, width: int, idx: int = 0) -> torch.Tensor:
+        halves = [d // 2 for d in self.axes_dim]
+        fp = self.pos_freqs.split(halves, dim=1)
+        fn = self.neg_freqs.split(halves, dim=1)
+        f_t = fp[0][idx:idx + frame].view(frame, 1, 1, -1).expand(frame, height, width, -1)
+        if self.scale_rope:
+            rows = torch.cat([fn[1][-(height - height // 2):], fp[1][: height // 2]], dim=0)
+            cols = torch.cat([fn[2][-(width - width // 2):], fp[2][: width // 2]], dim=0)
+        else:
+            rows, cols = fp[1][:height], fp[2][:width]
+        f_h = rows.view(1, height, 1, -1).expand(frame, height, width, -1)
+        f_w = cols.view(1, 1, width, -1).expand(frame, height, width, -1)
+        return torch.cat([f_t, f_h, f_w], dim=-1).reshape(frame * height * width, -1).contiguous()
+
+    def _build(self, shapes: tuple[tuple[int, int, int], ...], txt_len: int, device: str):
+        vids, start = [], 0
+        for idx, (f, h, w) in enumerate(shapes):
+            vids.append(self._video_freqs(f, h, w, idx))
+            start = max(start, max(h // 2, w // 2) if self.scale_rope else max(h, w))
+        vid = torch.cat(vids, dim=0).to(device)
+        txt = self.pos_freqs[start:start + txt_len].to(device)
+        return vid, txt
+
+    @staticmethod
+    def _norm_shapes(video_fhw) -> tuple[tuple[int, int, int], ...]:
+        if isinstance(video_fhw, list) and video_fhw and isinstance(video_fhw[0], list):
+            video_fhw = video_fhw[0]  # per-sample list of shapes: the first sample's (qit.py:349-352)
+        if isinstance(video_fhw, tuple) and len(video_fhw) == 3 and all(isinstance(v, int) for v in video_fhw):
+            video_fhw = [video_fhw]
+        return tuple(tuple(int(v) for v in s) for s in video_fhw)
+
+    def forward(self, video_fhw, txt_seq_lens, device):
+        return self._tables(self._norm_shapes(video_fhw), int(max(txt_seq_lens)), str(device))
+
+
+class RotaryTables:
+    """Complex tables as the reference passes them between modules, plus float32 cos/sin views."""
+
+    def __init__(self, vid_freqs: torch.Tensor, txt_freqs: torch.Tensor):
+        self.vid_freqs, self.txt_freqs = vid_freqs, txt_freqs
+        self.img_cos, self.img_sin = vid_freqs.real.contiguous(), vid_freqs.imag.contiguous()
+        self.txt_cos, self.txt_sin = txt_freqs.real.contiguous(), txt_freqs.imag.contiguous()
+
+    def __iter__(self):  # unpacks like the reference's (vid_freqs, txt_freqs) tuple
+        return iter((self.vid_freqs, self.txt_freqs))
+
+    def __getitem__(self, i: int):
+        return (self.vid_freqs, self.txt_freqs)[i]
+
+
+class QwenImageCrossAttention(nn.Module):
+    """Joint text+image attention of one block (qit.py:469-661)."""
+
+    def __init__(self, dim: int, num_heads: int, head_dim: int, added_kv_proj_dim: int,
+                 out_bias: bool = True, eps: float = 1e-6, ref_rounding: bool = False):
+        super().__init__()
+        assert dim % num_heads == 0
+        self.dim, self.head_dim, self.total_num_heads, self.eps = dim, head_dim, num_heads, eps
+        inner = head_dim * num_heads
+        self.inner_dim = inner
+        self.to_qkv = nn.Linear(dim, 3 * inner, bias=True)
+        self.add_kv_proj = nn.Linear(added_kv_proj_dim, 3 * inner, bias=True)
+        self.query_num_heads = self.kv_num_heads = num_heads
+        self.norm_q = RMSNorm(head_dim, eps=eps)
+        self.norm_k = RMSNorm(head_dim, eps=eps)
+        self.norm_added_q = RMSNorm(head_dim, eps=eps)
+        self.norm_added_k = RMSNorm(head_dim, eps=eps)
+        self.to_out = nn.Linear(inner, dim, bias=out_bias)
+        self.to_add_out = nn.Linear(inner, dim, bias=out_bias)
+        self.attn = Attention(num_heads=num_heads, head_size=head_dim, softmax_scale=1.0 / (head_dim ** 0.5),
+                              causal=False, num_kv_heads=num_heads)
+        self.rope = RotaryEmbedding(is_neox_style=False)
+        self.ref_rounding = ref_rounding
+
+    def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, vid_freqs, txt_freqs=None,
+                hidden_states_mask: torch.Tensor | None = None,
+                encoder_hidden_states_mask: torch.Tensor | None = None):
+        tables = vid_freqs if isinstance(vid_freqs, RotaryTables) else RotaryTables(vid_freqs, txt_freqs)
+        B, S_img, _ = hidden_states.shape
+        S_txt = encoder_hidden_states.shape[1]
+        H, D = self.total_num_heads, self.head_dim
+        img_qkv = self.to_qkv(hidden_states).view(B, S_img, 3, H, D)
+        txt_qkv = self.add_kv_proj(encoder_hidden_states).view(B, S_txt, 3, H, D)
+        S = S_txt + S_img
+        jq = torch.empty((B, S, H, D), dtype=img_qkv.dtype, device=img_qkv.device)
+        jk = torch.empty_like(jq)
+        jv = torch.empty_like(jq)
+        rr = self.ref_rounding
+        kernels.qknorm_rope(txt_qkv[:, :, 0], txt_qkv[:, :, 1], txt_qkv[:, :, 2], jq, jk, jv,
+                            self.norm_added_q.weight, self.norm_added_k.weight, tables.txt_cos, tables.txt_sin,
+                            eps=self.eps, out_seq_offset=0, norm_mode=ODIT_NORM_HEAD, ref_rounding=rr)
+        kernels.qknorm_rope(img_qkv[:, :, 0], img_qkv[:, :, 1], img_qkv[:, :, 2], jq, jk, jv,
+                            self.norm_q.weight, self.norm_k.weight, tables.img_cos, tables.img_sin,
+                            eps=self.eps, out_seq_offset=S_txt, norm_mode=ODIT_NORM_HEAD, ref_rounding=rr)
+        meta = None
+        if hidden_states_mask is not None or encoder_hidden_states_mask is not None:
+            ones = lambda n: torch.ones((B, n), dtype=torch.bool, device=jq.device)  # noqa: E731
+            txt_m = encoder_hidden_states_mask if encoder_hidden_states_mask is not None else ones(S_txt)
+            img_m = hidden_states_mask if hidden_states_mask is not None else ones(S_img)
+            meta = AttentionMetadata(attn_mask=torch.cat([txt_m.bool(), img_m.bool()], dim=1))
+        joint = self.attn(jq, jk, jv, meta).flatten(2, 3)
+        img_out = self.to_out(joint[:, S_txt:, :])
+        txt_out = self.to_add_out(joint[:, :S_txt, :])
+        return img_out, txt_out
+
+
+class QwenImageTransformerBlock(nn.Module):
+    """One dual-stream block (qit.py:664-814); returns (encoder_hidden_states, hidden_states)."""
+
+    def __init__(self, dim: int, num_attention_heads: int, attention_head_dim: int, eps: float = 1e-6,
+                 zero_cond_t: bool = False, mlp_ratio: int = 4, ref_rounding: bool = False):
+        super().__init__()
+        self.dim = dim
+        self.num_attention_heads, self.attention_head_dim = num_attention_heads, attention_head_dim
+        self.img_mod = nn.Sequential(SiLU(), nn.Linear(dim, 6 * dim, bias=True))
+        self.img_norm1 = AdaLayerNorm(dim, elementwise_affine=False, eps=eps, ref_rounding=ref_rounding)
+        self.attn = QwenImageCrossAttention(dim=dim, num_heads=num_attention_heads, head_dim=attention_head_dim,
+                                            added_kv_proj_dim=dim, eps=eps, ref_rounding=ref_rounding)
+        self.img_norm2 = AdaLayerNorm(dim, elementwise_affine=False, eps=eps, ref_rounding=ref_rounding)
+        self.img_mlp = FeedForward(dim=dim, dim_out=dim, mult=mlp_ratio)
+        self.txt_mod = nn.Sequential(SiLU(), nn.Linear(dim, 6 * dim, bias=True))
+        self.txt_norm1 = AdaLayerNorm(dim, elementwise_affine=False, eps=eps, ref_rounding=ref_rounding)
+        self.txt_norm2 = AdaLayerNorm(dim, elementwise_affine=False, eps=eps, ref_rounding=ref_rounding)
+        self.txt_mlp = FeedForward(dim=dim, dim_out=dim, mult=mlp_ratio)
+        self.zero_cond_t = zero_cond_t
+        self.ref_rounding = ref_rounding
+
+    def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor,
+                encoder_hidden_states_mask: torch.Tensor | None, temb: torch.Tensor, image_rotary_emb,
+                joint_attention_kwargs: dict[str, Any] | None = None, modulate_index: torch.Tensor | None = None,
+                hidden_states_mask: torch.Tensor | None = None):
+        rr = self.ref_rounding
+        img_mod_params = self.img_mod(temb)
+        if self.zero_cond_t:
+            temb = torch.chunk(temb, 2, dim=0)[0]
+        txt_mod_params = self.txt_mod(temb)
+        img_mod1, img_mod2 = img_mod_params.chunk(2, dim=-1)
+        txt_mod1, txt_mod2 = txt_mod_params.chunk(2, dim=-1)
+
+        img_modulated, img_gate1 = self.img_norm1(hidden_states, img_mod1, modulate_index)
+        txt_modulated, txt_gate1 = self.txt_norm1(encoder_hidden_states, txt_mod1)
+        tables = image_rotary_emb if isinstance(image_rotary_emb, RotaryTables) else RotaryTables(*image_rotary_emb)
+        img_attn, txt_attn = self.attn(img_modulated, txt_modulated, tables,
+                                       hidden_states_mask=hidden_states_mask,
+                                       encoder_hidden_states_mask=encoder_hidden_states_mask)
+        # the block's inputs are never written: callers (TeaCache) keep them to form residuals
+        hidden_states = kernels.gated_residual(hidden_states, img_attn, img_gate1, ref_rounding=rr)
+        encoder_hidden_states = kernels.gated_residual(encoder_hidden_states, txt_attn, txt_gate1, ref_rounding=rr)
+
+        img_modulated2, img_gate2 = self.img_norm2(hidden_states, img_mod2, modulate_index)
+        hidden_states = kernels.gated_residual(hidden_states, self.img_mlp(img_modulated2), img_gate2,
+                                               out=hidden_states, ref_rounding=rr)
+        txt_modulated2, txt_gate2 = self.txt_norm2(encoder_hidden_states, txt_mod2)
+        encoder_hidden_states = kernels.gated_residual(encoder_hidden_states, self.txt_mlp(txt_modulated2),
+                                                       txt_gate2, out=encoder_hidden_states, ref_rounding=rr)
+        if encoder_hidden_states.dtype == torch.float16:
+            encoder_hidden_states = encoder_hidden_states.clip(-65504, 65504)
+        if hidden_states.dtype == torch.float16:
+            hidden_states = hidden_states.clip(-65504, 65504)
+        return encoder_hidden_states, hidden_states
+
+
+class TimestepEmbedding(nn.Module):
+    def __init__(self, in_channels: int, time_embed_dim: int):
+        super().__init__()
+        self.linear_1 = nn.Linear(in_channels, time_embed_dim)
+        self.linear_2 = nn.Linear(time_embed_dim, time_embed_dim)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.linear_2(kernels.silu(self.linear_1(x)))
+
+
+class QwenTimestepProjEmbeddings(nn.Module):
+    """Sinusoid(256 channels, cos first, scale 1000) -> MLP (qit.py:159-181)."""
+
+    def __init__(self, embedding_dim: int):
+        super().__init__()
+        self.timestep_embedder = TimestepEmbedding(256, embedding_dim)
+
+    @staticmethod
+    def time_proj(t: torch.Tensor, dim: int = 256, max_period: int = 10000, scale: float = 1000.0):
+        half = dim // 2
+        import math
+
+        freqs = torch.exp(-math.log(max_period) * torch.arange(half, dtype=torch.float32, device=t.device) / half)
+        arg = scale * (t[:, None].float() * freqs[None, :].to(t.dtype))
+        return torch.cat((torch.cos(arg), torch.sin(arg)), dim=-1)
+
+    def forward(self, timestep: torch.Tensor, hidden_states: torch.Tensor, addition_t_cond=None):
+        return self.timestep_embedder(self.time_proj(timestep).to(hidden_states.dtype))
+
+
+class AdaLayerNormContinuous(nn.Module):
+    """Final norm: (scale, shift) = Linear(SiLU(cond)).chunk(2); LN(x)(1+scale)+shift (qit.py:936, 1065)."""
+
+    def __init__(self, embedding_dim: int, conditioning_embedding_dim: int, eps: float = 1e-6):
+        super().__init__()
+        self.eps = eps
+        self.linear = nn.Linear(conditioning_embedding_dim, 2 * embedding_dim, bias=True)
+
+    def forward(self, x: torch.Tensor, cond: torch.Tensor) -> torch.Tensor:
+        emb = self.linear(kernels.silu(cond).to(x.dtype))
+        scale, shift = emb.chunk(2, dim=1)
+        return kernels.adaln_modulate(x, shift, scale, eps=self.eps)
+
+
+class QwenImageTransformer2DModel(nn.Module):
+    """Stem, N dual-stream blocks, head (qit.py:817-1071). ``prepare`` / ``run_blocks`` / ``finish``
+    are the three stages TeaCache needs to call separately (cache/teacache/extractors.py:147-279)."""
+
+    _repeated_blocks = ["QwenImageTransformerBlock"]
+
+    def __init__(self, patch_size: int = 2, in_channels: int = 64, out_channels: int | None = 16,
+                 num_layers: int = 60, attention_head_dim: int = 128, num_attention_heads: int = 24,
+                 joint_attention_dim: int = 3584, axes_dims_rope: tuple[int, int, int] = (16, 56, 56),
+                 mlp_ratio: int = 4, ref_rounding: bool = False):
+        super().__init__()
+        self.in_channels = in_channels
+        self.out_channels = out_channels or in_channels
+        self.inner_dim = num_attention_heads * attention_head_dim
+        self.pos_embed = QwenEmbedRope(theta=10000, axes_dim=list(axes_dims_rope), scale_rope=True)
+        self.time_text_embed = QwenTimestepProjEmbeddings(embedding_dim=self.inner_dim)
+        self.txt_norm = RMSNorm(joint_attention_dim, eps=1e-6)
+        self.img_in = nn.Linear(in_channels, self.inner_dim)
+        self.txt_in = nn.Linear(joint_attention_dim, self.inner_dim)
+        self.transformer_blocks = nn.ModuleList([
+            QwenImageTransformerBlock(self.inner_dim, num_attention_heads, attention_head_dim,
+                                      mlp_ratio=mlp_ratio, ref_rounding=ref_rounding)
+            for _ in range(num_layers)])
+        self.norm_out = AdaLayerNormContinuous(self.inner_dim, self.inner_dim, eps=1e-6)
+        self.proj_out = nn.Linear(self.inner_dim, patch_size * patch_size * self.out_channels, bias=True)
+        self.zero_cond_t = False
+        self.parallel_config = None
+        self.do_true_cfg = False
+
+    # -- stages ---------------------------------------------------------------------------------
+    def prepare(self, hidden_states, encoder_hidden_states, timestep, img_shapes, txt_seq_lens):
+        img = self.img_in(hidden_states)
+        timestep = timestep.to(device=img.device, dtype=img.dtype)
+        txt = self.txt_in(self.txt_norm(encoder_hidden_states))
+        temb = self.time_text_embed(timestep, img)
+        if txt_seq_lens is None:
+            txt_seq_lens = [encoder_hidden_states.shape[1]]
+        vid_freqs, txt_freqs = self.pos_embed(img_shapes, txt_seq_lens, device=img.device)
+        return img, txt, temb, RotaryTables(vid_freqs, txt_freqs)
+
+    def run_blocks(self, img, txt, temb, rotary, encoder_hidden_states_mask=None, attention_kwargs=None):
+        mask = encoder_hidden_states_mask
+        if mask is not None and bool(mask.all()):
+            mask = None  # all-true masks are dropped (qit.py:1044-1048)
+        for block in self.transformer_blocks:
+            txt, img = block(hidden_states=img, encoder_hidden_states=txt, encoder_hidden_states_mask=mask,
+                             temb=temb, image_rotary_emb=rotary, joint_attention_kwargs=attention_kwargs)
+        return img, txt
+
+    def finish(self, img, temb, return_dict: bool = True):
+        out = self.proj_out(self.norm_out(img, temb))
+        return Transformer2DModelOutput(sample=out) if return_dict else (out,)
+
+    def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor = None,
+                encoder_hidden_states_mask: torch.Tensor = None, timestep: torch.Tensor = None,
+                img_shapes=None, txt_seq_lens=None, guidance: torch.Tensor = None,
+                attention_kwargs: dict[str, Any] | None = None, additional_t_cond=None, return_dict: bool = True):
+        img, txt, temb, rotary = self.prepare(hidden_states, encoder_hidden_states, timestep, img_shapes, txt_seq_lens)
+        img, txt = self.run_blocks(img, txt, temb, rotary, encoder_hidden_states_mask, attention_kwargs)
+        return self.finish(img, temb, return_dict=return_dict)
+
+    # -- weights --------------------------------------------------------------------------------
+    def load_flat_state(self, weights: dict[str, torch.Tensor]) -> None:
+        """Load a flat name->tensor dict keyed with the reference's parameter names."""
+        own = dict(self.named_parameters())
+        missing = [k for k in own if k not in weights]
+        extra = [k for k in weights if k not in own]
+        if missing or extra:
+            raise KeyError(f"state mismatch: missing {missing[:4]}..., unexpected {extra[:4]}...")
+        with torch.no_grad():
+            for k, p in own.items():
+                p.copy_(weights[k].to(device=p.device, dtype=p.dtype))

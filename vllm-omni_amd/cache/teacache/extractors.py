@@ -1,0 +1,103 @@
+"""CacheContext and the extractor registry (vllm_omni/diffusion/cache/teacache/extractors.py:26-144,
+575-650), plus extractors for the transformers built in this package."""
+
+from __future__ import annotations
+
+from collections.abc import Callable
+from dataclasses import dataclass
+from typing import Any
+
+import torch
+import torch.nn as nn
+
+
+@dataclass
+class CacheContext:
+    """What a model-specific extractor hands to the generic hook.
+
+    modulated_input          tensor whose step-to-step change drives the skip decision
+    hidden_states            stem output entering the blocks
+    encoder_hidden_states    text stream for dual-stream models, else None
+    temb                     timestep embedding
+    run_transformer_blocks   () -> (hidden,) or (hidden, encoder) after all blocks
+    postprocess              hidden -> model output
+    run_transformer_blocks_rows  optional (rows: list[int]) -> same tuple for a subset of batch rows;
+                             lets a CFG-batched call recompute only the rows whose branch must compute
+    """
+
+    modulated_input: torch.Tensor
+    hidden_states: torch.Tensor
+    encoder_hidden_states: torch.Tensor | None
+    temb: torch.Tensor
+    run_transformer_blocks: Callable[[], tuple[torch.Tensor, ...]]
+    postprocess: Callable[[torch.Tensor], Any]
+    extra_states: dict[str, Any] | None = None
+    run_transformer_blocks_rows: Callable[[list[int]], tuple[torch.Tensor, ...]] | None = None
+
+    def validate(self) -> None:
+        for name in ("modulated_input", "hidden_states", "temb"):
+            if not isinstance(getattr(self, name), torch.Tensor):
+                raise TypeError(f"{name} must be torch.Tensor, got {type(getattr(self, name))}")
+        if self.encoder_hidden_states is not None and not isinstance(self.encoder_hidden_states, torch.Tensor):
+            raise TypeError(f"encoder_hidden_states must be torch.Tensor or None, got {type(self.encoder_hidden_states)}")
+        for name in ("run_transformer_blocks", "postprocess"):
+            if not callable(getattr(self, name)):
+                raise TypeError(f"{name} must be callable, got {type(getattr(self, name))}")
+        if self.modulated_input.shape[0] != self.hidden_states.shape[0]:
+            raise ValueError(f"Batch size mismatch: modulated_input has batch size {self.modulated_input.shape[0]}, "
+                             f"but hidden_states has {self.hidden_states.shape[0]}")
+        if self.modulated_input.device != self.hidden_states.device:
+            raise ValueError(f"Device mismatch: modulated_input on {self.modulated_input.device}, "
+                             f"hidden_states on {self.hidden_states.device}")
+
+
+def extract_qwen_context(module: nn.Module, hidden_states: torch.Tensor,
+                         encoder_hidden_states: torch.Tensor, encoder_hidden_states_mask: torch.Tensor | None = None,
+                         timestep: torch.Tensor | None = None, img_shapes=None, txt_seq_lens=None,
+                         guidance: torch.Tensor | None = None, additional_t_cond=None,
+                         attention_kwargs: dict[str, Any] | None = None, **kwargs: Any) -> CacheContext:
+    """Qwen-Image: stem, then block 0's img_norm1 on the stem output is the decision tensor
+    (extractors.py:147-279). ``module`` is this package's QwenImageTransformer2DModel."""
+    if not hasattr(module, "transformer_blocks") or len(module.transformer_blocks) == 0:
+        raise ValueError("Module must have transformer_blocks")
+    img, txt, temb, rotary = module.prepare(hidden_states, encoder_hidden_states, timestep, img_shapes, txt_seq_lens)
+    block0 = module.transformer_blocks[0]
+    mod1 = block0.img_mod(temb).chunk(2, dim=-1)[0]
+    modulated, _ = block0.img_norm1(img, mod1)
+    mask = encoder_hidden_states_mask
+    return_dict = kwargs.get("return_dict", True)
+
+    def run_rows(rows: list[int] | None):
+        if rows is None:
+            h, e, t, m = img, txt, temb, mask
+        else:
+            idx = torch.as_tensor(rows, device=img.device)
+            h, e, t = img.index_select(0, idx), txt.index_select(0, idx), temb.index_select(0, idx)
+            m = mask.index_select(0, idx) if mask is not None else None
+        h, e = module.run_blocks(h, e, t, rotary, m, attention_kwargs)
+        return (h, e)
+
+    def postprocess(h):
+        return module.finish(h, temb, return_dict=return_dict)
+
+    return CacheContext(modulated_input=modulated, hidden_states=img, encoder_hidden_states=txt, temb=temb,
+                        run_transformer_blocks=lambda: run_rows(None), postprocess=postprocess,
+                        run_transformer_blocks_rows=run_rows)
+
+
+EXTRACTOR_REGISTRY: dict[str, Callable] = {
+    "QwenImageTransformer2DModel": extract_qwen_context,
+}
+
+
+def register_extractor(transformer_cls_name: str, extractor_fn: Callable) -> None:
+    EXTRACTOR_REGISTRY[transformer_cls_name] = extractor_fn
+
+
+def get_extractor(transformer_cls_name: str) -> Callable:
+    try:
+        return EXTRACTOR_REGISTRY[transformer_cls_name]
+    except KeyError:
+        raise ValueError(
+            f"Unknown model type: '{transformer_cls_name}'. Available types: {list(EXTRACTOR_REGISTRY)}\n"
+            "To add support for a new model, use register_extractor() or add to EXTRACTOR_REGISTRY.") from None

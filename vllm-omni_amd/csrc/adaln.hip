@@ -1,0 +1,226 @@
+// K3: fused LayerNorm + adaLN shift/scale modulation, one 64-lane wavefront per token row.
+//
+// The row is read from HBM exactly once: each lane keeps NV 16-byte vectors of it in registers,
+// the two LayerNorm statistics are reduced across the wavefront with cross-lane shuffles (no LDS,
+// no barrier), and the modulated row is written back once. Algorithmic traffic is therefore
+// 2 * B*S*C * sizeof(T) (+ the [B,C] shift/scale rows, which stay L2-resident).
+#include "odit_common.h"
+
+namespace odit {
+
+template <typename TM> struct ModLoader {
+  // returns element c of a modulation row (or 0 when the pointer is null)
+  static __device__ __forceinline__ float at(const TM* p, int c) { return p ? to_float(p[c]) : 0.f; }
+};
+
+// N consecutive parameters starting at p (16-byte aligned, N * sizeof(TP) a multiple of 16),
+// fetched with 16-byte loads; `fill` when p is null.
+template <typename TP, int N>
+__device__ __forceinline__ void load_params(const TP* p, float fill, float (&dst)[N]) {
+  constexpr int E = Vec16<TP>::N;
+  static_assert(N % E == 0, "parameter run must be whole 16-byte vectors");
+  if (p == nullptr) {
+#pragma unroll
+    for (int j = 0; j < N; ++j) dst[j] = fill;
+    return;
+  }
+#pragma unroll
+  for (int q = 0; q < N / E; ++q) {
+    Vec16<TP> t = load16(p + q * E);
+#pragma unroll
+    for (int j = 0; j < E; ++j) dst[q * E + j] = to_float(t.e[j]);
+  }
+}
+
+template <typename T, typename TM, int NV, bool REF_ROUND>
+__global__ __launch_bounds__(256) void adaln_rows_kernel(
+    const T* __restrict__ x, T* __restrict__ out, const TM* __restrict__ shift,
+    const TM* __restrict__ scale, const int32_t* __restrict__ index,
+    const float* __restrict__ ln_w, const float* __restrict__ ln_b, int B, int S, int C,
+    int64_t xs_b, int64_t xs_s, int64_t os_b, int64_t os_s, int64_t mod_stride_b, float eps) {
+  constexpr int EPV = Vec16<T>::N;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= static_cast<int64_t>(B) * S) return;
+  const int b = static_cast<int>(row / S);
+  const int s = static_cast<int>(row - static_cast<int64_t>(b) * S);
+  const T* xr = x + b * xs_b + s * xs_s;
+  T* orow = out + b * os_b + s * os_s;
+
+  float v[NV][EPV];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c0 = (i * 64 + lane) * EPV;
+    if (c0 < C) {
+      Vec16<T> t = load16(xr + c0);
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) { v[i][j] = to_float(t.e[j]); sum += v[i][j]; }
+    } else {
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) v[i][j] = 0.f;
+    }
+  }
+  const float inv_c = 1.f / static_cast<float>(C);
+  const float mean = wave_sum(sum) * inv_c;
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c0 = (i * 64 + lane) * EPV;
+    if (c0 < C) {
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) { const float d = v[i][j] - mean; sq += d * d; }
+    }
+  }
+  const float rstd = rsqrtf(wave_sum(sq) * inv_c + eps);
+
+  int mrow = b;
+  if (index != nullptr && index[static_cast<int64_t>(b) * S + s] != 0) mrow = b + B;
+  const TM* sh = shift ? shift + mrow * mod_stride_b : nullptr;
+  const TM* sc = scale ? scale + mrow * mod_stride_b : nullptr;
+
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c0 = (i * 64 + lane) * EPV;
+    if (c0 < C) {
+      Vec16<T> o;
+      float scl_v[EPV], shf_v[EPV], lw_v[EPV], lb_v[EPV];
+      load_params<TM, EPV>(sc ? sc + c0 : nullptr, 0.f, scl_v);
+      load_params<TM, EPV>(sh ? sh + c0 : nullptr, 0.f, shf_v);
+      load_params<float, EPV>(ln_w ? ln_w + c0 : nullptr, 1.f, lw_v);
+      load_params<float, EPV>(ln_b ? ln_b + c0 : nullptr, 0.f, lb_v);
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) {
+        float y = (v[i][j] - mean) * rstd;
+        if (ln_w) y *= lw_v[j];
+        if (ln_b) y += lb_v[j];
+        const float scl = scl_v[j];
+        const float shf = shf_v[j];
+        float r;
+        if (REF_ROUND) {
+          // torch path: LN -> T, (1 + scale) -> T, product -> T, sum -> T
+          r = round_to<T>(round_to<T>(y) * round_to<T>(1.f + scl));
+          r = r + shf;
+        } else {
+          r = fmaf(y, 1.f + scl, shf);
+        }
+        o.e[j] = from_float<T>(r);
+      }
+      store16(orow + c0, o);
+    }
+  }
+}
+
+// Any C (no vector-width or register-cache constraint): the row is read three times through L2.
+template <typename T, typename TM, bool REF_ROUND>
+__global__ __launch_bounds__(256) void adaln_rows_generic_kernel(
+    const T* __restrict__ x, T* __restrict__ out, const TM* __restrict__ shift,
+    const TM* __restrict__ scale, const int32_t* __restrict__ index,
+    const float* __restrict__ ln_w, const float* __restrict__ ln_b, int B, int S, int C,
+    int64_t xs_b, int64_t xs_s, int64_t os_b, int64_t os_s, int64_t mod_stride_b, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= static_cast<int64_t>(B) * S) return;
+  const int b = static_cast<int>(row / S);
+  const int s = static_cast<int>(row - static_cast<int64_t>(b) * S);
+  const T* xr = x + b * xs_b + s * xs_s;
+  T* orow = out + b * os_b + s * os_s;
+  float sum = 0.f;
+  for (int c = lane; c < C; c += 64) sum += to_float(xr[c]);
+  const float inv_c = 1.f / static_cast<float>(C);
+  const float mean = wave_sum(sum) * inv_c;
+  float sq = 0.f;
+  for (int c = lane; c < C; c += 64) { const float d = to_float(xr[c]) - mean; sq += d * d; }
+  const float rstd = rsqrtf(wave_sum(sq) * inv_c + eps);
+  int mrow = b;
+  if (index != nullptr && index[static_cast<int64_t>(b) * S + s] != 0) mrow = b + B;
+  const TM* sh = shift ? shift + mrow * mod_stride_b : nullptr;
+  const TM* sc = scale ? scale + mrow * mod_stride_b : nullptr;
+  for (int c = lane; c < C; c += 64) {
+    float y = (to_float(xr[c]) - mean) * rstd;
+    if (ln_w) y *= ln_w[c];
+    if (ln_b) y += ln_b[c];
+    const float scl = ModLoader<TM>::at(sc, c);
+    const float shf = ModLoader<TM>::at(sh, c);
+    float r;
+    if (REF_ROUND) {
+      r = round_to<T>(round_to<T>(y) * round_to<T>(1.f + scl)) + shf;
+    } else {
+      r = fmaf(y, 1.f + scl, shf);
+    }
+    orow[c] = from_float<T>(r);
+  }
+}
+
+template <typename T, typename TM, bool REF_ROUND>
+static int launch_adaln(const void* x, void* out, const void* shift, const void* scale,
+                        const int32_t* index, const float* ln_w, const float* ln_b, int B, int S,
+                        int C, const int64_t* xs, const int64_t* os, int64_t mod_stride_b, float eps,
+                        hipStream_t stream) {
+  constexpr int EPV = Vec16<T>::N;
+  const int64_t rows = static_cast<int64_t>(B) * S;
+  const dim3 block(256);
+  const dim3 grid(static_cast<unsigned>((rows + 3) / 4));
+  constexpr int EPM = Vec16<TM>::N;
+  // EPV >= EPM always (TM is T or float), so C % EPV == 0 keeps parameter runs vector-aligned too.
+  const bool vec_ok = (C % EPV == 0) && aligned16(x) && aligned16(out) && xs[0] % EPV == 0 &&
+                      xs[1] % EPV == 0 && os[0] % EPV == 0 && os[1] % EPV == 0 &&
+                      aligned16(shift) && aligned16(scale) && mod_stride_b % EPM == 0 &&
+                      aligned16(ln_w) && aligned16(ln_b);
+  const int nv = (C + 64 * EPV - 1) / (64 * EPV);
+#define ODIT_ADALN_CASE(NVV)                                                                   \
+  hipLaunchKernelGGL((adaln_rows_kernel<T, TM, NVV, REF_ROUND>), grid, block, 0, stream,       \
+                     static_cast<const T*>(x), static_cast<T*>(out),                           \
+                     static_cast<const TM*>(shift), static_cast<const TM*>(scale), index, ln_w, \
+                     ln_b, B, S, C, xs[0], xs[1], os[0], os[1], mod_stride_b, eps)
+  if (vec_ok && nv <= 16) {
+    if (nv <= 1) ODIT_ADALN_CASE(1);
+    else if (nv <= 2) ODIT_ADALN_CASE(2);
+    else if (nv <= 4) ODIT_ADALN_CASE(4);
+    else if (nv <= 6) ODIT_ADALN_CASE(6);
+    else if (nv <= 8) ODIT_ADALN_CASE(8);
+    else if (nv <= 10) ODIT_ADALN_CASE(10);
+    else if (nv <= 12) ODIT_ADALN_CASE(12);
+    else ODIT_ADALN_CASE(16);
+  } else {
+    hipLaunchKernelGGL((adaln_rows_generic_kernel<T, TM, REF_ROUND>), grid, block, 0, stream,
+                       static_cast<const T*>(x), static_cast<T*>(out),
+                       static_cast<const TM*>(shift), static_cast<const TM*>(scale), index, ln_w,
+                       ln_b, B, S, C, xs[0], xs[1], os[0], os[1], mod_stride_b, eps);
+  }
+#undef ODIT_ADALN_CASE
+  return check_launch("odit_adaln_modulate");
+}
+
+}  // namespace odit
+
+extern "C" int odit_adaln_modulate(const void* x, void* out, const void* shift, const void* scale,
+                                   const int32_t* index, const float* ln_weight,
+                                   const float* ln_bias, int B, int S, int C,
+                                   const int64_t x_strides[2], const int64_t out_strides[2],
+                                   int64_t mod_stride_b, float eps, int mod_dtype, int dtype,
+                                   unsigned flags, void* stream) {
+  using namespace odit;
+  ODIT_CHECK_ARG(x && out, "odit_adaln_modulate: x/out must not be null");
+  ODIT_CHECK_ARG(x_strides && out_strides, "odit_adaln_modulate: strides must not be null");
+  ODIT_CHECK_ARG(B >= 0 && S >= 0 && C > 0, "odit_adaln_modulate: bad shape B=%d S=%d C=%d", B, S, C);
+  ODIT_CHECK_ARG(mod_dtype == dtype || mod_dtype == ODIT_F32,
+                 "odit_adaln_modulate: mod_dtype must equal dtype or be ODIT_F32 (got %d vs %d)",
+                 mod_dtype, dtype);
+  ODIT_CHECK_ARG(static_cast<int64_t>(B) * S < (1ll << 33), "odit_adaln_modulate: too many rows");
+  if (B == 0 || S == 0) return ODIT_OK;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool rr = (flags & ODIT_FLAG_REF_ROUNDING) && mod_dtype == dtype && dtype != ODIT_F32;
+#define ODIT_ADALN_GO(T, TM)                                                                     \
+  return rr ? launch_adaln<T, TM, true>(x, out, shift, scale, index, ln_weight, ln_bias, B, S, C, \
+                                        x_strides, out_strides, mod_stride_b, eps, st)           \
+            : launch_adaln<T, TM, false>(x, out, shift, scale, index, ln_weight, ln_bias, B, S, C, \
+                                         x_strides, out_strides, mod_stride_b, eps, st)
+  if (mod_dtype == dtype) {
+    ODIT_DISPATCH_DTYPE(dtype, T, ODIT_ADALN_GO(T, T));
+  } else {
+    ODIT_DISPATCH_DTYPE(dtype, T, ODIT_ADALN_GO(T, float));
+  }
+#undef ODIT_ADALN_GO
+  return ODIT_OK;
+}

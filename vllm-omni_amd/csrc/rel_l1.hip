@@ -1,0 +1,137 @@
+// K5: TeaCache relative-L1 reduction. One streaming read of `cur` and `prev`
+// (algorithmic traffic 2 * B*n * sizeof(T)), per-batch-row sums, fixed reduction tree:
+//   stage 1  grid (nblk, B): every block reduces one contiguous slice of one row to two fp32 partials
+//   stage 2  grid (B): one wavefront adds the row's partials in fp64 and writes sums[b] = {sum|cur-prev|, sum|prev|}
+// The tree depends only on (B, n), never on timing, so repeated calls give bit-identical sums.
+#include "odit_common.h"
+
+namespace odit {
+
+constexpr int kRelL1MaxBlocksPerRow = 1024;
+constexpr int kRelL1VecsPerThread = 4;
+
+static inline int rel_l1_blocks_per_row(int64_t n) {
+  // sized on bf16 vectors (8 elements); fp32 rows simply get twice the vectors per thread
+  const int64_t per_block = 256ll * kRelL1VecsPerThread * 8;
+  int64_t nb = (n + per_block - 1) / per_block;
+  if (nb < 1) nb = 1;
+  if (nb > kRelL1MaxBlocksPerRow) nb = kRelL1MaxBlocksPerRow;
+  return static_cast<int>(nb);
+}
+
+template <typename T, bool REF_ROUND>
+__global__ __launch_bounds__(256) void rel_l1_stage1_kernel(const T* __restrict__ cur,
+                                                            const T* __restrict__ prev,
+                                                            float* __restrict__ partials,
+                                                            int64_t n, int64_t n_vec,
+                                                            int64_t cur_stride, int64_t prev_stride) {
+  constexpr int EPV = Vec16<T>::N;
+  const int b = blockIdx.y;
+  const int nblk = gridDim.x;
+  const T* c = cur + b * cur_stride;
+  const T* p = prev + b * prev_stride;
+  // contiguous slice of vectors for this block
+  const int64_t per_blk = (n_vec + nblk - 1) / nblk;
+  const int64_t v_begin = static_cast<int64_t>(blockIdx.x) * per_blk;
+  const int64_t v_end = v_begin + per_blk < n_vec ? v_begin + per_blk : n_vec;
+  float sd = 0.f, sp = 0.f;
+  for (int64_t i = v_begin + threadIdx.x; i < v_end; i += blockDim.x) {
+    const Vec16<T> cv = load16(c + i * EPV);
+    const Vec16<T> pv = load16(p + i * EPV);
+#pragma unroll
+    for (int j = 0; j < EPV; ++j) {
+      const float pf = to_float(pv.e[j]);
+      float d = to_float(cv.e[j]) - pf;
+      if (REF_ROUND) d = round_to<T>(d);
+      sd += fabsf(d);
+      sp += fabsf(pf);
+    }
+  }
+  if (blockIdx.x == 0) {  // scalar tail (also the whole row when vector loads are not possible)
+    for (int64_t i = n_vec * EPV + threadIdx.x; i < n; i += blockDim.x) {
+      const float pf = to_float(p[i]);
+      float d = to_float(c[i]) - pf;
+      if (REF_ROUND) d = round_to<T>(d);
+      sd += fabsf(d);
+      sp += fabsf(pf);
+    }
+  }
+  sd = wave_sum(sd);
+  sp = wave_sum(sp);
+  __shared__ float red[2][4];
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) { red[0][wave] = sd; red[1][wave] = sp; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float* out = partials + (static_cast<int64_t>(b) * nblk + blockIdx.x) * 2;
+    out[0] = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
+    out[1] = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+  }
+}
+
+__global__ __launch_bounds__(64) void rel_l1_stage2_kernel(const float* __restrict__ partials,
+                                                           double* __restrict__ sums, int nblk) {
+  const int b = blockIdx.x;
+  const float* p = partials + static_cast<int64_t>(b) * nblk * 2;
+  double sd = 0.0, sp = 0.0;
+  for (int i = threadIdx.x; i < nblk; i += 64) { sd += p[2 * i]; sp += p[2 * i + 1]; }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    sd += __shfl_xor(sd, off, 64);
+    sp += __shfl_xor(sp, off, 64);
+  }
+  if (threadIdx.x == 0) { sums[2 * b] = sd; sums[2 * b + 1] = sp; }
+}
+
+template <typename T>
+static int launch_rel_l1(const void* cur, const void* prev, double* sums, float* partials, int B,
+                         int64_t n, int64_t cur_stride, int64_t prev_stride, bool ref_round,
+                         hipStream_t stream) {
+  constexpr int EPV = Vec16<T>::N;
+  const bool vec_ok = aligned16(cur) && aligned16(prev) && cur_stride % EPV == 0 &&
+                      prev_stride % EPV == 0;
+  const int64_t n_vec = vec_ok ? n / EPV : 0;
+  const int nblk = rel_l1_blocks_per_row(n);
+  const dim3 grid(nblk, B);
+  if (ref_round) {
+    hipLaunchKernelGGL((rel_l1_stage1_kernel<T, true>), grid, dim3(256), 0, stream,
+                       static_cast<const T*>(cur), static_cast<const T*>(prev), partials, n, n_vec,
+                       cur_stride, prev_stride);
+  } else {
+    hipLaunchKernelGGL((rel_l1_stage1_kernel<T, false>), grid, dim3(256), 0, stream,
+                       static_cast<const T*>(cur), static_cast<const T*>(prev), partials, n, n_vec,
+                       cur_stride, prev_stride);
+  }
+  int rc = check_launch("odit_rel_l1 (stage 1)");
+  if (rc != ODIT_OK) return rc;
+  hipLaunchKernelGGL(rel_l1_stage2_kernel, dim3(B), dim3(64), 0, stream, partials, sums, nblk);
+  return check_launch("odit_rel_l1 (stage 2)");
+}
+
+}  // namespace odit
+
+extern "C" size_t odit_rel_l1_workspace_bytes(int B, int64_t n) {
+  if (B <= 0 || n < 0) return 0;
+  return static_cast<size_t>(B) * odit::rel_l1_blocks_per_row(n) * 2 * sizeof(float);
+}
+
+extern "C" int odit_rel_l1(const void* cur, const void* prev, double* sums, void* workspace,
+                           size_t workspace_bytes, int B, int64_t n, int64_t cur_stride,
+                           int64_t prev_stride, int dtype, unsigned flags, void* stream) {
+  using namespace odit;
+  ODIT_CHECK_ARG(cur && prev && sums && workspace, "odit_rel_l1: null pointer argument");
+  ODIT_CHECK_ARG(B > 0 && B <= 65535 && n >= 0, "odit_rel_l1: bad shape B=%d n=%lld", B,
+                 static_cast<long long>(n));
+  ODIT_CHECK_ARG(aligned16(workspace), "odit_rel_l1: workspace must be 16-byte aligned");
+  if (workspace_bytes < odit_rel_l1_workspace_bytes(B, n)) {
+    set_error("odit_rel_l1: workspace has %zu bytes, needs %zu", workspace_bytes,
+              odit_rel_l1_workspace_bytes(B, n));
+    return ODIT_EWORKSPACE;
+  }
+  const bool rr = (flags & ODIT_FLAG_REF_ROUNDING) && dtype != ODIT_F32;
+  ODIT_DISPATCH_DTYPE(dtype, T,
+                      return launch_rel_l1<T>(cur, prev, sums, static_cast<float*>(workspace), B, n,
+                                              cur_stride, prev_stride, rr,
+                                              static_cast<hipStream_t>(stream)));
+  return ODIT_OK;
+}

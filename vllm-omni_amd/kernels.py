@@ -1,0 +1,344 @@
+"""Tensor-level wrappers over the C ABI of libomni_dit_hip.so.
+
+Each function validates on the host what the kernel assumes (device, dtype, contiguity of the last
+axis, alignment is checked again inside the library), passes raw device pointers, element strides and
+torch's current HIP stream, and raises if the library reports an error. Nothing here computes: a
+missing library or a CPU tensor is an error, never a fallback.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from ._lib import (
+    ODIT_BF16,
+    ODIT_F16,
+    ODIT_F32,
+    ODIT_FLAG_NEOX,
+    ODIT_FLAG_REF_ROUNDING,
+    ODIT_NORM_HEAD,
+    ODIT_NORM_NONE,
+    ODIT_NORM_ROW,
+)
+
+_DTYPE_CODE = {torch.bfloat16: ODIT_BF16, torch.float16: ODIT_F16, torch.float32: ODIT_F32}
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {t.dtype}; expected bfloat16, float16 or float32") from None
+
+
+def _dev(*tensors: torch.Tensor | None) -> None:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError(
+                "omni_dit HIP kernels need tensors on a GPU (got device "
+                f"{t.device}); there is no CPU path in this package"
+            )
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} and {t.device}")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _last_contig(t: torch.Tensor, name: str) -> None:
+    if t.stride(-1) != 1:
+        raise ValueError(f"{name}: last dimension must be contiguous (stride {t.stride(-1)})")
+
+
+# --------------------------------------------------------------------------------------------- K1
+def attn_fwd(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    scale: float,
+    key_mask: torch.Tensor | None = None,
+    return_lse: bool = False,
+):
+    """softmax(q k^T * scale) v for q [B,Sq,H,D], k/v [B,Sk,Hkv,D] (BSHD, bf16/fp16).
+
+    key_mask: optional [B,Sk] bool/uint8, False/0 = key excluded. Returns o [B,Sq,H,D]
+    (and lse [B,H,Sq] float32 when return_lse).
+    """
+    _dev(q, k, v, key_mask)
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("attn_fwd expects 4-D [B,S,H,D] tensors")
+    if not (q.dtype == k.dtype == v.dtype):
+        raise TypeError("q, k, v must share a dtype")
+    B, Sq, H, D = q.shape
+    Bk, Sk, Hkv, Dk = k.shape
+    if (Bk, Dk) != (B, D) or tuple(v.shape) != tuple(k.shape):
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
+
+    def _prep(t):
+        ok = t.stride(-1) == 1 and all(s % 8 == 0 for s in t.stride()[:3]) and t.data_ptr() % 16 == 0
+        return t if ok else t.contiguous()
+
+    q, k, v = _prep(q), _prep(k), _prep(v)
+    o = torch.empty((B, Sq, H, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device) if return_lse else None
+    mask_u8 = None
+    if key_mask is not None:
+        if tuple(key_mask.shape) != (B, Sk):
+            raise ValueError(f"key_mask must be [B,Sk]={B, Sk}, got {tuple(key_mask.shape)}")
+        mask_u8 = (key_mask != 0).to(torch.uint8).contiguous()
+    lib = _lib.load()
+    rc = lib.odit_attn_fwd(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), _ptr(mask_u8), _ptr(lse),
+        B, Sq, Sk, H, Hkv, D,
+        _lib.i64_array(q.stride()[:3]), _lib.i64_array(k.stride()[:3]),
+        _lib.i64_array(v.stride()[:3]), _lib.i64_array(o.stride()[:3]),
+        float(scale), _code(q), _stream(),
+    )
+    _lib.check(rc, "odit_attn_fwd")
+    return (o, lse) if return_lse else o
+
+
+# --------------------------------------------------------------------------------------------- K2
+def qknorm_rope(
+    q: torch.Tensor,
+    k: torch.Tensor | None,
+    v: torch.Tensor | None,
+    q_out: torch.Tensor,
+    k_out: torch.Tensor | None,
+    v_out: torch.Tensor | None,
+    wq: torch.Tensor | None,
+    wk: torch.Tensor | None,
+    cos: torch.Tensor | None,
+    sin: torch.Tensor | None,
+    *,
+    eps: float = 1e-6,
+    out_seq_offset: int = 0,
+    norm_mode: int = ODIT_NORM_HEAD,
+    neox: bool = False,
+    ref_rounding: bool = False,
+) -> None:
+    """RMS-normalise q,k (per head or per row), rotate them, and write q,k,v rows into joint buffers.
+
+    q,k,v: [B,S,H,D] views sharing (batch, seq) strides with heads D apart (e.g. the three slices of
+    a fused-QKV projection). *_out: dense [B,S_total,H,D]; input row s goes to row out_seq_offset+s.
+    cos/sin: float32 [S, rot/2] or None.
+    """
+    _dev(q, k, v, q_out, k_out, v_out, wq, wk, cos, sin)
+    if q.dim() != 4:
+        raise ValueError("qknorm_rope expects [B,S,H,D] inputs")
+    B, S, H, D = q.shape
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        if t is None:
+            continue
+        if tuple(t.shape) != (B, S, H, D) or t.dtype != q.dtype:
+            raise ValueError(f"{name}: expected shape {(B, S, H, D)} and dtype {q.dtype}")
+        if t.stride(3) != 1 or t.stride(2) != D:
+            raise ValueError(f"{name}: heads must be laid out D apart with a contiguous last axis")
+        if t.stride()[:2] != q.stride()[:2]:
+            raise ValueError(f"{name}: (batch, seq) strides must match q's")
+    S_total = q_out.shape[1]
+    for name, t, src in (("q_out", q_out, q), ("k_out", k_out, k), ("v_out", v_out, v)):
+        if (t is None) != (src is None):
+            raise ValueError(f"{name} must be given exactly when its input is")
+        if t is None:
+            continue
+        if tuple(t.shape) != (B, S_total, H, D) or t.dtype != q.dtype or not t.is_contiguous():
+            raise ValueError(f"{name}: expected dense {(B, S_total, H, D)} of {q.dtype}")
+    rot = 0
+    if cos is not None:
+        if sin is None or cos.shape != sin.shape or cos.dim() != 2 or cos.shape[0] != S:
+            raise ValueError("cos/sin must both be [S, rot/2]")
+        if cos.dtype != torch.float32 or sin.dtype != torch.float32:
+            raise TypeError("cos/sin must be float32")
+        cos, sin = cos.contiguous(), sin.contiguous()
+        rot = 2 * cos.shape[1]
+    w_dtype = _code(q)
+    if norm_mode != ODIT_NORM_NONE:
+        for name, w in (("wq", wq), ("wk", wk)):
+            if w is None:
+                continue
+            want = D if norm_mode == ODIT_NORM_HEAD else H * D
+            if w.numel() != want or not w.is_contiguous():
+                raise ValueError(f"{name}: expected {want} contiguous elements")
+        ws = [w for w in (wq, wk) if w is not None]
+        if ws:
+            if any(w.dtype != ws[0].dtype for w in ws):
+                raise TypeError("wq and wk must share a dtype")
+            w_dtype = _code(ws[0])
+    flags = (ODIT_FLAG_NEOX if neox else 0) | (ODIT_FLAG_REF_ROUNDING if ref_rounding else 0)
+    lib = _lib.load()
+    rc = lib.odit_qknorm_rope(
+        q.data_ptr(), _ptr(k), _ptr(v), q_out.data_ptr(), _ptr(k_out), _ptr(v_out),
+        _ptr(wq), _ptr(wk), _ptr(cos), _ptr(sin),
+        B, S, H, D, rot, _lib.i64_array(q.stride()[:2]), int(out_seq_offset), int(S_total),
+        float(eps), int(norm_mode), w_dtype, _code(q), flags, _stream(),
+    )
+    _lib.check(rc, "odit_qknorm_rope")
+
+
+# --------------------------------------------------------------------------------------------- K3
+def adaln_modulate(
+    x: torch.Tensor,
+    shift: torch.Tensor | None,
+    scale: torch.Tensor | None,
+    *,
+    eps: float = 1e-6,
+    index: torch.Tensor | None = None,
+    ln_weight: torch.Tensor | None = None,
+    ln_bias: torch.Tensor | None = None,
+    ref_rounding: bool = False,
+    out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """LayerNorm(x) * (1 + scale) + shift for x [B,S,C]; shift/scale [Bm,C] views of one modulation
+    tensor (Bm = B, or 2B with a per-token `index` [B,S] choosing row b or b+B)."""
+    _dev(x, shift, scale, index, ln_weight, ln_bias, out)
+    if x.dim() != 3:
+        raise ValueError("adaln_modulate expects x [B,S,C]")
+    B, S, Cdim = x.shape
+    _last_contig(x, "x")
+    mod_dtype = _code(x)
+    mod_stride = 0
+    rows_needed = 2 * B if index is not None else B
+    for name, t in (("shift", shift), ("scale", scale)):
+        if t is None:
+            continue
+        if t.dim() != 2 or t.shape[1] != Cdim or t.shape[0] < rows_needed:
+            raise ValueError(f"{name}: expected [{rows_needed},{Cdim}], got {tuple(t.shape)}")
+        _last_contig(t, name)
+        mod_dtype = _code(t)
+    if shift is not None and scale is not None:
+        if shift.dtype != scale.dtype or shift.stride(0) != scale.stride(0):
+            raise ValueError("shift and scale must share dtype and batch stride")
+    first = shift if shift is not None else scale
+    if first is not None:
+        mod_stride = first.stride(0) if first.shape[0] > 1 else first.shape[1]
+    if index is not None:
+        if tuple(index.shape) != (B, S):
+            raise ValueError(f"index must be [B,S]={B, S}")
+        index = index.to(torch.int32).contiguous()
+    for name, t in (("ln_weight", ln_weight), ("ln_bias", ln_bias)):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != Cdim or not t.is_contiguous()):
+            raise ValueError(f"{name}: expected contiguous float32 [{Cdim}]")
+    if out is None:
+        out = torch.empty((B, S, Cdim), dtype=x.dtype, device=x.device)
+    elif tuple(out.shape) != (B, S, Cdim) or out.dtype != x.dtype or out.stride(-1) != 1:
+        raise ValueError("out must match x in shape and dtype with a contiguous last axis")
+    lib = _lib.load()
+    rc = lib.odit_adaln_modulate(
+        x.data_ptr(), out.data_ptr(), _ptr(shift), _ptr(scale), _ptr(index), _ptr(ln_weight),
+        _ptr(ln_bias), B, S, Cdim, _lib.i64_array(x.stride()[:2]), _lib.i64_array(out.stride()[:2]),
+        int(mod_stride), float(eps), mod_dtype, _code(x),
+        ODIT_FLAG_REF_ROUNDING if ref_rounding else 0, _stream(),
+    )
+    _lib.check(rc, "odit_adaln_modulate")
+    return out
+
+
+# --------------------------------------------------------------------------------------------- K4
+def gated_residual(
+    h: torch.Tensor,
+    y: torch.Tensor,
+    gate: torch.Tensor | None,
+    *,
+    out: torch.Tensor | None = None,
+    ref_rounding: bool = False,
+) -> torch.Tensor:
+    """h + gate * y for h,y [B,S,C]; gate [B,C], [B,1,C] (broadcast over S) or [B,S,C]; None = ones."""
+    _dev(h, y, gate, out)
+    if h.dim() != 3 or tuple(y.shape) != tuple(h.shape) or y.dtype != h.dtype:
+        raise ValueError("gated_residual expects h and y of identical [B,S,C] shape and dtype")
+    B, S, Cdim = h.shape
+    _last_contig(h, "h")
+    _last_contig(y, "y")
+    gate_dtype = _code(h)
+    gs = (0, 0)
+    if gate is not None:
+        _last_contig(gate, "gate")
+        gate_dtype = _code(gate)
+        if gate.dim() == 2 and tuple(gate.shape) == (B, Cdim):
+            gs = (gate.stride(0) if B > 1 else 0, 0)
+        elif gate.dim() == 3 and gate.shape[0] == B and gate.shape[2] == Cdim and gate.shape[1] in (1, S):
+            gs = (gate.stride(0) if B > 1 else 0, gate.stride(1) if gate.shape[1] == S and S > 1 else 0)
+        else:
+            raise ValueError(f"gate shape {tuple(gate.shape)} does not broadcast against {(B, S, Cdim)}")
+    if out is None:
+        out = torch.empty_like(h, memory_format=torch.contiguous_format)
+    elif tuple(out.shape) != tuple(h.shape) or out.dtype != h.dtype or out.stride(-1) != 1:
+        raise ValueError("out must match h in shape and dtype with a contiguous last axis")
+    lib = _lib.load()
+    rc = lib.odit_gated_residual(
+        h.data_ptr(), y.data_ptr(), _ptr(gate), out.data_ptr(), B, S, Cdim,
+        _lib.i64_array(h.stride()[:2]), _lib.i64_array(y.stride()[:2]),
+        _lib.i64_array(out.stride()[:2]), _lib.i64_array(gs), gate_dtype, _code(h),
+        ODIT_FLAG_REF_ROUNDING if ref_rounding else 0, _stream(),
+    )
+    _lib.check(rc, "odit_gated_residual")
+    return out
+
+
+# --------------------------------------------------------------------------------------------- K5
+_REL_L1_SCRATCH: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def rel_l1_sums(cur: torch.Tensor, prev: torch.Tensor, *, ref_rounding: bool = True) -> torch.Tensor:
+    """Per-batch-row (sum |cur - prev|, sum |prev|) as a float64 [B,2] DEVICE tensor (no sync)."""
+    _dev(cur, prev)
+    if cur.shape != prev.shape or cur.dtype != prev.dtype or cur.dim() < 1:
+        raise ValueError("rel_l1_sums expects two tensors of identical shape and dtype")
+    B = cur.shape[0]
+    c2 = cur.reshape(B, -1)
+    p2 = prev.reshape(B, -1)
+    if c2.stride(-1) != 1:
+        c2 = c2.contiguous()
+    if p2.stride(-1) != 1:
+        p2 = p2.contiguous()
+    n = c2.shape[1]
+    lib = _lib.load()
+    need = int(lib.odit_rel_l1_workspace_bytes(B, n))
+    key = (cur.device.index or 0, need)
+    ws = _REL_L1_SCRATCH.get(key)
+    if ws is None:
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device=cur.device)
+        _REL_L1_SCRATCH[key] = ws
+    sums = torch.empty((B, 2), dtype=torch.float64, device=cur.device)
+    rc = lib.odit_rel_l1(
+        c2.data_ptr(), p2.data_ptr(), sums.data_ptr(), ws.data_ptr(), ws.numel(), B, n,
+        c2.stride(0) if B > 1 else n, p2.stride(0) if B > 1 else n, _code(cur),
+        ODIT_FLAG_REF_ROUNDING if ref_rounding else 0, _stream(),
+    )
+    _lib.check(rc, "odit_rel_l1")
+    return sums
+
+
+# ------------------------------------------------------------------------------------- activations
+def _unary(name: str, x: torch.Tensor, out: torch.Tensor | None) -> torch.Tensor:
+    _dev(x, out)
+    if not x.is_contiguous():
+        x = x.contiguous()
+    if out is None:
+        out = torch.empty_like(x)
+    elif out.shape != x.shape or out.dtype != x.dtype or not out.is_contiguous():
+        raise ValueError("out must be a contiguous tensor matching x")
+    lib = _lib.load()
+    rc = getattr(lib, name)(x.data_ptr(), out.data_ptr(), x.numel(), _code(x), _stream())
+    _lib.check(rc, name)
+    return out
+
+
+def gelu_tanh(x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    return _unary("odit_gelu_tanh", x, out)
+
+
+def silu(x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    return _unary("odit_silu", x, out)
