@@ -1,0 +1,279 @@
+"""Headline benchmark: denoise steps/s of the Qwen-Image-shape MMDiT at 1024x1024 on one MI355X.
+
+One "step" = one CFG-batched (B=2) transformer forward — stem, 60 dual-stream blocks, head — plus the
+CFG combine and the Euler update, on synthetic inputs already resident in HBM. Prints ONE JSON line:
+steps/s, the attention kernel's live-measured roofline fraction (bf16 MFMA), per-kernel GB/s and
+TFLOP/s for the other kernels on the path, and the CPU oracle timed on the host cores.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--blocks N] [--no-cpu] [--no-kernels]
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, vendor figure
+PEAK_HBM_GBS = 8000.0            # MI355X HBM3E, vendor figure
+
+# Qwen-Image shape at 1024x1024 (BASELINE.json configs[2])
+LAYERS, HEADS, HEAD_DIM, MLP_RATIO = 60, 24, 128, 4
+C = HEADS * HEAD_DIM
+S_IMG, S_TXT, TEXT_DIM, IN_CH = 4096, 256, 3584, 64
+IMG_SHAPE = (1, 64, 64)
+B = 2
+
+
+def _events(torch):
+    return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+
+def _time_op(torch, fn, iters=20, warmup=3):
+    """Average duration (ms) of fn() from HIP events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    a, b = _events(torch)
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters
+
+
+class AttnTimer:
+    """Brackets every attention launch of the timed region with HIP events on the launch stream."""
+
+    def __init__(self, torch, kernels):
+        self.torch, self.kernels = torch, kernels
+        self.orig = kernels.attn_fwd
+        self.pairs = []
+        self.active = False
+
+    def __enter__(self):
+        def timed(*a, **kw):
+            if not self.active:
+                return self.orig(*a, **kw)
+            s, e = _events(self.torch)
+            s.record()
+            out = self.orig(*a, **kw)
+            e.record()
+            self.pairs.append((s, e))
+            return out
+
+        self.kernels.attn_fwd = timed
+        return self
+
+    def __exit__(self, *exc):
+        self.kernels.attn_fwd = self.orig
+
+    def mean_ms(self):
+        return sum(s.elapsed_time(e) for s, e in self.pairs) / max(len(self.pairs), 1)
+
+
+def build_model(torch, layers):
+    from vllm_omni_amd.blocks.qwen_image import QwenImageTransformer2DModel
+
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device("cuda"):
+            model = QwenImageTransformer2DModel(num_layers=layers, attention_head_dim=HEAD_DIM,
+                                                num_attention_heads=HEADS, joint_attention_dim=TEXT_DIM,
+                                                in_channels=IN_CH, out_channels=16, mlp_ratio=MLP_RATIO)
+    finally:
+        torch.set_default_dtype(prev)
+    g = torch.Generator(device="cuda").manual_seed(0)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if name.endswith("norm_q.weight") or name.endswith("norm_k.weight") or name == "txt_norm.weight":
+                p.fill_(1.0)
+            elif name.endswith(".bias"):
+                p.zero_()
+            else:
+                p.normal_(0.0, 0.02, generator=g)
+    return model.eval()
+
+
+def kernel_rooflines(torch):
+    """Achieved GB/s (bandwidth-bound kernels) and TFLOP/s (attention, GEMM) at the config shapes."""
+    from vllm_omni_amd import kernels
+    from vllm_omni_amd._lib import ODIT_NORM_HEAD
+
+    dev = "cuda"
+    bf = torch.bfloat16
+    out = {}
+    x = torch.randn(B, S_IMG, C, device=dev, dtype=bf)
+    y = torch.randn(B, S_IMG, C, device=dev, dtype=bf)
+    mod = torch.randn(B, 3 * C, device=dev, dtype=bf)
+    shift, scale, gate = mod.chunk(3, dim=-1)
+    o = torch.empty_like(x)
+    ms = _time_op(torch, lambda: kernels.adaln_modulate(x, shift, scale, out=o))
+    byt = 2 * x.numel() * 2
+    out["adaln_modulate"] = {"ms": ms, "GB/s": byt / ms / 1e6, "frac_hbm": byt / ms / 1e6 / PEAK_HBM_GBS}
+    ms = _time_op(torch, lambda: kernels.gated_residual(x, y, gate, out=o))
+    byt = 3 * x.numel() * 2
+    out["gated_residual"] = {"ms": ms, "GB/s": byt / ms / 1e6, "frac_hbm": byt / ms / 1e6 / PEAK_HBM_GBS}
+    ms = _time_op(torch, lambda: kernels.rel_l1_sums(x, y))
+    byt = 2 * x.numel() * 2
+    out["rel_l1"] = {"ms": ms, "GB/s": byt / ms / 1e6, "frac_hbm": byt / ms / 1e6 / PEAK_HBM_GBS}
+    qkv = torch.randn(B, S_IMG, 3, HEADS, HEAD_DIM, device=dev, dtype=bf)
+    jq = torch.empty(B, S_IMG + S_TXT, HEADS, HEAD_DIM, device=dev, dtype=bf)
+    jk, jv = torch.empty_like(jq), torch.empty_like(jq)
+    w = torch.ones(HEAD_DIM, device=dev, dtype=bf)
+    cos = torch.rand(S_IMG, HEAD_DIM // 2, device=dev)
+    sin = torch.rand(S_IMG, HEAD_DIM // 2, device=dev)
+    ms = _time_op(torch, lambda: kernels.qknorm_rope(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], jq, jk, jv, w, w,
+                                                     cos, sin, out_seq_offset=S_TXT, norm_mode=ODIT_NORM_HEAD))
+    byt = 2 * qkv.numel() * 2
+    out["qknorm_rope"] = {"ms": ms, "GB/s": byt / ms / 1e6, "frac_hbm": byt / ms / 1e6 / PEAK_HBM_GBS}
+    u = torch.randn(B * S_IMG, MLP_RATIO * C, device=dev, dtype=bf)
+    ms = _time_op(torch, lambda: kernels.gelu_tanh(u, out=u))
+    byt = 2 * u.numel() * 2
+    out["gelu_tanh"] = {"ms": ms, "GB/s": byt / ms / 1e6, "frac_hbm": byt / ms / 1e6 / PEAK_HBM_GBS}
+    S = S_IMG + S_TXT
+    q = torch.randn(B, S, HEADS, HEAD_DIM, device=dev, dtype=bf)
+    k, v = torch.randn_like(q), torch.randn_like(q)
+    sc = 1.0 / math.sqrt(HEAD_DIM)
+    ms = _time_op(torch, lambda: kernels.attn_fwd(q, k, v, sc))
+    fl = 4.0 * B * HEADS * S * S * HEAD_DIM
+    out["attn_fwd"] = {"ms": ms, "TFLOP/s": fl / ms / 1e9, "frac_mfma": fl / ms / 1e9 / PEAK_MFMA_BF16_TFLOPS}
+    xm = torch.randn(B * S_IMG, C, device=dev, dtype=bf)
+    wm = torch.randn(MLP_RATIO * C, C, device=dev, dtype=bf)
+    bm = torch.zeros(MLP_RATIO * C, device=dev, dtype=bf)
+    ms = _time_op(torch, lambda: torch.nn.functional.linear(xm, wm, bm))
+    fl = 2.0 * xm.shape[0] * C * MLP_RATIO * C
+    out["gemm_mlp_up(hipBLASLt)"] = {"ms": ms, "TFLOP/s": fl / ms / 1e9,
+                                     "frac_mfma": fl / ms / 1e9 / PEAK_MFMA_BF16_TFLOPS}
+    return out
+
+
+def cpu_baseline(torch):
+    """The CPU oracle (plain-torch restatement of the reference path) on the host cores: ONE block of
+    the 60 at the full B=2 shape in fp32, extrapolated to a step."""
+    from oracle import qwen_image as oq
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    cfg = oq.QwenConfig(num_layers=1)
+    w = oq.init_params(cfg, seed=0, dtype=torch.float32)
+    g = torch.Generator().manual_seed(0)
+    img = torch.randn(B, S_IMG, C, generator=g)
+    txt = torch.randn(B, S_TXT, C, generator=g)
+    temb = torch.randn(B, C, generator=g)
+    vf, tf = oq.qwen_rope_freqs(cfg, *IMG_SHAPE, txt_len=S_TXT)
+    with torch.inference_mode():
+        oq.block_forward(w, 0, cfg, img[:, :256], txt, temb, vf[:256], tf)  # page in / warm threads
+        t0 = time.perf_counter()
+        oq.block_forward(w, 0, cfg, img, txt, temb, vf, tf)
+        dt = time.perf_counter() - t0
+    return {"value": 1.0 / (dt * LAYERS), "unit": "steps/s", "cores": cores, "kind": "port",
+            "sample": f"1 of {LAYERS} blocks at the full B=2, 4096+256-token shape, fp32 torch on {cores} threads, "
+                      f"{dt:.2f} s measured; step time extrapolated as {LAYERS} x block (stem/head < 0.5%)",
+            "block_seconds": dt}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--blocks", type=int, default=LAYERS, help="debug only: fewer blocks (result is then marked invalid)")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-kernels", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs the DiT step on ONE GPU (CFG branches are batched on it; "
+                 "there are no collectives). Run with --gpus 1.")
+
+    import torch
+
+    from vllm_omni_amd import _lib, kernels
+    from vllm_omni_amd.denoise import combine_cfg_noise, euler_step, flow_match_sigmas
+
+    _lib.load()
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+    model = build_model(torch, args.blocks)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    latents = torch.randn(1, S_IMG, IN_CH, device=dev, generator=g).bfloat16()
+    text = torch.randn(B, S_TXT, TEXT_DIM, device=dev, generator=g).bfloat16()
+    total_steps = args.steps + args.warmup
+    sig = flow_match_sigmas(max(total_steps, 20), S_IMG)
+
+    def step(i, lat):
+        t = torch.full((B,), float(sig[i]), device=dev, dtype=torch.bfloat16)
+        out = model(hidden_states=lat.expand(B, -1, -1), encoder_hidden_states=text, encoder_hidden_states_mask=None,
+                    timestep=t, img_shapes=[IMG_SHAPE], txt_seq_lens=[S_TXT] * B, return_dict=False)[0]
+        noise = combine_cfg_noise(out[0:1], out[1:2], 4.0, True)
+        return euler_step(lat, noise, float(sig[i]), float(sig[i + 1]))
+
+    with torch.inference_mode(), AttnTimer(torch, kernels) as timer:
+        lat = latents
+        for i in range(args.warmup):
+            lat = step(i, lat)
+        torch.cuda.synchronize()
+        timer.active = True
+        t0 = time.perf_counter()
+        for i in range(args.warmup, total_steps):
+            lat = step(i, lat)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        timer.active = False
+        attn_ms = timer.mean_ms()
+        n_attn = len(timer.pairs)
+    assert bool(torch.isfinite(lat.float()).all()), "non-finite latents"
+    ms_per_step = elapsed * 1e3 / args.steps
+    S = S_IMG + S_TXT
+    attn_flop = 4.0 * B * HEADS * S * S * HEAD_DIM
+    attn_tflops = attn_flop / attn_ms / 1e9
+    result = {
+        "metric": "DiT denoise steps/s @1024² Qwen-Image shape (1 GPU); attn % bf16 MFMA peak",
+        "value": args.steps / elapsed,
+        "unit": "steps/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"Qwen-Image-shape MMDiT denoise step: {args.blocks} dual-stream blocks, hidden {C}, "
+                               f"{HEADS} heads x {HEAD_DIM}, MLP {MLP_RATIO * C}, {S_IMG} image + {S_TXT} text tokens, "
+                               "CFG batch 2, random weights N(0,0.02)",
+                   "valid": args.blocks == LAYERS},
+        "roofline": {"kernel": "attn_fwd_kernel (joint attention, B=2, 24x128, S=4352)", "bound": "mfma",
+                     "achieved": attn_tflops, "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": attn_tflops / PEAK_MFMA_BF16_TFLOPS, "traffic": None,
+                     "launches_timed": n_attn, "avg_ms": attn_ms, "flop_per_launch": attn_flop},
+        "step_flop": None,
+    }
+    gemm_flop = 2.0 * (B * S_IMG + B * S_TXT) * (3 * C * C + C * C + 2 * MLP_RATIO * C * C) * args.blocks
+    result["step_flop"] = {"gemm": gemm_flop, "attention": attn_flop * args.blocks,
+                           "achieved_TFLOP/s": (gemm_flop + attn_flop * args.blocks) / elapsed * args.steps / 1e12}
+    if not args.no_kernels:
+        with torch.inference_mode():
+            result["kernels"] = kernel_rooflines(torch)
+    del model
+    torch.cuda.empty_cache()
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(torch)
+        result["gpu_over_cpu"] = result["value"] / result["cpu_baseline"]["value"]
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

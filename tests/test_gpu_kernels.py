@@ -1,0 +1,398 @@
+"""Parity of every HIP kernel (called through the C ABI) against the CPU oracle on seeded inputs.
+
+Tolerances: bf16/fp16 results are compared with the oracle evaluated in fp32 on the same (already
+16-bit-rounded) inputs; the bound is a few units of the output format's rounding step. With
+reference rounding switched on, elementwise results must match the oracle's 16-bit torch path
+bit for bit up to a stated number of ulps where reduction order differs.
+"""
+
+import math
+
+import pytest
+import torch
+
+from oracle import ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _rand(*shape, seed=0, dtype=torch.bfloat16, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+def _cos_sin(S, half, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    ang = torch.rand(S, half, generator=g) * 6.0 - 3.0
+    return torch.cos(ang), torch.sin(ang)
+
+
+def _close(got, want, atol, rtol=0.0, what=""):
+    got, want = got.float().cpu(), want.float().cpu()
+    err = (got - want).abs()
+    bound = atol + rtol * want.abs()
+    assert bool((err <= bound).all()), f"{what}: max err {err.max().item():.3e} (bound {atol}+{rtol}*|x|)"
+
+
+def _cosine(a, b):
+    a, b = a.float().flatten().cpu(), b.float().flatten().cpu()
+    return float(torch.dot(a, b) / (a.norm() * b.norm()))
+
+
+# ========================================================================================= K3
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("B,S,C", [(2, 33, 3072), (1, 7, 256), (2, 5, 5120), (3, 4, 40), (1, 3, 1000), (2, 3, 37)])
+def test_adaln_modulate(gpu, dtype, B, S, C):
+    from vllm_omni_amd import kernels
+
+    x = _rand(B, S, C, seed=1, dtype=dtype, scale=2.0) + 0.5
+    mod = _rand(B, 3 * C, seed=2, dtype=dtype, scale=0.5)
+    want, _ = ops.ada_layer_norm(x.float(), mod.float())
+    shift, scale, _ = mod.to(gpu).chunk(3, dim=-1)
+    got = kernels.adaln_modulate(x.to(gpu), shift, scale)
+    tol = {torch.bfloat16: 2e-2, torch.float16: 3e-3, torch.float32: 2e-5}[dtype]
+    _close(got, want, atol=tol, rtol=tol, what="adaln")
+    if dtype != torch.float32:
+        # reference rounding: LN -> dtype, (1+scale) -> dtype, product -> dtype, sum -> dtype
+        want_rr, _ = ops.ada_layer_norm(x, mod)
+        got_rr = kernels.adaln_modulate(x.to(gpu), shift, scale, ref_rounding=True)
+        ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+        _close(got_rr, want_rr, atol=1e-6, rtol=2.1 * ulp, what="adaln ref-rounding")
+        frac_equal = (got_rr.cpu() == want_rr).float().mean().item()
+        assert frac_equal > 0.97, f"only {frac_equal:.3f} of elements bit-identical"
+
+
+def test_adaln_index_fp32_params_affine_and_strides(gpu):
+    from vllm_omni_amd import kernels
+
+    B, S, C = 2, 9, 512
+    x = _rand(B, S, C, seed=3)
+    mod = _rand(2 * B, 3 * C, seed=4, scale=0.3)
+    index = (torch.arange(B * S).reshape(B, S) % 3 == 0).int()
+    want, _ = ops.ada_layer_norm(x.float(), mod.float(), index)
+    shift, scale, _ = mod.to(gpu).chunk(3, dim=-1)
+    got = kernels.adaln_modulate(x.to(gpu), shift, scale, index=index.to(gpu))
+    _close(got, want, atol=2e-2, rtol=2e-2, what="adaln index")
+    # fp32 modulation on bf16 activations, LayerNorm affine (Wan's norm2 / fp32 modulation path)
+    modf = _rand(B, 2 * C, seed=5, dtype=torch.float32, scale=0.3)
+    lw, lb = _rand(C, seed=6, dtype=torch.float32) + 1, _rand(C, seed=7, dtype=torch.float32)
+    ln = torch.nn.functional.layer_norm(x.float(), (C,), lw, lb, 1e-6)
+    want2 = ln * (1 + modf[:, None, C:]) + modf[:, None, :C]
+    mg = modf.to(gpu)
+    got2 = kernels.adaln_modulate(x.to(gpu), mg[:, :C], mg[:, C:], ln_weight=lw.to(gpu), ln_bias=lb.to(gpu))
+    _close(got2, want2, atol=2e-2, rtol=1e-2, what="adaln fp32 params + affine")
+    # strided input rows (a slice of a wider buffer) and no modulation at all
+    wide = _rand(B, S, 2 * C, seed=8)
+    got3 = kernels.adaln_modulate(wide.to(gpu)[:, :, C:], None, None)
+    _close(got3, torch.nn.functional.layer_norm(wide[:, :, C:].float(), (C,), eps=1e-6), atol=2e-2, what="plain LN")
+
+
+# ========================================================================================= K4
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_gated_residual(gpu, dtype):
+    from vllm_omni_amd import kernels
+
+    B, S, C = 2, 17, 3072
+    h, y = _rand(B, S, C, seed=1, dtype=dtype), _rand(B, S, C, seed=2, dtype=dtype)
+    mod = _rand(B, 3 * C, seed=3, dtype=dtype)
+    gate = mod.chunk(3, dim=-1)[2]
+    want = ops.gated_residual(h.float(), y.float(), gate.float()[:, None])
+    got = kernels.gated_residual(h.to(gpu), y.to(gpu), mod.to(gpu).chunk(3, dim=-1)[2].unsqueeze(1))
+    tol = {torch.bfloat16: 2 ** -8, torch.float16: 2 ** -11, torch.float32: 1e-6}[dtype]
+    _close(got, want, atol=1e-6, rtol=tol, what="gated residual")
+    if dtype != torch.float32:
+        want_rr = ops.gated_residual(h, y, gate[:, None])
+        got_rr = kernels.gated_residual(h.to(gpu), y.to(gpu), gate.to(gpu), ref_rounding=True)
+        assert torch.equal(got_rr.cpu(), want_rr), "reference-rounding path must be bit-exact"
+    # gate = 0 is the identity, gate = None a plain residual, in-place output, per-token fp32 gate
+    z = torch.zeros(B, C, dtype=dtype, device=gpu)
+    assert torch.equal(kernels.gated_residual(h.to(gpu), y.to(gpu), z).cpu(), h)
+    _close(kernels.gated_residual(h.to(gpu), y.to(gpu), None), h.float() + y.float(), atol=1e-6, rtol=tol)
+    hg = h.to(gpu).clone()
+    gtok = _rand(B, S, C, seed=4, dtype=torch.float32)
+    out = kernels.gated_residual(hg, y.to(gpu), gtok.to(gpu), out=hg)
+    assert out.data_ptr() == hg.data_ptr()
+    _close(hg, h.float() + gtok * y.float(), atol=1e-6, rtol=tol, what="per-token fp32 gate, in place")
+
+
+def test_gated_residual_odd_sizes(gpu):
+    from vllm_omni_amd import kernels
+
+    h, y, g = _rand(2, 3, 37, seed=1), _rand(2, 3, 37, seed=2), _rand(2, 37, seed=3)
+    _close(kernels.gated_residual(h.to(gpu), y.to(gpu), g.to(gpu)),
+           h.float() + g.float()[:, None] * y.float(), atol=1e-6, rtol=2 ** -8)
+
+
+# ========================================================================================= K5
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("B,n", [(2, 64 * 3072), (1, 4096 * 3072), (3, 1000), (2, 8 * 1024 * 8 + 5)])
+def test_rel_l1(gpu, dtype, B, n):
+    from vllm_omni_amd import kernels
+    from vllm_omni_amd.cache.teacache.hook import rel_l1_from_sums
+
+    prev = _rand(B, n, seed=1, dtype=dtype)
+    cur = (prev.float() * 1.04 + 0.03 * _rand(B, n, seed=2, dtype=torch.float32)).to(dtype)
+    sums = kernels.rel_l1_sums(cur.to(gpu), prev.to(gpu), ref_rounding=True).cpu()
+    for b in range(B):
+        sd = (cur[b] - prev[b]).abs().double().sum().item()   # difference rounded to dtype, as torch does
+        sp = prev[b].abs().double().sum().item()
+        assert sums[b, 0].item() == pytest.approx(sd, rel=5e-6)
+        assert sums[b, 1].item() == pytest.approx(sp, rel=5e-6)
+        # the scalar TeaCache thresholds is IDENTICAL to the reference expression's
+        want = ops.rel_l1(cur[b:b + 1], prev[b:b + 1])
+        got = rel_l1_from_sums(sums[b, 0].item(), sums[b, 1].item(), n, dtype)
+        if dtype == torch.bfloat16:
+            assert got == want
+        else:
+            assert got == pytest.approx(want, rel=1e-5)
+    # deterministic: a second launch gives bit-identical sums
+    again = kernels.rel_l1_sums(cur.to(gpu), prev.to(gpu), ref_rounding=True).cpu()
+    assert torch.equal(again, sums)
+
+
+def test_rel_l1_closed_forms(gpu):
+    from vllm_omni_amd import kernels
+
+    prev = (_rand(2, 5000, seed=3, dtype=torch.float32).abs() + 0.5)
+    s = kernels.rel_l1_sums(prev.to(gpu), prev.to(gpu)).cpu()
+    assert torch.all(s[:, 0] == 0)
+    s = kernels.rel_l1_sums((1.5 * prev).to(gpu), prev.to(gpu), ref_rounding=False).cpu()
+    assert torch.allclose(s[:, 0] / s[:, 1], torch.full((2,), 0.5, dtype=torch.float64), rtol=1e-6)
+
+
+# ========================================================================================= K2
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("H,D", [(24, 128), (4, 64)])
+def test_qknorm_rope_joint(gpu, dtype, H, D):
+    """Fused QKV slices of an image and a text stream -> joint [txt;img] buffers."""
+    from vllm_omni_amd import kernels
+    from vllm_omni_amd._lib import ODIT_NORM_HEAD
+
+    B, S_img, S_txt = 2, 50, 11
+    wq = (_rand(D, seed=1, dtype=torch.float32) * 0.2 + 1).to(dtype)
+    wk = (_rand(D, seed=2, dtype=torch.float32) * 0.2 + 1).to(dtype)
+    streams = {}
+    for name, S, seed in (("txt", S_txt, 10), ("img", S_img, 20)):
+        qkv = _rand(B, S, 3, H, D, seed=seed, dtype=dtype)
+        cos, sin = _cos_sin(S, D // 2, seed=seed + 1)
+        streams[name] = (qkv, cos, sin)
+    S = S_txt + S_img
+    jq = torch.zeros(B, S, H, D, dtype=dtype, device=gpu)
+    jk, jv = torch.zeros_like(jq), torch.zeros_like(jq)
+    want_q, want_k, want_v, want_q_rr, want_k_rr = [], [], [], [], []
+    off = 0
+    for name in ("txt", "img"):
+        qkv, cos, sin = streams[name]
+        g = qkv.to(gpu)
+        kernels.qknorm_rope(g[:, :, 0], g[:, :, 1], g[:, :, 2], jq, jk, jv, wq.to(gpu), wk.to(gpu),
+                            cos.to(gpu), sin.to(gpu), eps=1e-6, out_seq_offset=off, norm_mode=ODIT_NORM_HEAD)
+        off += qkv.shape[1]
+        f = qkv.float()
+        want_q.append(ops.apply_rotary(ops.rms_norm_head(f[:, :, 0], wq.float()), cos, sin))
+        want_k.append(ops.apply_rotary(ops.rms_norm_head(f[:, :, 1], wk.float()), cos, sin))
+        want_v.append(qkv[:, :, 2])
+        want_q_rr.append(ops.apply_rotary(ops.rms_norm_head(qkv[:, :, 0], wq), cos.to(dtype), sin.to(dtype)))
+        want_k_rr.append(ops.apply_rotary(ops.rms_norm_head(qkv[:, :, 1], wk), cos.to(dtype), sin.to(dtype)))
+    tol = {torch.bfloat16: 2e-2, torch.float16: 3e-3, torch.float32: 2e-5}[dtype]
+    _close(jq, torch.cat(want_q, 1), atol=tol, rtol=tol, what="joint q")
+    _close(jk, torch.cat(want_k, 1), atol=tol, rtol=tol, what="joint k")
+    assert torch.equal(jv.cpu(), torch.cat(want_v, 1)), "v must be copied bit for bit"
+    if dtype != torch.float32:
+        off = 0
+        for name in ("txt", "img"):
+            qkv, cos, sin = streams[name]
+            g = qkv.to(gpu)
+            kernels.qknorm_rope(g[:, :, 0], g[:, :, 1], g[:, :, 2], jq, jk, jv, wq.to(gpu), wk.to(gpu),
+                                cos.to(gpu), sin.to(gpu), eps=1e-6, out_seq_offset=off,
+                                norm_mode=ODIT_NORM_HEAD, ref_rounding=True)
+            off += qkv.shape[1]
+        ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+        _close(jq, torch.cat(want_q_rr, 1), atol=2 * ulp, rtol=2.1 * ulp, what="joint q, ref rounding")
+        _close(jk, torch.cat(want_k_rr, 1), atol=2 * ulp, rtol=2.1 * ulp, what="joint k, ref rounding")
+        assert (jq.cpu() == torch.cat(want_q_rr, 1)).float().mean().item() > 0.95
+
+
+def test_rotary_layer_and_neox_and_partial(gpu):
+    from vllm_omni_amd.layers.rope import RotaryEmbedding
+
+    B, S, H, D = 2, 13, 3, 128
+    x = _rand(B, S, H, D, seed=1)
+    cos, sin = _cos_sin(S, D // 2, seed=2)
+    for neox in (False, True):
+        layer = RotaryEmbedding(is_neox_style=neox)
+        got = layer(x.to(gpu), cos.to(gpu), sin.to(gpu))
+        _close(got, ops.apply_rotary(x.float(), cos, sin, interleaved=not neox), atol=2e-2, rtol=1e-2,
+               what=f"rotary neox={neox}")
+    # [B,S,rot/2] tables use the first batch row; rot < D leaves the tail alone
+    c3, s3 = cos[:, :32].expand(B, S, 32), sin[:, :32].expand(B, S, 32)
+    got = RotaryEmbedding()(x.to(gpu), c3.to(gpu), s3.to(gpu))
+    _close(got, ops.apply_rotary(x.float(), cos[:, :32], sin[:, :32]), atol=2e-2, rtol=1e-2, what="partial rotary")
+    assert torch.equal(got[..., 64:].cpu(), x[..., 64:])
+    # identity tables (text rows of the joint-attention config) return x bit for bit
+    same = RotaryEmbedding()(x.to(gpu), torch.ones(S, 64, device=gpu), torch.zeros(S, 64, device=gpu))
+    assert torch.equal(same.cpu(), x)
+
+
+def test_rmsnorm_layer_row_mode_and_wan_qknorm(gpu):
+    from vllm_omni_amd import kernels
+    from vllm_omni_amd._lib import ODIT_NORM_ROW
+    from vllm_omni_amd.layers.rmsnorm import RMSNorm
+
+    # txt_norm: 3584-wide rows
+    x = _rand(2, 19, 3584, seed=1)
+    layer = RMSNorm(3584).to(gpu).to(torch.bfloat16)
+    with torch.no_grad():
+        layer.weight.copy_((_rand(3584, seed=2, dtype=torch.float32) * 0.1 + 1).to(gpu))
+    _close(layer(x.to(gpu)), ops.rms_norm_head(x.float(), layer.weight.float().cpu()), atol=2e-2, rtol=1e-2,
+           what="RMSNorm 3584")
+    # Wan: whole-row RMS over H*D = 5120 with fp32 weights, then rotary with half tables
+    B, S, H, D = 1, 21, 40, 128
+    qkv = _rand(B, S, 3, H, D, seed=3)
+    wq, wk = _rand(H * D, seed=4, dtype=torch.float32) * 0.1 + 1, _rand(H * D, seed=5, dtype=torch.float32) * 0.1 + 1
+    cos, sin = _cos_sin(S, D // 2, seed=6)
+    g = qkv.to(gpu)
+    q_out = torch.empty(B, S, H, D, dtype=torch.bfloat16, device=gpu)
+    k_out, v_out = torch.empty_like(q_out), torch.empty_like(q_out)
+    kernels.qknorm_rope(g[:, :, 0], g[:, :, 1], g[:, :, 2], q_out, k_out, v_out, wq.to(gpu), wk.to(gpu),
+                        cos.to(gpu), sin.to(gpu), eps=1e-6, norm_mode=ODIT_NORM_ROW)
+    fc = cos.repeat_interleave(2, -1).view(1, S, 1, D)
+    fs = sin.repeat_interleave(2, -1).view(1, S, 1, D)
+    for got, src, w in ((q_out, qkv[:, :, 0], wq), (k_out, qkv[:, :, 1], wk)):
+        n = ops.rms_norm_row_fp32(src.float().flatten(2), w).unflatten(2, (H, D))
+        _close(got, ops.apply_rotary_wan(n, fc, fs), atol=2e-2, rtol=1e-2, what="wan qk norm+rope")
+    assert torch.equal(v_out.cpu(), qkv[:, :, 2])
+
+
+# ========================================================================================= activations
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_activations(gpu, dtype):
+    from vllm_omni_amd import kernels
+
+    x = _rand(3, 1001, seed=1, dtype=dtype, scale=3.0)
+    tol = 2 ** -8 if dtype == torch.bfloat16 else 2e-6
+    _close(kernels.gelu_tanh(x.to(gpu)), ops.gelu_tanh(x.float()), atol=tol, rtol=tol, what="gelu")
+    _close(kernels.silu(x.to(gpu)), torch.nn.functional.silu(x.float()), atol=tol, rtol=tol, what="silu")
+    big = torch.tensor([-100.0, -20.0, 0.0, 20.0, 100.0], dtype=dtype)
+    _close(kernels.gelu_tanh(big.to(gpu)), ops.gelu_tanh(big.float()), atol=1e-6, rtol=tol, what="gelu tails")
+
+
+# ========================================================================================= K1
+def _attn_inputs(B, Sq, Sk, H, Hkv, D, seed, dtype=torch.bfloat16):
+    q = _rand(B, Sq, H, D, seed=seed, dtype=dtype)
+    k = _rand(B, Sk, Hkv, D, seed=seed + 1, dtype=dtype)
+    v = _rand(B, Sk, Hkv, D, seed=seed + 2, dtype=dtype)
+    return q, k, v
+
+
+ATTN_SHAPES = [
+    # B, Sq, Sk, H, Hkv, D
+    (2, 64, 64, 8, 8, 64),       # the reference's own test shape (tests/diffusion/attention/test_flash_attn.py)
+    (1, 320, 320, 4, 4, 128),    # tiny config-like
+    (2, 300, 300, 3, 3, 128),    # ragged: tails in both q blocks and key tiles
+    (1, 1, 1, 1, 1, 128),        # smallest possible
+    (1, 70, 515, 2, 2, 64),      # cross-attention shape, ragged keys
+    (1, 257, 129, 4, 2, 128),    # grouped KV heads
+]
+
+
+@pytest.mark.parametrize("variant", ["14", "18", "24"])
+@pytest.mark.parametrize("shape", ATTN_SHAPES)
+def test_attention_parity(gpu, monkeypatch, variant, shape):
+    from vllm_omni_amd import kernels
+
+    monkeypatch.setenv("ODIT_ATTN_VARIANT", variant)
+    B, Sq, Sk, H, Hkv, D = shape
+    q, k, v = _attn_inputs(B, Sq, Sk, H, Hkv, D, seed=42)
+    scale = 1.0 / math.sqrt(D)
+    print(f"attn variant={variant} shape={shape}", flush=True)
+    got, lse = kernels.attn_fwd(q.to(gpu), k.to(gpu), v.to(gpu), scale, return_lse=True)
+    torch.cuda.synchronize()
+    want = ops.sdpa(q.float(), k.float(), v.float(), scale)
+    # bf16 output of values in [-~3, 3]: error budget = P rounded to bf16 inside + one output rounding
+    _close(got, want, atol=2e-2, rtol=2e-2, what="attention")
+    assert _cosine(got, want) >= 0.9995
+    # the reference's own thresholds for backend agreement (test_flash_attn.py:144-147)
+    d = (got.float().cpu() - want).abs()
+    assert d.max() < 0.1 and d.mean() < 0.01
+    kf = k.float().repeat_interleave(H // Hkv, dim=2)
+    s = torch.einsum("bqhd,bkhd->bhqk", q.float(), kf) * scale
+    _close(lse, torch.logsumexp(s, dim=-1), atol=2e-2, rtol=1e-3, what="lse")
+
+
+def test_attention_fp16_and_strided_views(gpu):
+    from vllm_omni_amd import kernels
+
+    B, S, H, D = 2, 200, 4, 128
+    qkv = _rand(B, S, 3, H, D, seed=7, dtype=torch.float16)
+    g = qkv.to(gpu)
+    got = kernels.attn_fwd(g[:, :, 0], g[:, :, 1], g[:, :, 2], 0.09)   # views of a fused buffer, no copies
+    want = ops.sdpa(qkv[:, :, 0].float(), qkv[:, :, 1].float(), qkv[:, :, 2].float(), 0.09)
+    _close(got, want, atol=3e-3, rtol=3e-3, what="fp16 strided attention")
+
+
+def test_attention_key_mask_equals_deleting_keys(gpu):
+    """The reference's padding-equivalence property (test_flash_attn.py:60-147)."""
+    from vllm_omni_amd import kernels
+    from vllm_omni_amd.attention.backends.abstract import AttentionMetadata
+    from vllm_omni_amd.attention.layer import Attention
+
+    B, S, H, D, pad = 2, 84, 8, 64, 20
+    q, k, v = _attn_inputs(B, S, S, H, H, D, seed=123)
+    mask = torch.ones(B, S, dtype=torch.bool)
+    mask[:, S - pad:] = False
+    layer = Attention(num_heads=H, head_size=D, causal=False, softmax_scale=0.125)
+    got = layer(q.to(gpu), k.to(gpu), v.to(gpu), AttentionMetadata(attn_mask=mask.to(gpu)))
+    unpadded = kernels.attn_fwd(q.to(gpu), k[:, :S - pad].to(gpu), v[:, :S - pad].to(gpu), 0.125)
+    assert torch.equal(got.cpu(), unpadded.cpu()), "masking keys must equal removing them"
+    _close(got, ops.sdpa(q.float(), k.float(), v.float(), 0.125, key_mask=mask), atol=2e-2, rtol=2e-2)
+    # scattered mask, different per batch row
+    g = torch.Generator().manual_seed(5)
+    m2 = torch.rand(B, S, generator=g) > 0.3
+    m2[:, 0] = True
+    got2 = kernels.attn_fwd(q.to(gpu), k.to(gpu), v.to(gpu), 0.125, key_mask=m2.to(gpu))
+    _close(got2, ops.sdpa(q.float(), k.float(), v.float(), 0.125, key_mask=m2), atol=2e-2, rtol=2e-2)
+    # an all-true mask is dropped and gives the unmasked result bit for bit
+    ones = AttentionMetadata(attn_mask=torch.ones(B, S, dtype=torch.bool, device=gpu))
+    assert torch.equal(layer(q.to(gpu), k.to(gpu), v.to(gpu), ones).cpu(),
+                       layer(q.to(gpu), k.to(gpu), v.to(gpu)).cpu())
+
+
+def test_attention_fp32_goes_to_sdpa(gpu):
+    from vllm_omni_amd.attention.layer import Attention
+
+    q, k, v = _attn_inputs(1, 40, 40, 2, 2, 64, seed=9, dtype=torch.float32)
+    layer = Attention(num_heads=2, head_size=64, causal=False, softmax_scale=0.125)
+    _close(layer(q.to(gpu), k.to(gpu), v.to(gpu)), ops.sdpa(q, k, v, 0.125), atol=1e-4, rtol=1e-4)
+
+
+def test_attention_full_size_properties(gpu):
+    """BASELINE config 2 shape (B=2, 24 heads x 128, 4096 image + 256 text tokens): properties that
+    do not need the full CPU product, plus the oracle on two heads."""
+    from vllm_omni_amd import kernels
+
+    B, S, H, D = 2, 4352, 24, 128
+    scale = 1.0 / math.sqrt(D)
+    g = torch.Generator(device="cpu").manual_seed(0)
+    q = torch.randn(B, S, H, D, generator=g).bfloat16().to(gpu)
+    k = torch.randn(B, S, H, D, generator=g).bfloat16().to(gpu)
+    v = torch.randn(B, S, H, D, generator=g).bfloat16().to(gpu)
+    out, lse = kernels.attn_fwd(q, k, v, scale, return_lse=True)
+    # (1) V = 1 -> every output is exactly 1 up to the final rounding of sum(P)/sum(P)
+    ones = kernels.attn_fwd(q, k, torch.ones_like(v), scale)
+    _close(ones, torch.ones(1), atol=2 ** -7, what="rows of P sum to 1")
+    # (2) permuting keys with their values leaves the result unchanged (to rounding)
+    perm = torch.randperm(S, generator=g).to(gpu)
+    outp = kernels.attn_fwd(q, k[:, perm].contiguous(), v[:, perm].contiguous(), scale)
+    _close(outp, out, atol=2e-2, what="key permutation invariance")
+    # (3) split keys in two halves and merge with the LSE identity
+    oa, la = kernels.attn_fwd(q, k[:, :2000], v[:, :2000], scale, return_lse=True)
+    ob, lb = kernels.attn_fwd(q, k[:, 2000:], v[:, 2000:], scale, return_lse=True)
+    merged, lse_m = ops.merge_lse(oa.float(), la, ob.float(), lb)
+    _close(merged, out, atol=2e-2, what="split-K + LSE merge")
+    _close(lse_m, lse, atol=1e-2, what="merged lse")
+    # (4) oracle on two (batch, head) slices
+    for b, h in ((0, 0), (1, 23)):
+        sl = lambda t: t[b:b + 1, :, h:h + 1].float().cpu()  # noqa: E731
+        want = ops.sdpa(sl(q), sl(k), sl(v), scale)
+        _close(out[b:b + 1, :, h:h + 1], want, atol=2e-2, rtol=2e-2, what=f"head ({b},{h})")
+        assert _cosine(out[b:b + 1, :, h:h + 1], want) >= 0.9995
