@@ -101,6 +101,7 @@ def build_model(torch, layers):
                 p.zero_()
             else:
                 p.normal_(0.0, 0.02, generator=g)
+    model.fuse_modulation()
     return model.eval()
 
 

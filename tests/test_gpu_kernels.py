@@ -297,7 +297,7 @@ ATTN_SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("variant", ["14", "18", "24"])
+@pytest.mark.parametrize("variant", ["14", "18", "24", "28", "29"])
 @pytest.mark.parametrize("shape", ATTN_SHAPES)
 def test_attention_parity(gpu, monkeypatch, variant, shape):
     from vllm_omni_amd import kernels
@@ -332,9 +332,12 @@ def test_attention_fp16_and_strided_views(gpu):
     _close(got, want, atol=3e-3, rtol=3e-3, what="fp16 strided attention")
 
 
-def test_attention_key_mask_equals_deleting_keys(gpu):
+@pytest.mark.parametrize("variant", ["18", "24", "28"])
+def test_attention_key_mask_equals_deleting_keys(gpu, monkeypatch, variant):
     """The reference's padding-equivalence property (test_flash_attn.py:60-147)."""
     from vllm_omni_amd import kernels
+
+    monkeypatch.setenv("ODIT_ATTN_VARIANT", variant)
     from vllm_omni_amd.attention.backends.abstract import AttentionMetadata
     from vllm_omni_amd.attention.layer import Attention
 
@@ -353,6 +356,14 @@ def test_attention_key_mask_equals_deleting_keys(gpu):
     m2[:, 0] = True
     got2 = kernels.attn_fwd(q.to(gpu), k.to(gpu), v.to(gpu), 0.125, key_mask=m2.to(gpu))
     _close(got2, ops.sdpa(q.float(), k.float(), v.float(), 0.125, key_mask=m2), atol=2e-2, rtol=2e-2)
+    # single excluded keys at tile edges, a fully excluded first tile, everything but one key excluded
+    for S2, cut in ((64, [63]), (128, [0, 64, 127]), (128, list(range(0, 64))), (200, list(range(1, 200)))):
+        q2, k2, v2 = _attn_inputs(1, S2, S2, 2, 2, 64, seed=S2)
+        m3 = torch.ones(1, S2, dtype=torch.bool)
+        m3[:, cut] = False
+        got3 = kernels.attn_fwd(q2.to(gpu), k2.to(gpu), v2.to(gpu), 0.125, key_mask=m3.to(gpu))
+        _close(got3, ops.sdpa(q2.float(), k2.float(), v2.float(), 0.125, key_mask=m3), atol=2e-2, rtol=2e-2,
+               what=f"mask S={S2} cut={cut[:3]}")
     # an all-true mask is dropped and gives the unmasked result bit for bit
     ones = AttentionMetadata(attn_mask=torch.ones(B, S, dtype=torch.bool, device=gpu))
     assert torch.equal(layer(q.to(gpu), k.to(gpu), v.to(gpu), ones).cpu(),

@@ -224,12 +224,18 @@ class QwenImageTransformerBlock(nn.Module):
     def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor,
                 encoder_hidden_states_mask: torch.Tensor | None, temb: torch.Tensor, image_rotary_emb,
                 joint_attention_kwargs: dict[str, Any] | None = None, modulate_index: torch.Tensor | None = None,
-                hidden_states_mask: torch.Tensor | None = None):
+                hidden_states_mask: torch.Tensor | None = None,
+                mod_params: tuple[torch.Tensor, torch.Tensor] | None = None):
+        """``mod_params`` = (img [B,6C], txt [B,6C]) computed by the caller for all blocks at once
+        (they depend on ``temb`` only); when absent they are computed here as in the reference."""
         rr = self.ref_rounding
-        img_mod_params = self.img_mod(temb)
-        if self.zero_cond_t:
-            temb = torch.chunk(temb, 2, dim=0)[0]
-        txt_mod_params = self.txt_mod(temb)
+        if mod_params is not None:
+            img_mod_params, txt_mod_params = mod_params
+        else:
+            img_mod_params = self.img_mod(temb)
+            if self.zero_cond_t:
+                temb = torch.chunk(temb, 2, dim=0)[0]
+            txt_mod_params = self.txt_mod(temb)
         img_mod1, img_mod2 = img_mod_params.chunk(2, dim=-1)
         txt_mod1, txt_mod2 = txt_mod_params.chunk(2, dim=-1)
 
@@ -340,13 +346,43 @@ class QwenImageTransformer2DModel(nn.Module):
         vid_freqs, txt_freqs = self.pos_embed(img_shapes, txt_seq_lens, device=img.device)
         return img, txt, temb, RotaryTables(vid_freqs, txt_freqs)
 
+    def fuse_modulation(self) -> None:
+        """Stack every block's img_mod / txt_mod Linear into one [L, 2, 6C, C] weight so that the
+        2L modulation projections of a step (each a weight-streaming M=B GEMV: the largest
+        non-GEMM HBM stream of the model) run as ONE pass over the weights. The per-block parameters
+        become views of the stacked tensors: names, shapes and values are unchanged."""
+        L, C = len(self.transformer_blocks), self.inner_dim
+        ref = self.transformer_blocks[0].img_mod[1].weight
+        w_all = torch.empty((L, 2, 6 * C, C), dtype=ref.dtype, device=ref.device)
+        b_all = torch.empty((L, 2, 6 * C), dtype=ref.dtype, device=ref.device)
+        with torch.no_grad():
+            for i, blk in enumerate(self.transformer_blocks):
+                for j, lin in enumerate((blk.img_mod[1], blk.txt_mod[1])):
+                    w_all[i, j].copy_(lin.weight)
+                    b_all[i, j].copy_(lin.bias)
+                    lin.weight.data = w_all[i, j]
+                    lin.bias.data = b_all[i, j]
+        self._mod_weight, self._mod_bias = w_all, b_all
+
+    def all_modulations(self, temb: torch.Tensor) -> torch.Tensor | None:
+        """[B, L, 2, 6C] modulation parameters of every block, or None when not fused."""
+        w = getattr(self, "_mod_weight", None)
+        if w is None or self.zero_cond_t:
+            return None
+        L, C = w.shape[0], self.inner_dim
+        out = F.linear(kernels.silu(temb), w.view(L * 2 * 6 * C, C), self._mod_bias.view(-1))
+        return out.view(temb.shape[0], L, 2, 6 * C)
+
     def run_blocks(self, img, txt, temb, rotary, encoder_hidden_states_mask=None, attention_kwargs=None):
         mask = encoder_hidden_states_mask
         if mask is not None and bool(mask.all()):
             mask = None  # all-true masks are dropped (qit.py:1044-1048)
-        for block in self.transformer_blocks:
+        mods = self.all_modulations(temb)
+        for i, block in enumerate(self.transformer_blocks):
+            mp = (mods[:, i, 0], mods[:, i, 1]) if mods is not None else None
             txt, img = block(hidden_states=img, encoder_hidden_states=txt, encoder_hidden_states_mask=mask,
-                             temb=temb, image_rotary_emb=rotary, joint_attention_kwargs=attention_kwargs)
+                             temb=temb, image_rotary_emb=rotary, joint_attention_kwargs=attention_kwargs,
+                             mod_params=mp)
         return img, txt
 
     def finish(self, img, temb, return_dict: bool = True):

@@ -230,7 +230,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(const AttnParams p) {
 
     // ---- exclusions: keys past Sk (last tile) and keys the padding mask removes ----
     const bool tail = (j + 1) * BN > p.Sk;
-    if (tail || mrow != nullptr) {
+    if (tail || mrow != nullptr) {  // branch-free selects inside
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
@@ -238,10 +238,12 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(const AttnParams p) {
 #pragma unroll
           for (int t = 0; t < 4; ++t) {
             const int key = j * BN + kt * 32 + g * 8 + hh * 4 + t;
-            const bool dead = key >= p.Sk || (mrow != nullptr && mrow[key] == 0);
-            if (dead) {
+            const int kc = key < p.Sk ? key : p.Sk - 1;
+            const bool live = (key < p.Sk) & (mrow == nullptr || mrow[kc] != 0);
 #pragma unroll
-              for (int qt = 0; qt < QT; ++qt) s[kt][qt][g * 4 + t] = -INFINITY;
+            for (int qt = 0; qt < QT; ++qt) {
+              const float x = s[kt][qt][g * 4 + t];
+              s[kt][qt][g * 4 + t] = live ? x : -INFINITY;
             }
           }
     }
@@ -340,6 +342,298 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(const AttnParams p) {
   }
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// Software-pipelined variant (one 32-query tile per wavefront).
+//
+// Per key tile j a wavefront runs two stages:
+//   A:  S(j+1)^T = K(j+1) Q^T on the matrix cores   while the vector ALU turns S(j) into P(j)
+//       (exp2, row sums, 16-bit packing) — the two instruction streams are independent and are
+//       written interleaved, one MFMA per seven vector instructions;
+//   B:  O^T += V(j)^T P(j)^T.
+// The row maximum of S(j+1) and the (rare) rescale of O are settled between B and the next A.
+// K runs one tile ahead of V through the double-buffered LDS stage, so one barrier per tile is
+// enough. V stays row-major in LDS; its transposed A fragments come from ds_read_b64_tr_b16, whose
+// 16-lane transpose delivers, for lane i of a group, element (i % 4) of the 8-byte words fetched by
+// lanes 4k + i/4 (k = 0..3): four consecutive keys of one head-dim column.
+// ------------------------------------------------------------------------------------------------
+typedef short s16x4_v __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) s16x4_v* lds_s16x4_ptr;
+
+template <typename T, int D, int NW>
+__global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_pipe_kernel(const AttnParams p) {
+  using M = Mma<T>;
+  using frag = typename M::frag;
+  constexpr int BN = 64;
+  constexpr int NT = NW * 64;
+  constexpr int BM = NW * 32;
+  constexpr int KS = D / 16;
+  constexpr int DT = D / 32;
+  constexpr int KROW = D + 8;    // +16 B per row: the 16 lanes of a quarter-wave b128 read cover all banks
+  constexpr int VROW = D + 32;   // +64 B per row: the 4 keys x 4 words of a transpose read cover disjoint banks
+  constexpr int CPR = D / 8;
+  constexpr int TCH = BN * CPR;  // 16-byte chunks per tile
+  constexpr int TPT = (TCH + NT - 1) / NT;
+
+  __shared__ __attribute__((aligned(16))) T Ks[2][BN * KROW];
+  __shared__ __attribute__((aligned(16))) T Vs[2][BN * VROW];
+
+  const int pid = xcd_remap(blockIdx.x, p.total_blocks);
+  const int qb = pid % p.n_qblocks;
+  const int bh = pid / p.n_qblocks;
+  const int h = bh % p.H;
+  const int b = bh / p.H;
+  const int hkv = h / (p.H / p.Hkv);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hh = lane >> 5;
+  const int q0 = qb * BM + wave * 32;
+
+  const T* qbase = static_cast<const T*>(p.q) + b * p.qs_b + h * p.qs_h;
+  const T* kbase = static_cast<const T*>(p.k) + b * p.ks_b + hkv * p.ks_h;
+  const T* vbase = static_cast<const T*>(p.v) + b * p.vs_b + hkv * p.vs_h;
+
+  frag qf[KS];
+  {
+    int row = q0 + l32;
+    row = row < p.Sq ? row : p.Sq - 1;
+    const T* qp = qbase + row * p.qs_s + hh * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      qf[ks] = __builtin_bit_cast(frag, *reinterpret_cast<const u32x4_v*>(qp + ks * 16));
+  }
+
+  u32x4_v kreg[TPT], vreg[TPT];
+  auto gload = [&](const T* base, int64_t stride_s, int j, u32x4_v(&reg)[TPT]) {
+#pragma unroll
+    for (int i = 0; i < TPT; ++i) {
+      const int c = tid + i * NT;
+      if (TCH % NT == 0 || c < TCH) {
+        int key = j * BN + c / CPR;
+        key = key < p.Sk ? key : p.Sk - 1;
+        reg[i] = *reinterpret_cast<const u32x4_v*>(base + key * stride_s + (c % CPR) * 8);
+      }
+    }
+  };
+  auto sstore = [&](T* dst, int pitch, const u32x4_v(&reg)[TPT]) {
+#pragma unroll
+    for (int i = 0; i < TPT; ++i) {
+      const int c = tid + i * NT;
+      if (TCH % NT == 0 || c < TCH)
+        *reinterpret_cast<u32x4_v*>(dst + (c / CPR) * pitch + (c % CPR) * 8) = reg[i];
+    }
+  };
+
+  f32x16_v o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o[dt][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  const int n_tiles = (p.Sk + BN - 1) / BN;
+  const float c = p.scale_log2;
+  const uint8_t* mrow = p.mask ? p.mask + static_cast<int64_t>(b) * p.Sk : nullptr;
+  const int k_off = l32 * KROW + hh * 8;                                       // K fragment, per lane
+  const int v_off = (((lane & 15) >> 2) + 4 * hh) * VROW + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+  // S^T tile = K(tile in Ks[buf]) Q^T, no softmax work to overlap (prologue only)
+  auto qk_plain = [&](int buf, f32x16_v(&s)[2]) {
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s[kt][e] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+        const frag a = __builtin_bit_cast(
+            frag, *reinterpret_cast<const u32x4_v*>(&Ks[buf][kt * 32 * KROW + k_off + ks * 16]));
+        s[kt] = M::run(a, qf[ks], s[kt]);
+      }
+  };
+
+  // exclusions (keys past Sk, padding mask), then the lane-local part of the row maximum
+  auto mask_and_max = [&](int j, f32x16_v(&s)[2]) -> float {
+    // branch-free selects: every lane rewrites all its scores, excluded ones with -inf
+    if (mrow != nullptr) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const int key = j * BN + kt * 32 + g * 8 + hh * 4 + t;
+            const int kc = key < p.Sk ? key : p.Sk - 1;
+            const bool live = (key < p.Sk) & (mrow[kc] != 0);
+            const float x = s[kt][g * 4 + t];
+            s[kt][g * 4 + t] = live ? x : -INFINITY;
+          }
+    } else if ((j + 1) * BN > p.Sk) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const int key = j * BN + kt * 32 + g * 8 + hh * 4 + t;
+            const float x = s[kt][g * 4 + t];
+            s[kt][g * 4 + t] = key < p.Sk ? x : -INFINITY;
+          }
+    }
+    float mx = s[0][0];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[kt][e]);
+    return mx;
+  };
+
+  // move the reference maximum (and rescale O, l) only when some query outgrew it by more than 2^8
+  auto settle_max = [&](float mx) {
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx);
+    if (__any((m_new - m_run) * c > 8.f)) {
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * c);
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[dt][e] *= alpha;
+      m_run = m_new;
+    }
+  };
+
+  // one tile: s_cur holds S(j) (max already settled); s_next receives S(j+1)
+  auto tile = [&](int j, f32x16_v(&s_cur)[2], f32x16_v(&s_next)[2]) {
+    const int buf = j & 1;
+    const bool has_next = j + 1 < n_tiles;
+    if (j + 2 < n_tiles) gload(kbase, p.ks_s, j + 2, kreg);
+    if (has_next) gload(vbase, p.vs_s, j + 1, vreg);
+
+    const float mc = (m_run == -INFINITY) ? 0.f : m_run * c;
+    uint32_t pf[2][2][4];
+    float psum = 0.f;
+    // ---- stage A ----
+    if (has_next) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s_next[kt][e] = 0.f;
+#pragma unroll
+      for (int i = 0; i < 2 * KS; ++i) {
+        const int ks = i >> 1, kt = i & 1;
+        const frag a = __builtin_bit_cast(
+            frag, *reinterpret_cast<const u32x4_v*>(&Ks[buf ^ 1][kt * 32 * KROW + k_off + ks * 16]));
+        s_next[kt] = M::run(a, qf[ks], s_next[kt]);
+        // 32 / (2*KS) score pairs of S(j) per MFMA
+        constexpr int PAIRS = 16 / (2 * KS) > 0 ? 16 / (2 * KS) : 1;
+#pragma unroll
+        for (int q = 0; q < PAIRS; ++q) {
+          const int pi = i * PAIRS + q;
+          if (pi < 16) {
+            const int pkt = pi >> 3, e0 = (pi & 7) * 2;
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(s_cur[pkt][e0], c, -mc));
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(s_cur[pkt][e0 + 1], c, -mc));
+            psum += p0 + p1;
+            pf[pkt][(pi & 7) >> 2][pi & 3] = M::pack2(p0, p1);
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int pi = 0; pi < 16; ++pi) {
+        const int pkt = pi >> 3, e0 = (pi & 7) * 2;
+        const float p0 = __builtin_amdgcn_exp2f(fmaf(s_cur[pkt][e0], c, -mc));
+        const float p1 = __builtin_amdgcn_exp2f(fmaf(s_cur[pkt][e0 + 1], c, -mc));
+        psum += p0 + p1;
+        pf[pkt][(pi & 7) >> 2][pi & 3] = M::pack2(p0, p1);
+      }
+    }
+    l_run += psum;
+
+    // ---- stage B: O^T += V(j)^T P(j)^T ----
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int g2 = 0; g2 < 2; ++g2) {
+          T* vp = &Vs[buf][(kt * 32 + g2 * 16) * VROW + dt * 32 + v_off];
+          const s16x4_v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(vp));
+          const s16x4_v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(vp + 8 * VROW));
+          typedef short s16x8_v __attribute__((ext_vector_type(8)));
+          const s16x8_v av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          u32x4_v pb;
+          pb.x = pf[kt][g2][0]; pb.y = pf[kt][g2][1]; pb.z = pf[kt][g2][2]; pb.w = pf[kt][g2][3];
+          o[dt] = M::run(__builtin_bit_cast(frag, av), __builtin_bit_cast(frag, pb), o[dt]);
+        }
+
+    float mx = -INFINITY;
+    if (has_next) mx = mask_and_max(j + 1, s_next);
+    if (j + 2 < n_tiles) sstore(&Ks[buf][0], KROW, kreg);
+    if (has_next) sstore(&Vs[buf ^ 1][0], VROW, vreg);
+    __syncthreads();
+    if (has_next) settle_max(mx);
+  };
+
+  // ---- prologue: K(0), V(0), K(1) staged; S(0) computed and its maximum settled ----
+  gload(kbase, p.ks_s, 0, kreg);
+  gload(vbase, p.vs_s, 0, vreg);
+  sstore(&Ks[0][0], KROW, kreg);
+  sstore(&Vs[0][0], VROW, vreg);
+  if (n_tiles > 1) {
+    gload(kbase, p.ks_s, 1, kreg);
+    sstore(&Ks[1][0], KROW, kreg);
+  }
+  __syncthreads();
+  f32x16_v sa[2], sb[2];
+  qk_plain(0, sa);
+  settle_max(mask_and_max(0, sa));
+
+  for (int j = 0; j < n_tiles; j += 2) {
+    tile(j, sa, sb);
+    if (j + 1 < n_tiles) tile(j + 1, sb, sa);
+  }
+
+  // ---- epilogue ----
+  T* obase = static_cast<T*>(p.o) + b * p.os_b + h * p.os_h;
+  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  const int row = q0 + l32;
+  if (row < p.Sq) {
+    T* op = obase + row * p.os_s;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2_v w;
+        w.x = M::pack2(o[dt][g * 4 + 0] * inv, o[dt][g * 4 + 1] * inv);
+        w.y = M::pack2(o[dt][g * 4 + 2] * inv, o[dt][g * 4 + 3] * inv);
+        *reinterpret_cast<u32x2_v*>(op + dt * 32 + g * 8 + hh * 4) = w;
+      }
+    if (p.lse != nullptr && hh == 0) {
+      const float lse = l_tot > 0.f ? m_run * p.scale + __logf(l_tot) : -INFINITY;
+      p.lse[(static_cast<int64_t>(b) * p.H + h) * p.Sq + row] = lse;
+    }
+  }
+}
+
+template <typename T, int D, int NW>
+static int launch_attn_pipe(AttnParams& p, hipStream_t stream) {
+  constexpr int BM = NW * 32;
+  p.n_qblocks = (p.Sq + BM - 1) / BM;
+  const int64_t total = static_cast<int64_t>(p.n_qblocks) * p.H * p.B;
+  if (total > 0x7fffffffll) {
+    set_error("odit_attn_fwd: grid of %lld workgroups is too large", static_cast<long long>(total));
+    return ODIT_EINVAL;
+  }
+  p.total_blocks = static_cast<int>(total);
+  hipLaunchKernelGGL((attn_fwd_pipe_kernel<T, D, NW>), dim3(p.total_blocks), dim3(NW * 64), 0, stream, p);
+  return check_launch("odit_attn_fwd");
+}
+
 template <typename T, int D, int QT, int NW>
 static int launch_attn(AttnParams& p, hipStream_t stream) {
   constexpr int BM = NW * QT * 32;
@@ -362,6 +656,8 @@ static int dispatch_attn(AttnParams& p, int variant, hipStream_t stream) {
     case 14: return launch_attn<T, D, 1, 4>(p, stream);
     case 18: return launch_attn<T, D, 1, 8>(p, stream);
     case 24: return launch_attn<T, D, 2, 4>(p, stream);
+    case 28: return launch_attn_pipe<T, D, 8>(p, stream);
+    case 29: return launch_attn_pipe<T, D, 4>(p, stream);
     default:
       set_error("odit_attn_fwd: unknown tile variant %d", variant);
       return ODIT_EINVAL;
@@ -409,7 +705,7 @@ extern "C" int odit_attn_fwd(const void* q, const void* k, const void* v, void* 
   p.scale = scale;
   p.scale_log2 = scale * 1.4426950408889634f;
 
-  int variant = 24;
+  int variant = 28;
   if (const char* e = getenv("ODIT_ATTN_VARIANT")) variant = atoi(e);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == ODIT_BF16) {
