@@ -105,42 +105,64 @@ def build_model(torch, layers):
     return model.eval()
 
 
+def _time_rot(torch, fns, iters=40, warmup=4):
+    """Average duration (ms) of the closures in `fns`, called round-robin: each closure works on its
+    own buffers, and together the sets exceed the 256 MB last-level cache, so the figure is HBM
+    traffic, not cache hits."""
+    n = len(fns)
+    for i in range(warmup):
+        fns[i % n]()
+    torch.cuda.synchronize()
+    a, b = _events(torch)
+    a.record()
+    for i in range(iters):
+        fns[i % n]()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters
+
+
 def kernel_rooflines(torch):
-    """Achieved GB/s (bandwidth-bound kernels) and TFLOP/s (attention, GEMM) at the config shapes."""
+    """Achieved GB/s (bandwidth-bound kernels) and TFLOP/s (attention, GEMM) at the config shapes.
+    Bytes are the ALGORITHMIC bytes of each kernel (inputs read once + outputs written once)."""
     from vllm_omni_amd import kernels
     from vllm_omni_amd._lib import ODIT_NORM_HEAD
 
     dev = "cuda"
     bf = torch.bfloat16
     out = {}
-    x = torch.randn(B, S_IMG, C, device=dev, dtype=bf)
-    y = torch.randn(B, S_IMG, C, device=dev, dtype=bf)
+    NSET = 8  # 8 x (>= 100 MB) per kernel
+
+    def bw(name, fns, byt):
+        ms = _time_rot(torch, fns)
+        out[name] = {"ms": ms, "GB/s": byt / ms / 1e6, "frac_hbm": byt / ms / 1e6 / PEAK_HBM_GBS,
+                     "algorithmic_bytes": byt}
+
+    xs = [torch.randn(B, S_IMG, C, device=dev, dtype=bf) for _ in range(NSET)]
+    ys = [torch.randn(B, S_IMG, C, device=dev, dtype=bf) for _ in range(NSET)]
+    os_ = [torch.empty(B, S_IMG, C, device=dev, dtype=bf) for _ in range(NSET)]
     mod = torch.randn(B, 3 * C, device=dev, dtype=bf)
     shift, scale, gate = mod.chunk(3, dim=-1)
-    o = torch.empty_like(x)
-    ms = _time_op(torch, lambda: kernels.adaln_modulate(x, shift, scale, out=o))
-    byt = 2 * x.numel() * 2
-    out["adaln_modulate"] = {"ms": ms, "GB/s": byt / ms / 1e6, "frac_hbm": byt / ms / 1e6 / PEAK_HBM_GBS}
-    ms = _time_op(torch, lambda: kernels.gated_residual(x, y, gate, out=o))
-    byt = 3 * x.numel() * 2
-    out["gated_residual"] = {"ms": ms, "GB/s": byt / ms / 1e6, "frac_hbm": byt / ms / 1e6 / PEAK_HBM_GBS}
-    ms = _time_op(torch, lambda: kernels.rel_l1_sums(x, y))
-    byt = 2 * x.numel() * 2
-    out["rel_l1"] = {"ms": ms, "GB/s": byt / ms / 1e6, "frac_hbm": byt / ms / 1e6 / PEAK_HBM_GBS}
-    qkv = torch.randn(B, S_IMG, 3, HEADS, HEAD_DIM, device=dev, dtype=bf)
-    jq = torch.empty(B, S_IMG + S_TXT, HEADS, HEAD_DIM, device=dev, dtype=bf)
-    jk, jv = torch.empty_like(jq), torch.empty_like(jq)
+    n_el = xs[0].numel()
+    bw("adaln_modulate", [lambda i=i: kernels.adaln_modulate(xs[i], shift, scale, out=os_[i]) for i in range(NSET)],
+       2 * n_el * 2)
+    bw("gated_residual", [lambda i=i: kernels.gated_residual(xs[i], ys[i], gate, out=os_[i]) for i in range(NSET)],
+       3 * n_el * 2)
+    bw("rel_l1", [lambda i=i: kernels.rel_l1_sums(xs[i], ys[i]) for i in range(NSET)], 2 * n_el * 2)
+    del ys
+    qkvs = [torch.randn(B, S_IMG, 3, HEADS, HEAD_DIM, device=dev, dtype=bf) for _ in range(NSET)]
+    jqs = [[torch.empty(B, S_IMG + S_TXT, HEADS, HEAD_DIM, device=dev, dtype=bf) for _ in range(3)] for _ in range(NSET)]
     w = torch.ones(HEAD_DIM, device=dev, dtype=bf)
     cos = torch.rand(S_IMG, HEAD_DIM // 2, device=dev)
     sin = torch.rand(S_IMG, HEAD_DIM // 2, device=dev)
-    ms = _time_op(torch, lambda: kernels.qknorm_rope(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], jq, jk, jv, w, w,
-                                                     cos, sin, out_seq_offset=S_TXT, norm_mode=ODIT_NORM_HEAD))
-    byt = 2 * qkv.numel() * 2
-    out["qknorm_rope"] = {"ms": ms, "GB/s": byt / ms / 1e6, "frac_hbm": byt / ms / 1e6 / PEAK_HBM_GBS}
-    u = torch.randn(B * S_IMG, MLP_RATIO * C, device=dev, dtype=bf)
-    ms = _time_op(torch, lambda: kernels.gelu_tanh(u, out=u))
-    byt = 2 * u.numel() * 2
-    out["gelu_tanh"] = {"ms": ms, "GB/s": byt / ms / 1e6, "frac_hbm": byt / ms / 1e6 / PEAK_HBM_GBS}
+    bw("qknorm_rope",
+       [lambda i=i: kernels.qknorm_rope(qkvs[i][:, :, 0], qkvs[i][:, :, 1], qkvs[i][:, :, 2], jqs[i][0], jqs[i][1],
+                                        jqs[i][2], w, w, cos, sin, out_seq_offset=S_TXT, norm_mode=ODIT_NORM_HEAD)
+        for i in range(NSET)], 2 * qkvs[0].numel() * 2)
+    del qkvs, jqs, xs, os_
+    us = [torch.randn(B * S_IMG, MLP_RATIO * C, device=dev, dtype=bf) for _ in range(4)]
+    bw("gelu_tanh", [lambda i=i: kernels.gelu_tanh(us[i], out=us[i]) for i in range(4)], 2 * us[0].numel() * 2)
+    del us
     S = S_IMG + S_TXT
     q = torch.randn(B, S, HEADS, HEAD_DIM, device=dev, dtype=bf)
     k, v = torch.randn_like(q), torch.randn_like(q)

@@ -1,9 +1,9 @@
-// K3: fused LayerNorm + adaLN shift/scale modulation, one 64-lane wavefront per token row.
+// K3: fused LayerNorm + adaLN shift/scale modulation.
 //
-// The row is read from HBM exactly once: each lane keeps NV 16-byte vectors of it in registers,
-// the two LayerNorm statistics are reduced across the wavefront with cross-lane shuffles (no LDS,
-// no barrier), and the modulated row is written back once. Algorithmic traffic is therefore
-// 2 * B*S*C * sizeof(T) (+ the [B,C] shift/scale rows, which stay L2-resident).
+// The row is read from HBM exactly once (each lane keeps one or two 16-byte vectors of it in
+// registers), both LayerNorm moments come from that single sweep, and the modulated row is written
+// back once. Algorithmic traffic is therefore 2 * B*S*C * sizeof(T) (+ the [B,C] shift/scale rows,
+// which stay L2-resident).
 #include "odit_common.h"
 
 namespace odit {
@@ -32,47 +32,60 @@ __device__ __forceinline__ void load_params(const TP* p, float fill, float (&dst
   }
 }
 
-template <typename T, typename TM, int NV, bool REF_ROUND>
-__global__ __launch_bounds__(256) void adaln_rows_kernel(
+// One workgroup of W wavefronts per token row; every lane holds at most NVL 16-byte vectors of the
+// row (as loaded, unpacked where used), so the kernel needs few registers and many rows are in flight
+// per CU: while some waves wait for their loads others reduce or store, which is what keeps a
+// read-once / write-once pass near the HBM rate. The two LayerNorm moments are taken in one sweep
+// about the row's first element (a shift every wave can fetch by itself) and combined across the W
+// waves through 2*W floats of LDS.
+template <typename T, typename TM, int W, int NVL, bool REF_ROUND>
+__global__ __launch_bounds__(W * 64) void adaln_rows_kernel(
     const T* __restrict__ x, T* __restrict__ out, const TM* __restrict__ shift,
     const TM* __restrict__ scale, const int32_t* __restrict__ index,
     const float* __restrict__ ln_w, const float* __restrict__ ln_b, int B, int S, int C,
     int64_t xs_b, int64_t xs_s, int64_t os_b, int64_t os_s, int64_t mod_stride_b, float eps) {
   constexpr int EPV = Vec16<T>::N;
-  const int lane = threadIdx.x & 63;
-  const int64_t row = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (row >= static_cast<int64_t>(B) * S) return;
+  const int tid = threadIdx.x;
+  const int64_t row = blockIdx.x;
   const int b = static_cast<int>(row / S);
   const int s = static_cast<int>(row - static_cast<int64_t>(b) * S);
   const T* xr = x + b * xs_b + s * xs_s;
   T* orow = out + b * os_b + s * os_s;
 
-  float v[NV][EPV];
-  float sum = 0.f;
+  u32x4 raw[NVL];
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int c0 = (i * 64 + lane) * EPV;
+  for (int i = 0; i < NVL; ++i) {
+    const int c0 = (i * (W * 64) + tid) * EPV;
+    raw[i] = c0 < C ? load_raw(xr + c0) : u32x4{0u, 0u, 0u, 0u};
+  }
+  const float k0 = to_float(xr[0]);  // same address for the whole workgroup: one broadcast load
+  float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < NVL; ++i) {
+    const int c0 = (i * (W * 64) + tid) * EPV;
     if (c0 < C) {
-      Vec16<T> t = load16(xr + c0);
 #pragma unroll
-      for (int j = 0; j < EPV; ++j) { v[i][j] = to_float(t.e[j]); sum += v[i][j]; }
-    } else {
-#pragma unroll
-      for (int j = 0; j < EPV; ++j) v[i][j] = 0.f;
+      for (int j = 0; j < EPV; ++j) {
+        const float d = Raw<T>::get(raw[i], j) - k0;
+        s1 += d;
+        s2 = fmaf(d, d, s2);
+      }
     }
+  }
+  s1 = wave_sum(s1);
+  s2 = wave_sum(s2);
+  if (W > 1) {
+    __shared__ float red[2][W];
+    if ((tid & 63) == 0) { red[0][tid >> 6] = s1; red[1][tid >> 6] = s2; }
+    __syncthreads();
+    s1 = 0.f; s2 = 0.f;
+#pragma unroll
+    for (int w = 0; w < W; ++w) { s1 += red[0][w]; s2 += red[1][w]; }
   }
   const float inv_c = 1.f / static_cast<float>(C);
-  const float mean = wave_sum(sum) * inv_c;
-  float sq = 0.f;
-#pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int c0 = (i * 64 + lane) * EPV;
-    if (c0 < C) {
-#pragma unroll
-      for (int j = 0; j < EPV; ++j) { const float d = v[i][j] - mean; sq += d * d; }
-    }
-  }
-  const float rstd = rsqrtf(wave_sum(sq) * inv_c + eps);
+  const float m1 = s1 * inv_c;
+  const float mean = k0 + m1;
+  const float rstd = rsqrtf(fmaxf(s2 * inv_c - m1 * m1, 0.f) + eps);
 
   int mrow = b;
   if (index != nullptr && index[static_cast<int64_t>(b) * S + s] != 0) mrow = b + B;
@@ -80,33 +93,31 @@ __global__ __launch_bounds__(256) void adaln_rows_kernel(
   const TM* sc = scale ? scale + mrow * mod_stride_b : nullptr;
 
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int c0 = (i * 64 + lane) * EPV;
+  for (int i = 0; i < NVL; ++i) {
+    const int c0 = (i * (W * 64) + tid) * EPV;
     if (c0 < C) {
-      Vec16<T> o;
       float scl_v[EPV], shf_v[EPV], lw_v[EPV], lb_v[EPV];
       load_params<TM, EPV>(sc ? sc + c0 : nullptr, 0.f, scl_v);
       load_params<TM, EPV>(sh ? sh + c0 : nullptr, 0.f, shf_v);
       load_params<float, EPV>(ln_w ? ln_w + c0 : nullptr, 1.f, lw_v);
       load_params<float, EPV>(ln_b ? ln_b + c0 : nullptr, 0.f, lb_v);
+      float r[EPV];
 #pragma unroll
       for (int j = 0; j < EPV; ++j) {
-        float y = (v[i][j] - mean) * rstd;
+        float y = (Raw<T>::get(raw[i], j) - mean) * rstd;
         if (ln_w) y *= lw_v[j];
         if (ln_b) y += lb_v[j];
-        const float scl = scl_v[j];
-        const float shf = shf_v[j];
-        float r;
         if (REF_ROUND) {
           // torch path: LN -> T, (1 + scale) -> T, product -> T, sum -> T
-          r = round_to<T>(round_to<T>(y) * round_to<T>(1.f + scl));
-          r = r + shf;
+          r[j] = round_to<T>(round_to<T>(y) * round_to<T>(1.f + scl_v[j])) + shf_v[j];
         } else {
-          r = fmaf(y, 1.f + scl, shf);
+          r[j] = fmaf(y, 1.f + scl_v[j], shf_v[j]);
         }
-        o.e[j] = from_float<T>(r);
       }
-      store16(orow + c0, o);
+      u32x4 o;
+#pragma unroll
+      for (int j = 0; j < EPV / 2; ++j) Raw<T>::set2(o, j, r[2 * j], r[2 * j + 1]);
+      __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(orow + c0));
     }
   }
 }
@@ -158,32 +169,30 @@ static int launch_adaln(const void* x, void* out, const void* shift, const void*
                         int C, const int64_t* xs, const int64_t* os, int64_t mod_stride_b, float eps,
                         hipStream_t stream) {
   constexpr int EPV = Vec16<T>::N;
-  const int64_t rows = static_cast<int64_t>(B) * S;
-  const dim3 block(256);
-  const dim3 grid(static_cast<unsigned>((rows + 3) / 4));
   constexpr int EPM = Vec16<TM>::N;
+  const int64_t rows = static_cast<int64_t>(B) * S;
   // EPV >= EPM always (TM is T or float), so C % EPV == 0 keeps parameter runs vector-aligned too.
   const bool vec_ok = (C % EPV == 0) && aligned16(x) && aligned16(out) && xs[0] % EPV == 0 &&
                       xs[1] % EPV == 0 && os[0] % EPV == 0 && os[1] % EPV == 0 &&
                       aligned16(shift) && aligned16(scale) && mod_stride_b % EPM == 0 &&
                       aligned16(ln_w) && aligned16(ln_b);
-  const int nv = (C + 64 * EPV - 1) / (64 * EPV);
-#define ODIT_ADALN_CASE(NVV)                                                                   \
-  hipLaunchKernelGGL((adaln_rows_kernel<T, TM, NVV, REF_ROUND>), grid, block, 0, stream,       \
-                     static_cast<const T*>(x), static_cast<T*>(out),                           \
-                     static_cast<const TM*>(shift), static_cast<const TM*>(scale), index, ln_w, \
+  const int nvec = (C + EPV - 1) / EPV;  // 16-byte vectors per row
+#define ODIT_ADALN_CASE(WW, NVLL)                                                                  \
+  hipLaunchKernelGGL((adaln_rows_kernel<T, TM, WW, NVLL, REF_ROUND>), dim3(static_cast<unsigned>(rows)), \
+                     dim3(WW * 64), 0, stream, static_cast<const T*>(x), static_cast<T*>(out),     \
+                     static_cast<const TM*>(shift), static_cast<const TM*>(scale), index, ln_w,    \
                      ln_b, B, S, C, xs[0], xs[1], os[0], os[1], mod_stride_b, eps)
-  if (vec_ok && nv <= 16) {
-    if (nv <= 1) ODIT_ADALN_CASE(1);
-    else if (nv <= 2) ODIT_ADALN_CASE(2);
-    else if (nv <= 4) ODIT_ADALN_CASE(4);
-    else if (nv <= 6) ODIT_ADALN_CASE(6);
-    else if (nv <= 8) ODIT_ADALN_CASE(8);
-    else if (nv <= 10) ODIT_ADALN_CASE(10);
-    else if (nv <= 12) ODIT_ADALN_CASE(12);
-    else ODIT_ADALN_CASE(16);
+  if (vec_ok && nvec <= 8 * 64 * 2 && rows <= 0x7fffffffll) {
+    if (nvec <= 64) ODIT_ADALN_CASE(1, 1);
+    else if (nvec <= 128) ODIT_ADALN_CASE(2, 1);
+    else if (nvec <= 256) ODIT_ADALN_CASE(4, 1);
+    else if (nvec <= 384) ODIT_ADALN_CASE(3, 2);
+    else if (nvec <= 512) ODIT_ADALN_CASE(4, 2);
+    else if (nvec <= 768) ODIT_ADALN_CASE(6, 2);
+    else ODIT_ADALN_CASE(8, 2);
   } else {
-    hipLaunchKernelGGL((adaln_rows_generic_kernel<T, TM, REF_ROUND>), grid, block, 0, stream,
+    const dim3 grid(static_cast<unsigned>((rows + 3) / 4));
+    hipLaunchKernelGGL((adaln_rows_generic_kernel<T, TM, REF_ROUND>), grid, dim3(256), 0, stream,
                        static_cast<const T*>(x), static_cast<T*>(out),
                        static_cast<const TM*>(shift), static_cast<const TM*>(scale), index, ln_w,
                        ln_b, B, S, C, xs[0], xs[1], os[0], os[1], mod_stride_b, eps);

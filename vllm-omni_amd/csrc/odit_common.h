@@ -77,16 +77,84 @@ template <typename T> __device__ __forceinline__ void store16(T* p, const Vec16<
   *reinterpret_cast<uint4*>(p) = *reinterpret_cast<const uint4*>(&v);
 }
 
+// ---- raw 16-byte register vectors --------------------------------------------------------------
+// Rows kept in registers are held as the 16 bytes that were loaded (a native 4 x u32 vector) and
+// unpacked element by element where they are used: a bf16 unpack is one shift or one and.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+template <typename T> __device__ __forceinline__ u32x4 load_raw(const T* p) {
+  return *reinterpret_cast<const u32x4*>(p);
+}
+template <typename T> __device__ __forceinline__ void store_raw(T* p, u32x4 v) {
+  *reinterpret_cast<u32x4*>(p) = v;
+}
+
+template <typename T> struct Raw;
+template <> struct Raw<bf16_t> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ float get(u32x4 v, int j) {
+    const uint32_t w = v[j >> 1];
+    return __uint_as_float((j & 1) ? (w & 0xffff0000u) : (w << 16));
+  }
+  // writes elements 2*pair and 2*pair+1
+  static __device__ __forceinline__ void set2(u32x4& v, int pair, float lo, float hi) {
+    const f32x2 f = {lo, hi};
+    v[pair] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+  }
+};
+template <> struct Raw<f16_t> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ float get(u32x4 v, int j) {
+    const uint32_t w = v[j >> 1];
+    const uint16_t h = static_cast<uint16_t>((j & 1) ? (w >> 16) : (w & 0xffffu));
+    return static_cast<float>(__builtin_bit_cast(_Float16, h));
+  }
+  static __device__ __forceinline__ void set2(u32x4& v, int pair, float lo, float hi) {
+    const f32x2 f = {lo, hi};
+    v[pair] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
+  }
+};
+template <> struct Raw<float> {
+  static constexpr int N = 4;
+  static __device__ __forceinline__ float get(u32x4 v, int j) { return __uint_as_float(v[j]); }
+  static __device__ __forceinline__ void set2(u32x4& v, int pair, float lo, float hi) {
+    v[2 * pair] = __float_as_uint(lo);
+    v[2 * pair + 1] = __float_as_uint(hi);
+  }
+};
+
 // ---- wavefront (64 lanes) reductions ------------------------------------------------------------
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+// Cross-lane adds inside a 16-lane DPP row cost one VALU instruction each (no LDS crossbar trip):
+// xor-1 and xor-2 quad permutes, then the half-row and full-row mirrors.
+template <int CTRL> __device__ __forceinline__ float dpp_add(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
+  return v + __int_as_float(moved);
+}
+// sum over aligned groups of G consecutive lanes, G in {2,4,8,16}; every lane of a group gets the sum
+template <int G> __device__ __forceinline__ float row_group_sum(float v) {
+  static_assert(G == 1 || G == 2 || G == 4 || G == 8 || G == 16, "group must fit a 16-lane row");
+  if (G >= 2) v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+  if (G >= 4) v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+  if (G >= 8) v = dpp_add<0x141>(v);  // row_half_mirror
+  if (G >= 16) v = dpp_add<0x140>(v); // row_mirror
   return v;
+}
+// sum over the whole wavefront, returned in every lane (wave-uniform)
+__device__ __forceinline__ float wave_sum(float v) {
+  v = row_group_sum<16>(v);
+  const int iv = __float_as_int(v);
+  return __int_as_float(__builtin_amdgcn_readlane(iv, 0)) + __int_as_float(__builtin_amdgcn_readlane(iv, 16)) +
+         __int_as_float(__builtin_amdgcn_readlane(iv, 32)) + __int_as_float(__builtin_amdgcn_readlane(iv, 48));
 }
 // sum over aligned groups of G consecutive lanes (G power of two <= 64)
 template <int G> __device__ __forceinline__ float group_sum(float v) {
-#pragma unroll
-  for (int off = G / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  if (G <= 16) return row_group_sum<(G <= 16 ? G : 16)>(v);
+  v = row_group_sum<16>(v);
+  if (G >= 32) v += __shfl_xor(v, 16, 64);
+  if (G >= 64) v += __shfl_xor(v, 32, 64);
   return v;
 }
 

@@ -5,6 +5,8 @@
 
 namespace odit {
 
+constexpr int kStreamUnroll = 1;  // 16-byte vectors per thread; measured: more per thread streams slower here
+
 template <typename T, typename TG, bool REF_ROUND>
 __global__ __launch_bounds__(256) void gated_residual_kernel(
     const T* __restrict__ h, const T* __restrict__ y, const TG* __restrict__ gate,
@@ -12,36 +14,53 @@ __global__ __launch_bounds__(256) void gated_residual_kernel(
     int64_t ys_b, int64_t ys_s, int64_t os_b, int64_t os_s, int64_t gs_b, int64_t gs_s) {
   constexpr int EPV = Vec16<T>::N;
   constexpr int EPG = Vec16<TG>::N;
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total_vecs;
-       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-    const int64_t row = i / vec_per_row;
-    const int c0 = static_cast<int>(i - row * vec_per_row) * EPV;
-    const int b = static_cast<int>(row / S);
-    const int s = static_cast<int>(row - static_cast<int64_t>(b) * S);
-    const Vec16<T> hv = load16(h + b * hs_b + s * hs_s + c0);
-    const Vec16<T> yv = load16(y + b * ys_b + s * ys_s + c0);
-    float g[EPV];
-    if (gate != nullptr) {
-      const TG* gp = gate + b * gs_b + s * gs_s + c0;
+  constexpr int U = kStreamUnroll;
+  // a block owns 256*U consecutive vectors; vector u of a thread sits 256 vectors after vector u-1,
+  // so every load/store instruction of the block touches one contiguous 4 KB run
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * (256 * U) + threadIdx.x;
+  Vec16<T> hv[U], yv[U];
+  float g[U][EPV];
+  int64_t ooff[U];
+  bool ok[U];
 #pragma unroll
-      for (int q = 0; q < EPV / EPG; ++q) {
-        const Vec16<TG> gv = load16(gp + q * EPG);
+  for (int u = 0; u < U; ++u) {
+    const int64_t i = base + u * 256;
+    ok[u] = i < total_vecs;
+    if (ok[u]) {
+      const int64_t row = i / vec_per_row;
+      const int c0 = static_cast<int>(i - row * vec_per_row) * EPV;
+      const int b = static_cast<int>(row / S);
+      const int s = static_cast<int>(row - static_cast<int64_t>(b) * S);
+      hv[u] = load16(h + b * hs_b + s * hs_s + c0);
+      yv[u] = load16(y + b * ys_b + s * ys_s + c0);
+      ooff[u] = b * os_b + s * os_s + c0;
+      if (gate != nullptr) {
+        const TG* gp = gate + b * gs_b + s * gs_s + c0;
 #pragma unroll
-        for (int j = 0; j < EPG; ++j) g[q * EPG + j] = to_float(gv.e[j]);
+        for (int q = 0; q < EPV / EPG; ++q) {
+          const Vec16<TG> gv = load16(gp + q * EPG);
+#pragma unroll
+          for (int j = 0; j < EPG; ++j) g[u][q * EPG + j] = to_float(gv.e[j]);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) g[u][j] = 1.f;
       }
-    } else {
-#pragma unroll
-      for (int j = 0; j < EPV; ++j) g[j] = 1.f;
     }
-    Vec16<T> ov;
+  }
 #pragma unroll
-    for (int j = 0; j < EPV; ++j) {
-      const float hf = to_float(hv.e[j]);
-      const float yf = to_float(yv.e[j]);
-      const float r = REF_ROUND ? hf + round_to<T>(g[j] * yf) : fmaf(g[j], yf, hf);
-      ov.e[j] = from_float<T>(r);
+  for (int u = 0; u < U; ++u) {
+    if (ok[u]) {
+      Vec16<T> ov;
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) {
+        const float hf = to_float(hv[u].e[j]);
+        const float yf = to_float(yv[u].e[j]);
+        const float r = REF_ROUND ? hf + round_to<T>(g[u][j] * yf) : fmaf(g[u][j], yf, hf);
+        ov.e[j] = from_float<T>(r);
+      }
+      __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(&ov), reinterpret_cast<u32x4*>(out + ooff[u]));
     }
-    store16(out + b * os_b + s * os_s + c0, ov);
   }
 }
 
@@ -85,7 +104,8 @@ static int launch_gated(const void* h, const void* y, const void* gate, void* ou
   if (vec_ok) {
     const int vpr = C / EPV;
     const int64_t total = static_cast<int64_t>(B) * S * vpr;
-    hipLaunchKernelGGL((gated_residual_kernel<T, TG, REF_ROUND>), dim3(stream_grid(total)),
+    const int64_t nblk = (total + 256 * kStreamUnroll - 1) / (256 * kStreamUnroll);
+    hipLaunchKernelGGL((gated_residual_kernel<T, TG, REF_ROUND>), dim3(static_cast<unsigned>(nblk)),
                        dim3(256), 0, stream, static_cast<const T*>(h), static_cast<const T*>(y),
                        static_cast<const TG*>(gate), static_cast<T*>(out), S, vpr, total, hs[0],
                        hs[1], ys[0], ys[1], os[0], os[1], gs0, gs1);
@@ -115,24 +135,37 @@ template <typename T, typename F>
 __global__ __launch_bounds__(256) void unary_kernel(const T* __restrict__ x, T* __restrict__ out,
                                                     int64_t n_vec, int64_t n) {
   constexpr int EPV = Vec16<T>::N;
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
-  const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  for (int64_t i = tid; i < n_vec; i += stride) {
-    Vec16<T> v = load16(x + i * EPV);
+  constexpr int U = kStreamUnroll;
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * (256 * U) + threadIdx.x;
+  Vec16<T> v[U];
 #pragma unroll
-    for (int j = 0; j < EPV; ++j) v.e[j] = from_float<T>(F::apply(to_float(v.e[j])));
-    store16(out + i * EPV, v);
+  for (int u = 0; u < U; ++u) {
+    const int64_t i = base + u * 256;
+    if (i < n_vec) v[u] = load16(x + i * EPV);
   }
-  for (int64_t i = n_vec * EPV + tid; i < n; i += stride)
-    out[i] = from_float<T>(F::apply(to_float(x[i])));
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int64_t i = base + u * 256;
+    if (i < n_vec) {
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) v[u].e[j] = from_float<T>(F::apply(to_float(v[u].e[j])));
+      __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(&v[u]), reinterpret_cast<u32x4*>(out + i * EPV));
+    }
+  }
+  // scalar tail (and the whole array when 16-byte access is not possible): first block only
+  if (blockIdx.x == 0)
+    for (int64_t i = n_vec * EPV + threadIdx.x; i < n; i += 256)
+      out[i] = from_float<T>(F::apply(to_float(x[i])));
 }
 
 template <typename T, typename F>
 static int launch_unary(const void* x, void* out, int64_t n, hipStream_t stream, const char* what) {
   constexpr int EPV = Vec16<T>::N;
   const int64_t n_vec = (aligned16(x) && aligned16(out)) ? n / EPV : 0;
-  hipLaunchKernelGGL((unary_kernel<T, F>), dim3(stream_grid(n_vec > 0 ? n_vec : n)), dim3(256), 0,
-                     stream, static_cast<const T*>(x), static_cast<T*>(out), n_vec, n);
+  int64_t nblk = (n_vec + 256 * kStreamUnroll - 1) / (256 * kStreamUnroll);
+  if (nblk < 1) nblk = 1;
+  hipLaunchKernelGGL((unary_kernel<T, F>), dim3(static_cast<unsigned>(nblk)), dim3(256), 0, stream,
+                     static_cast<const T*>(x), static_cast<T*>(out), n_vec, n);
   return check_launch(what);
 }
 

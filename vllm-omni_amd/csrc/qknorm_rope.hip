@@ -1,14 +1,16 @@
 // K2: fused QK-RMSNorm + rotary embedding + scatter of q/k/v into the joint [txt;img] buffers.
 //
-// One 64-lane wavefront per token. The token's q, k and v rows (H*D elements each, usually three
-// adjacent slices of one fused-QKV GEMM output row) are each read once with 16-byte loads and
-// written once into row (out_seq_offset + s) of the dense joint buffers, so the three torch.cat
-// copies of the reference never happen. Algorithmic traffic: 2 * 3 * B*S*H*D * sizeof(T)
-// (+ S*rot*4 bytes of cos/sin, L2-resident across heads and batch).
+// The q, k and v rows of a token (H*D elements each, usually three adjacent slices of one fused-QKV
+// GEMM output row) are each read once with 16-byte loads and written once into row
+// (out_seq_offset + s) of the dense joint buffers, so the three torch.cat copies of the reference
+// never happen. Algorithmic traffic: 2 * 3 * B*S*H*D * sizeof(T) (+ S*rot*4 bytes of cos/sin and the
+// norm weights, cache-resident across heads and batch).
 //
-// Lane layout: vector i*64+lane of the row covers elements e0..e0+EPV-1, e0 = (i*64+lane)*EPV, i.e.
-// head e0/D, offset e0%D. A head row occupies D/EPV consecutive lanes, so the per-head mean square
-// is a shuffle reduction over an aligned lane group; the whole-row variant reduces over the wave.
+// Per-head statistics (and no statistics): one 16-byte vector per lane, a flat one-shot grid over
+// all vectors of one part (grid.y = q | k | v). A head row is D/EPV consecutive lanes, so its mean
+// square is a DPP reduction inside a 16-lane row (one shuffle more for 32 lanes); the kernel uses
+// ~40 registers, so a CU keeps many loads in flight. Whole-row statistics (Wan): one wavefront per
+// (token, part) holding the row in registers, reduced across the wavefront.
 // Interleaved rotary pairs (2i, 2i+1) live inside one lane's vector; NeoX pairs are fetched from the
 // lane rot/(2*EPV) away with a shuffle.
 #include "odit_common.h"
@@ -28,201 +30,203 @@ template <int N> __device__ __forceinline__ void load_floats(const float* p, flo
   }
 }
 
-// GENERAL = false compiles the hot variant only (interleaved pairs, one final rounding); GENERAL =
-// true takes NeoX pairing and reference rounding as wave-uniform run-time switches.
-template <typename T, typename TW, int NV, int NORM_MODE, bool GENERAL>
-__device__ __forceinline__ void norm_rope_row(const T* __restrict__ in, T* __restrict__ out,
-                                              const TW* __restrict__ w,
-                                              const float* __restrict__ cos_row,
-                                              const float* __restrict__ sin_row, int HD, int D,
-                                              int rot, float eps, int lane, bool neox_rt,
+// Weight multiply + rotation of ONE 16-byte vector x (already unpacked to float) that starts at
+// offset d0 of its head. `wp` points at the weights of this vector (or is null), `rstd` is the
+// reciprocal RMS that applies to it. GENERAL = false compiles the hot variant only (interleaved pairs,
+// one final rounding); GENERAL = true takes NeoX pairing and reference rounding as wave-uniform
+// run-time switches. Must be called by all lanes of the wavefront (the NeoX path shuffles).
+template <typename T, typename TW, bool NORM, bool HEAD_ROUNDING, bool GENERAL>
+__device__ __forceinline__ void transform_vec(float (&x)[Vec16<T>::N], float rstd, const TW* wp,
+                                              const float* cos_row, const float* sin_row, int d0,
+                                              int rot, bool valid, int lane, bool neox_rt,
                                               bool ref_round_rt) {
   constexpr int EPV = Vec16<T>::N;
   const bool NEOX = GENERAL && neox_rt;
   const bool REF_ROUND = GENERAL && ref_round_rt;
-  float v[NV][EPV];
+  if constexpr (NORM) {
+    float wv[EPV];
+    if (wp != nullptr && valid) {
+      constexpr int EW = Vec16<TW>::N;
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int e0 = (i * 64 + lane) * EPV;
-    if (e0 < HD) {
-      const Vec16<T> t = load16(in + e0);
+      for (int q = 0; q < EPV / EW; ++q) {
+        const Vec16<TW> t = load16(wp + q * EW);
 #pragma unroll
-      for (int j = 0; j < EPV; ++j) v[i][j] = to_float(t.e[j]);
+        for (int j = 0; j < EW; ++j) wv[q * EW + j] = to_float(t.e[j]);
+      }
     } else {
 #pragma unroll
-      for (int j = 0; j < EPV; ++j) v[i][j] = 0.f;
+      for (int j = 0; j < EPV; ++j) wv[j] = 1.f;
     }
-  }
-
-  // ---- RMS statistics ----
-  float rstd[NV];
-  if constexpr (NORM_MODE == ODIT_NORM_ROW) {
-    float sq = 0.f;
 #pragma unroll
-    for (int i = 0; i < NV; ++i)
-#pragma unroll
-      for (int j = 0; j < EPV; ++j) sq += v[i][j] * v[i][j];
-    const float r = rsqrtf(wave_sum(sq) / static_cast<float>(HD) + eps);
-#pragma unroll
-    for (int i = 0; i < NV; ++i) rstd[i] = r;
-  } else if constexpr (NORM_MODE == ODIT_NORM_HEAD) {
-    const int lanes_per_head = D / EPV;  // power of two, <= 64 (checked on the host)
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      float sq = 0.f;
-#pragma unroll
-      for (int j = 0; j < EPV; ++j) sq += v[i][j] * v[i][j];
-      for (int off = lanes_per_head >> 1; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
-      rstd[i] = rsqrtf(sq / static_cast<float>(D) + eps);
-    }
-  }
-
-#pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int e0 = (i * 64 + lane) * EPV;
-    const int d0 = e0 % D;
-    float x[EPV];
-#pragma unroll
-    for (int j = 0; j < EPV; ++j) x[j] = v[i][j];
-
-    if constexpr (NORM_MODE != ODIT_NORM_NONE) {
-      float wv[EPV];
-      if (w != nullptr && e0 < HD) {
-        const TW* wp = w + (NORM_MODE == ODIT_NORM_ROW ? e0 : d0);
-        constexpr int EW = Vec16<TW>::N;
-#pragma unroll
-        for (int q = 0; q < EPV / EW; ++q) {
-          const Vec16<TW> t = load16(wp + q * EW);
-#pragma unroll
-          for (int j = 0; j < EW; ++j) wv[q * EW + j] = to_float(t.e[j]);
-        }
+    for (int j = 0; j < EPV; ++j) {
+      if (REF_ROUND && HEAD_ROUNDING) {
+        x[j] = round_to<T>(round_to<T>(x[j] * rstd) * wv[j]);  // vLLM RMSNorm: cast, then weight
       } else {
-#pragma unroll
-        for (int j = 0; j < EPV; ++j) wv[j] = 1.f;
+        x[j] = x[j] * rstd * wv[j];
+        if (REF_ROUND) x[j] = round_to<T>(x[j]);
       }
+    }
+  }
+  if (cos_row == nullptr) return;
+  if (!NEOX) {
+    if (d0 < rot && valid) {
+      float c[EPV / 2], s[EPV / 2];
+      load_floats<EPV / 2>(cos_row + (d0 >> 1), c);
+      load_floats<EPV / 2>(sin_row + (d0 >> 1), s);
+#pragma unroll
+      for (int j = 0; j < EPV / 2; ++j) {
+        const float x0 = x[2 * j], x1 = x[2 * j + 1];
+        if (REF_ROUND) {
+          const float cc = round_to<T>(c[j]), ss = round_to<T>(s[j]);
+          x[2 * j] = round_to<T>(x0 * cc) - round_to<T>(x1 * ss);
+          x[2 * j + 1] = round_to<T>(x1 * cc) + round_to<T>(x0 * ss);
+        } else {
+          x[2 * j] = x0 * c[j] - x1 * s[j];
+          x[2 * j + 1] = x1 * c[j] + x0 * s[j];
+        }
+      }
+    }
+  } else {
+    // pair (d, d + rot/2): the partner vector sits rot/(2*EPV) lanes away inside the same head row
+    const int half = rot >> 1;
+    const int dist = half / EPV;
+    const bool lower = d0 < half;
+    const int src = lower ? lane + dist : lane - dist;
+    float px[EPV];
+#pragma unroll
+    for (int j = 0; j < EPV; ++j) px[j] = __shfl(x[j], src & 63, 64);
+    if (d0 < rot && valid) {
+      const int t0 = lower ? d0 : d0 - half;
+      const float sgn = lower ? -1.f : 1.f;
 #pragma unroll
       for (int j = 0; j < EPV; ++j) {
-        if (REF_ROUND && NORM_MODE == ODIT_NORM_HEAD) {
-          x[j] = round_to<T>(round_to<T>(x[j] * rstd[i]) * wv[j]);
+        const float cj = cos_row[t0 + j], sj = sin_row[t0 + j];
+        if (REF_ROUND) {
+          x[j] = round_to<T>(x[j] * round_to<T>(cj)) + round_to<T>(sgn * px[j] * round_to<T>(sj));
         } else {
-          x[j] = x[j] * rstd[i] * wv[j];
-          if (REF_ROUND) x[j] = round_to<T>(x[j]);
+          x[j] = x[j] * cj + sgn * px[j] * sj;
         }
       }
-    }
-
-    // ---- rotary ----
-    if (cos_row != nullptr) {
-      if (!NEOX) {
-        if (d0 < rot && e0 < HD) {
-          float c[EPV / 2], s[EPV / 2];
-          load_floats<EPV / 2>(cos_row + (d0 >> 1), c);
-          load_floats<EPV / 2>(sin_row + (d0 >> 1), s);
-#pragma unroll
-          for (int j = 0; j < EPV / 2; ++j) {
-            const float x0 = x[2 * j], x1 = x[2 * j + 1];
-            if (REF_ROUND) {
-              const float cc = round_to<T>(c[j]), ss = round_to<T>(s[j]);
-              x[2 * j] = round_to<T>(x0 * cc) - round_to<T>(x1 * ss);
-              x[2 * j + 1] = round_to<T>(x1 * cc) + round_to<T>(x0 * ss);
-            } else {
-              x[2 * j] = x0 * c[j] - x1 * s[j];
-              x[2 * j + 1] = x1 * c[j] + x0 * s[j];
-            }
-          }
-        }
-      } else {
-        // pair (d, d + rot/2): partner vector sits rot/(2*EPV) lanes away (same i: a head row never
-        // straddles two register vectors of one lane because D/EPV lanes hold it contiguously)
-        const int half = rot >> 1;
-        const int dist = half / EPV;
-        const bool lower = d0 < half;
-        const int src = lower ? lane + dist : lane - dist;
-        float px[EPV];
-#pragma unroll
-        for (int j = 0; j < EPV; ++j) px[j] = __shfl(x[j], src & 63, 64);
-        if (d0 < rot && e0 < HD) {
-          float c[EPV], s[EPV];
-          const int t0 = lower ? d0 : d0 - half;
-#pragma unroll
-          for (int j = 0; j < EPV; ++j) { c[j] = cos_row[t0 + j]; s[j] = sin_row[t0 + j]; }
-#pragma unroll
-          for (int j = 0; j < EPV; ++j) {
-            const float sgn = lower ? -1.f : 1.f;
-            if (REF_ROUND) {
-              const float cc = round_to<T>(c[j]), ss = round_to<T>(s[j]);
-              x[j] = round_to<T>(x[j] * cc) + round_to<T>(sgn * px[j] * ss);
-            } else {
-              x[j] = x[j] * c[j] + sgn * px[j] * s[j];
-            }
-          }
-        }
-      }
-    }
-
-    if (e0 < HD) {
-      Vec16<T> o;
-#pragma unroll
-      for (int j = 0; j < EPV; ++j) o.e[j] = from_float<T>(x[j]);
-      store16(out + e0, o);
     }
   }
 }
 
-template <typename T, int NV>
-__device__ __forceinline__ void copy_row(const T* __restrict__ in, T* __restrict__ out, int HD,
-                                         int lane) {
+template <typename T> __device__ __forceinline__ u32x4 pack_vec(const float (&x)[Vec16<T>::N]) {
+  u32x4 o;
+#pragma unroll
+  for (int j = 0; j < Vec16<T>::N / 2; ++j) Raw<T>::set2(o, j, x[2 * j], x[2 * j + 1]);
+  return o;
+}
+
+// ---- per-head (or no) statistics: one vector per lane, grid (vectors / 256, parts) ---------------
+template <typename T, typename TW, int NORM_MODE, bool GENERAL>
+__global__ __launch_bounds__(256) void qknorm_flat_kernel(
+    const T* __restrict__ q_in, const T* __restrict__ k_in, const T* __restrict__ v_in,
+    T* __restrict__ q_out, T* __restrict__ k_out, T* __restrict__ v_out,
+    const TW* __restrict__ wq, const TW* __restrict__ wk, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, int S, int HD, int D, int rot, int64_t is_b, int64_t is_s,
+    int out_seq_offset, int S_total, float eps, int vec_per_row, int64_t total_vec, bool neox,
+    bool ref_round) {
   constexpr int EPV = Vec16<T>::N;
-#pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int e0 = (i * 64 + lane) * EPV;
-    if (e0 < HD) store16(out + e0, load16(in + e0));
+  const int lane = threadIdx.x & 63;
+  // part: 0 = q, 1 = k, 2 = v (k and v may be absent)
+  const int kind = blockIdx.y == 0 ? 0 : (blockIdx.y == 1 && k_in != nullptr ? 1 : 2);
+  const int64_t i_raw = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  const bool valid = i_raw < total_vec;
+  const int64_t i = valid ? i_raw : total_vec - 1;  // clamped lanes compute, never store
+  const int64_t tok = i / vec_per_row;
+  const int e0 = static_cast<int>(i - tok * vec_per_row) * EPV;
+  const int b = static_cast<int>(tok / S);
+  const int s = static_cast<int>(tok - static_cast<int64_t>(b) * S);
+  const int64_t in_off = b * is_b + s * is_s + e0;
+  const int64_t out_off = (static_cast<int64_t>(b) * S_total + out_seq_offset + s) * HD + e0;
+  if (kind == 2) {  // block-uniform
+    const u32x4 r = load_raw(v_in + in_off);
+    if (valid) __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(v_out + out_off));
+    return;
   }
+  const u32x4 r = load_raw((kind == 0 ? q_in : k_in) + in_off);
+  float x[EPV];
+#pragma unroll
+  for (int j = 0; j < EPV; ++j) x[j] = Raw<T>::get(r, j);
+  const int d0 = e0 % D;
+  float rstd = 1.f;
+  if constexpr (NORM_MODE == ODIT_NORM_HEAD) {
+    float sq = 0.f;
+#pragma unroll
+    for (int j = 0; j < EPV; ++j) sq = fmaf(x[j], x[j], sq);
+    switch (D / EPV) {  // lanes per head row: wave-uniform
+      case 64: sq = group_sum<64>(sq); break;
+      case 32: sq = group_sum<32>(sq); break;
+      case 16: sq = group_sum<16>(sq); break;
+      case 8: sq = group_sum<8>(sq); break;
+      case 4: sq = group_sum<4>(sq); break;
+      case 2: sq = group_sum<2>(sq); break;
+      default: break;
+    }
+    rstd = rsqrtf(sq / static_cast<float>(D) + eps);
+  }
+  const TW* w = kind == 0 ? wq : wk;
+  const float* cr = cos_t ? cos_t + static_cast<int64_t>(s) * (rot >> 1) : nullptr;
+  const float* sr = sin_t ? sin_t + static_cast<int64_t>(s) * (rot >> 1) : nullptr;
+  transform_vec<T, TW, NORM_MODE != ODIT_NORM_NONE, true, GENERAL>(x, rstd, w ? w + d0 : nullptr, cr, sr, d0,
+                                                                   rot, true, lane, neox, ref_round);
+  if (valid)
+    __builtin_nontemporal_store(pack_vec<T>(x), reinterpret_cast<u32x4*>((kind == 0 ? q_out : k_out) + out_off));
 }
 
-template <typename T, typename TW, int NV, int NORM_MODE, bool GENERAL>
-__global__ __launch_bounds__(256) void qknorm_rope_kernel(
+// ---- whole-row statistics: one wavefront per (token, part), row held in registers ---------------
+template <typename T, typename TW, int NV, bool GENERAL>
+__global__ __launch_bounds__(256) void qknorm_row_kernel(
     const T* __restrict__ q_in, const T* __restrict__ k_in, const T* __restrict__ v_in,
     T* __restrict__ q_out, T* __restrict__ k_out, T* __restrict__ v_out,
     const TW* __restrict__ wq, const TW* __restrict__ wk, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, int B, int S, int HD, int D, int rot, int64_t is_b,
     int64_t is_s, int out_seq_offset, int S_total, float eps, bool neox, bool ref_round) {
+  constexpr int EPV = Vec16<T>::N;
   const int lane = threadIdx.x & 63;
+  const int kind = blockIdx.y == 0 ? 0 : (blockIdx.y == 1 && k_in != nullptr ? 1 : 2);
   const int64_t tok = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (tok >= static_cast<int64_t>(B) * S) return;
+  if (tok >= static_cast<int64_t>(B) * S) return;  // wave-uniform
   const int b = static_cast<int>(tok / S);
   const int s = static_cast<int>(tok - static_cast<int64_t>(b) * S);
-  const int64_t in_off = b * is_b + s * is_s;
-  const int64_t out_off = (static_cast<int64_t>(b) * S_total + out_seq_offset + s) * HD;
+  const T* in = (kind == 0 ? q_in : (kind == 1 ? k_in : v_in)) + b * is_b + s * is_s;
+  T* out = (kind == 0 ? q_out : (kind == 1 ? k_out : v_out)) +
+           (static_cast<int64_t>(b) * S_total + out_seq_offset + s) * HD;
+  u32x4 raw[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int e0 = (i * 64 + lane) * EPV;
+    raw[i] = e0 < HD ? load_raw(in + e0) : u32x4{0u, 0u, 0u, 0u};
+  }
+  if (kind == 2) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int e0 = (i * 64 + lane) * EPV;
+      if (e0 < HD) store_raw(out + e0, raw[i]);
+    }
+    return;
+  }
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+#pragma unroll
+    for (int j = 0; j < EPV; ++j) { const float t = Raw<T>::get(raw[i], j); sq = fmaf(t, t, sq); }
+  const float rstd = rsqrtf(wave_sum(sq) / static_cast<float>(HD) + eps);
+  const TW* w = kind == 0 ? wq : wk;
   const float* cr = cos_t ? cos_t + static_cast<int64_t>(s) * (rot >> 1) : nullptr;
   const float* sr = sin_t ? sin_t + static_cast<int64_t>(s) * (rot >> 1) : nullptr;
-  norm_rope_row<T, TW, NV, NORM_MODE, GENERAL>(q_in + in_off, q_out + out_off, wq, cr, sr, HD, D,
-                                                rot, eps, lane, neox, ref_round);
-  if (k_in != nullptr)
-    norm_rope_row<T, TW, NV, NORM_MODE, GENERAL>(k_in + in_off, k_out + out_off, wk, cr, sr, HD, D,
-                                                  rot, eps, lane, neox, ref_round);
-  if (v_in != nullptr) copy_row<T, NV>(v_in + in_off, v_out + out_off, HD, lane);
-}
-
-template <typename T, typename TW, int NORM_MODE, bool GENERAL>
-static int launch_qknorm_nv(bool neox, bool ref_round, int nv, dim3 grid, hipStream_t stream, const void* q_in,
-                            const void* k_in, const void* v_in, void* q_out, void* k_out,
-                            void* v_out, const void* wq, const void* wk, const float* cos_t,
-                            const float* sin_t, int B, int S, int HD, int D, int rot, int64_t is_b,
-                            int64_t is_s, int out_seq_offset, int S_total, float eps) {
-#define ODIT_QK_CASE(NVV)                                                                         \
-  hipLaunchKernelGGL((qknorm_rope_kernel<T, TW, NVV, NORM_MODE, GENERAL>), grid, dim3(256),        \
-                     0, stream, static_cast<const T*>(q_in), static_cast<const T*>(k_in),         \
-                     static_cast<const T*>(v_in), static_cast<T*>(q_out), static_cast<T*>(k_out), \
-                     static_cast<T*>(v_out), static_cast<const TW*>(wq),                          \
-                     static_cast<const TW*>(wk), cos_t, sin_t, B, S, HD, D, rot, is_b, is_s,      \
-                     out_seq_offset, S_total, eps, neox, ref_round)
-  if (nv <= 2) ODIT_QK_CASE(2);
-  else if (nv <= 6) ODIT_QK_CASE(6);
-  else if (nv <= 10) ODIT_QK_CASE(10);
-  else ODIT_QK_CASE(16);
-#undef ODIT_QK_CASE
-  return check_launch("odit_qknorm_rope");
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int e0 = (i * 64 + lane) * EPV;
+    const bool valid = e0 < HD;
+    float x[EPV];
+#pragma unroll
+    for (int j = 0; j < EPV; ++j) x[j] = Raw<T>::get(raw[i], j);
+    transform_vec<T, TW, true, false, GENERAL>(x, rstd, w ? w + e0 : nullptr, cr, sr, e0 % D, rot, valid, lane,
+                                               neox, ref_round);
+    if (valid) store_raw(out + e0, pack_vec<T>(x));
+  }
 }
 
 }  // namespace odit
@@ -255,23 +259,50 @@ int qknorm_rope_bf16(const QkArgs& a);
 int qknorm_rope_f16(const QkArgs& a);
 int qknorm_rope_f32(const QkArgs& a);
 
-template <typename T, typename TW> static int qk_go(const QkArgs& a) {
+template <typename T, typename TW, int NORM_MODE, bool GENERAL> static int qk_flat(const QkArgs& a) {
+  constexpr int EPV = Vec16<T>::N;
+  const int vpr = a.HD / EPV;
+  const int64_t total = static_cast<int64_t>(a.B) * a.S * vpr;
+  const int nparts = 1 + (a.k_in != nullptr) + (a.v_in != nullptr);
+  const dim3 grid(static_cast<unsigned>((total + 255) / 256), nparts);
+  hipLaunchKernelGGL((qknorm_flat_kernel<T, TW, NORM_MODE, GENERAL>), grid, dim3(256), 0, a.stream,
+                     static_cast<const T*>(a.q_in), static_cast<const T*>(a.k_in),
+                     static_cast<const T*>(a.v_in), static_cast<T*>(a.q_out), static_cast<T*>(a.k_out),
+                     static_cast<T*>(a.v_out), static_cast<const TW*>(a.wq), static_cast<const TW*>(a.wk),
+                     a.cos, a.sin, a.S, a.HD, a.D, a.rot, a.is_b, a.is_s, a.out_seq_offset, a.S_total,
+                     a.eps, vpr, total, a.neox, a.ref_round);
+  return check_launch("odit_qknorm_rope");
+}
+
+template <typename T, typename TW, int NV, bool GENERAL> static int qk_row(const QkArgs& a) {
   const int64_t toks = static_cast<int64_t>(a.B) * a.S;
-  const dim3 grid(static_cast<unsigned>((toks + 3) / 4));
-#define ODIT_QK_ARGS                                                                             \
-  a.neox, a.ref_round, a.nv, grid, a.stream, a.q_in, a.k_in, a.v_in, a.q_out, a.k_out, a.v_out,  \
-      a.wq, a.wk, a.cos, a.sin, a.B, a.S, a.HD, a.D, a.rot, a.is_b, a.is_s, a.out_seq_offset,    \
-      a.S_total, a.eps
-#define ODIT_QK_MODE(MODE)                                                             \
-  return (a.neox || a.ref_round) ? launch_qknorm_nv<T, TW, MODE, true>(ODIT_QK_ARGS)   \
-                                 : launch_qknorm_nv<T, TW, MODE, false>(ODIT_QK_ARGS);
+  const int nparts = 1 + (a.k_in != nullptr) + (a.v_in != nullptr);
+  const dim3 grid(static_cast<unsigned>((toks + 3) / 4), nparts);
+  hipLaunchKernelGGL((qknorm_row_kernel<T, TW, NV, GENERAL>), grid, dim3(256), 0, a.stream,
+                     static_cast<const T*>(a.q_in), static_cast<const T*>(a.k_in),
+                     static_cast<const T*>(a.v_in), static_cast<T*>(a.q_out), static_cast<T*>(a.k_out),
+                     static_cast<T*>(a.v_out), static_cast<const TW*>(a.wq), static_cast<const TW*>(a.wk),
+                     a.cos, a.sin, a.B, a.S, a.HD, a.D, a.rot, a.is_b, a.is_s, a.out_seq_offset,
+                     a.S_total, a.eps, a.neox, a.ref_round);
+  return check_launch("odit_qknorm_rope");
+}
+
+template <typename T, typename TW> static int qk_go(const QkArgs& a) {
+  const bool general = a.neox || a.ref_round;
   switch (a.norm_mode) {
-    case ODIT_NORM_NONE: ODIT_QK_MODE(ODIT_NORM_NONE)
-    case ODIT_NORM_HEAD: ODIT_QK_MODE(ODIT_NORM_HEAD)
-    default: ODIT_QK_MODE(ODIT_NORM_ROW)
+    case ODIT_NORM_NONE:
+      return general ? qk_flat<T, TW, ODIT_NORM_NONE, true>(a) : qk_flat<T, TW, ODIT_NORM_NONE, false>(a);
+    case ODIT_NORM_HEAD:
+      return general ? qk_flat<T, TW, ODIT_NORM_HEAD, true>(a) : qk_flat<T, TW, ODIT_NORM_HEAD, false>(a);
+    default:
+      break;
   }
-#undef ODIT_QK_MODE
-#undef ODIT_QK_ARGS
+#define ODIT_QK_ROW(NVV) return general ? qk_row<T, TW, NVV, true>(a) : qk_row<T, TW, NVV, false>(a)
+  if (a.nv <= 2) ODIT_QK_ROW(2);
+  else if (a.nv <= 6) ODIT_QK_ROW(6);
+  else if (a.nv <= 10) ODIT_QK_ROW(10);
+  else ODIT_QK_ROW(16);
+#undef ODIT_QK_ROW
 }
 
 #if ODIT_QK_TU == 0
@@ -331,7 +362,7 @@ extern "C" int odit_qknorm_rope(const void* q_in, const void* k_in, const void* 
                  "odit_qknorm_rope: pointers must be 16-byte aligned");
   const int64_t HD = static_cast<int64_t>(H) * D;
   const int nv = static_cast<int>((HD + 64 * epv - 1) / (64 * epv));
-  if (nv > 16) {
+  if (nv > 16 && norm_mode == ODIT_NORM_ROW) {
     set_error("odit_qknorm_rope: H*D=%lld exceeds the %d elements one wavefront keeps in registers",
               static_cast<long long>(HD), 16 * 64 * epv);
     return ODIT_ENOTSUP;

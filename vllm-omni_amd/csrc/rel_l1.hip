@@ -1,13 +1,13 @@
 // K5: TeaCache relative-L1 reduction. One streaming read of `cur` and `prev`
 // (algorithmic traffic 2 * B*n * sizeof(T)), per-batch-row sums, fixed reduction tree:
 //   stage 1  grid (nblk, B): every block reduces one contiguous slice of one row to two fp32 partials
-//   stage 2  grid (B): one wavefront adds the row's partials in fp64 and writes sums[b] = {sum|cur-prev|, sum|prev|}
+//   stage 2  grid (B): one workgroup adds the row's partials in fp64 and writes sums[b] = {sum|cur-prev|, sum|prev|}
 // The tree depends only on (B, n), never on timing, so repeated calls give bit-identical sums.
 #include "odit_common.h"
 
 namespace odit {
 
-constexpr int kRelL1MaxBlocksPerRow = 1024;
+constexpr int kRelL1MaxBlocksPerRow = 2048;
 constexpr int kRelL1VecsPerThread = 4;
 
 static inline int rel_l1_blocks_per_row(int64_t n) {
@@ -35,9 +35,7 @@ __global__ __launch_bounds__(256) void rel_l1_stage1_kernel(const T* __restrict_
   const int64_t v_begin = static_cast<int64_t>(blockIdx.x) * per_blk;
   const int64_t v_end = v_begin + per_blk < n_vec ? v_begin + per_blk : n_vec;
   float sd = 0.f, sp = 0.f;
-  for (int64_t i = v_begin + threadIdx.x; i < v_end; i += blockDim.x) {
-    const Vec16<T> cv = load16(c + i * EPV);
-    const Vec16<T> pv = load16(p + i * EPV);
+  auto accumulate = [&](const Vec16<T>& cv, const Vec16<T>& pv) {
 #pragma unroll
     for (int j = 0; j < EPV; ++j) {
       const float pf = to_float(pv.e[j]);
@@ -46,7 +44,21 @@ __global__ __launch_bounds__(256) void rel_l1_stage1_kernel(const T* __restrict_
       sd += fabsf(d);
       sp += fabsf(pf);
     }
+  };
+  // four vector pairs (eight 16-byte loads) in flight per lane before the first use
+  constexpr int U = 4;
+  int64_t i = v_begin + threadIdx.x;
+  for (; i + (U - 1) * 256 < v_end; i += U * 256) {
+    Vec16<T> cv[U], pv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      cv[u] = load16(c + (i + u * 256) * EPV);
+      pv[u] = load16(p + (i + u * 256) * EPV);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) accumulate(cv[u], pv[u]);
   }
+  for (; i < v_end; i += 256) accumulate(load16(c + i * EPV), load16(p + i * EPV));
   if (blockIdx.x == 0) {  // scalar tail (also the whole row when vector loads are not possible)
     for (int64_t i = n_vec * EPV + threadIdx.x; i < n; i += blockDim.x) {
       const float pf = to_float(p[i]);
@@ -69,18 +81,29 @@ __global__ __launch_bounds__(256) void rel_l1_stage1_kernel(const T* __restrict_
   }
 }
 
-__global__ __launch_bounds__(64) void rel_l1_stage2_kernel(const float* __restrict__ partials,
-                                                           double* __restrict__ sums, int nblk) {
+__global__ __launch_bounds__(256) void rel_l1_stage2_kernel(const float* __restrict__ partials,
+                                                            double* __restrict__ sums, int nblk) {
   const int b = blockIdx.x;
-  const float* p = partials + static_cast<int64_t>(b) * nblk * 2;
+  const float2* p = reinterpret_cast<const float2*>(partials) + static_cast<int64_t>(b) * nblk;
+  // all loads of a thread are independent; fixed assignment partial i -> thread i % 256
   double sd = 0.0, sp = 0.0;
-  for (int i = threadIdx.x; i < nblk; i += 64) { sd += p[2 * i]; sp += p[2 * i + 1]; }
+  for (int i = threadIdx.x; i < nblk; i += 256) {
+    const float2 v = p[i];
+    sd += v.x;
+    sp += v.y;
+  }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     sd += __shfl_xor(sd, off, 64);
     sp += __shfl_xor(sp, off, 64);
   }
-  if (threadIdx.x == 0) { sums[2 * b] = sd; sums[2 * b + 1] = sp; }
+  __shared__ double red[2][4];
+  if ((threadIdx.x & 63) == 0) { red[0][threadIdx.x >> 6] = sd; red[1][threadIdx.x >> 6] = sp; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    sums[2 * b] = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
+    sums[2 * b + 1] = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+  }
 }
 
 template <typename T>
@@ -104,7 +127,7 @@ static int launch_rel_l1(const void* cur, const void* prev, double* sums, float*
   }
   int rc = check_launch("odit_rel_l1 (stage 1)");
   if (rc != ODIT_OK) return rc;
-  hipLaunchKernelGGL(rel_l1_stage2_kernel, dim3(B), dim3(64), 0, stream, partials, sums, nblk);
+  hipLaunchKernelGGL(rel_l1_stage2_kernel, dim3(B), dim3(256), 0, stream, partials, sums, nblk);
   return check_launch("odit_rel_l1 (stage 2)");
 }
 
