@@ -226,6 +226,9 @@ def main():
     _lib.load()
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
+    from vllm_omni_amd import gemm_tuning
+
+    tuned = gemm_tuning.enable()  # hipBLASLt solution ids picked offline for this model's GEMM shapes
     torch.cuda.set_device(0)
     dev = torch.device("cuda:0")
     model = build_model(torch, args.blocks)
@@ -277,7 +280,7 @@ def main():
         "config": {"workload": f"Qwen-Image-shape MMDiT denoise step: {args.blocks} dual-stream blocks, hidden {C}, "
                                f"{HEADS} heads x {HEAD_DIM}, MLP {MLP_RATIO * C}, {S_IMG} image + {S_TXT} text tokens, "
                                "CFG batch 2, random weights N(0,0.02)",
-                   "valid": args.blocks == LAYERS},
+                   "valid": args.blocks == LAYERS, "gemm": "hipBLASLt via torch" + (" (tuned solution table)" if tuned else "")},
         "roofline": {"kernel": "attn_fwd_kernel (joint attention, B=2, 24x128, S=4352)", "bound": "mfma",
                      "achieved": attn_tflops, "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": attn_tflops / PEAK_MFMA_BF16_TFLOPS, "traffic": None,
