@@ -297,7 +297,7 @@ ATTN_SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("variant", ["14", "18", "24", "28", "29"])
+@pytest.mark.parametrize("variant", ["14", "18", "24", "28", "29", "38", "34"])
 @pytest.mark.parametrize("shape", ATTN_SHAPES)
 def test_attention_parity(gpu, monkeypatch, variant, shape):
     from vllm_omni_amd import kernels
@@ -332,7 +332,7 @@ def test_attention_fp16_and_strided_views(gpu):
     _close(got, want, atol=3e-3, rtol=3e-3, what="fp16 strided attention")
 
 
-@pytest.mark.parametrize("variant", ["18", "24", "28"])
+@pytest.mark.parametrize("variant", ["18", "24", "28", "38", "34"])
 def test_attention_key_mask_equals_deleting_keys(gpu, monkeypatch, variant):
     """The reference's padding-equivalence property (test_flash_attn.py:60-147)."""
     from vllm_omni_amd import kernels

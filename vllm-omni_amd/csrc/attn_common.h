@@ -1,0 +1,63 @@
+// Types shared by the attention kernels: MFMA wrappers, launch parameters, workgroup-id remap.
+#pragma once
+
+#include "odit_common.h"
+
+namespace odit {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_v;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_v;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_v;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2_v;
+typedef uint32_t u32x4_v __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_v __attribute__((ext_vector_type(2)));
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_v;
+typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_v;
+
+template <typename T> struct Mma;
+template <> struct Mma<bf16_t> {
+  using frag = bf16x8_v;
+  static __device__ __forceinline__ f32x16_v run(frag a, frag b, f32x16_v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    const f32x2_v f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_v));  // v_cvt_pk_bf16_f32
+  }
+};
+template <> struct Mma<f16_t> {
+  using frag = f16x8_v;
+  static __device__ __forceinline__ f32x16_v run(frag a, frag b, f32x16_v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    const f32x2_v f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2_v));
+  }
+};
+
+struct AttnParams {
+  const void* q; const void* k; const void* v; void* o;
+  const uint8_t* mask; float* lse;
+  int B, Sq, Sk, H, Hkv;
+  int64_t qs_b, qs_s, qs_h, ks_b, ks_s, ks_h, vs_b, vs_s, vs_h, os_b, os_s, os_h;
+  float scale, scale_log2;
+  int n_qblocks, total_blocks;
+};
+
+constexpr int kNumXcd = 8;
+
+// Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; give every XCD a contiguous
+// range of logical ids instead, so neighbours in (q-block, head) order share an L2.
+__device__ __forceinline__ int xcd_remap(int bid, int total) {
+  const int xcd = bid % kNumXcd, local = bid / kNumXcd;
+  const int per = total / kNumXcd, rem = total % kNumXcd;
+  return xcd * per + (xcd < rem ? xcd : rem) + local;
+}
+
+
+// software-pipelined kernel with direct global->LDS tile loads (attn_fwd_dma.hip); returns
+// ODIT_ENOTSUP when the tensors cannot be addressed with 32-bit buffer offsets
+int launch_attn_dma(AttnParams& p, int dtype, int D, int nw, hipStream_t stream);
+
+}  // namespace odit

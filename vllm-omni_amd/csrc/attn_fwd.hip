@@ -15,59 +15,9 @@
 // that the q-blocks of one (batch, head) — which share K/V — land on the same XCD and hit its L2.
 //
 // Algorithmic work: 4 * B * H * Sq * Sk * D flop; minimum traffic 2 * (2*B*Sq*H*D + 2*B*Sk*Hkv*D) bytes.
-#include "odit_common.h"
+#include "attn_common.h"
 
 namespace odit {
-
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_v;
-typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_v;
-typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_v;
-typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2_v;
-typedef uint32_t u32x4_v __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2_v __attribute__((ext_vector_type(2)));
-typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_v;
-typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_v;
-
-template <typename T> struct Mma;
-template <> struct Mma<bf16_t> {
-  using frag = bf16x8_v;
-  static __device__ __forceinline__ f32x16_v run(frag a, frag b, f32x16_v c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    const f32x2_v f = {lo, hi};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_v));  // v_cvt_pk_bf16_f32
-  }
-};
-template <> struct Mma<f16_t> {
-  using frag = f16x8_v;
-  static __device__ __forceinline__ f32x16_v run(frag a, frag b, f32x16_v c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    const f32x2_v f = {lo, hi};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2_v));
-  }
-};
-
-struct AttnParams {
-  const void* q; const void* k; const void* v; void* o;
-  const uint8_t* mask; float* lse;
-  int B, Sq, Sk, H, Hkv;
-  int64_t qs_b, qs_s, qs_h, ks_b, ks_s, ks_h, vs_b, vs_s, vs_h, os_b, os_s, os_h;
-  float scale, scale_log2;
-  int n_qblocks, total_blocks;
-};
-
-constexpr int kNumXcd = 8;
-
-// Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; give every XCD a contiguous
-// range of logical ids instead, so neighbours in (q-block, head) order share an L2.
-__device__ __forceinline__ int xcd_remap(int bid, int total) {
-  const int xcd = bid % kNumXcd, local = bid / kNumXcd;
-  const int per = total / kNumXcd, rem = total % kNumXcd;
-  return xcd * per + (xcd < rem ? xcd : rem) + local;
-}
 
 template <typename T, int D, int QT, int NW>
 __global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(const AttnParams p) {
@@ -705,9 +655,14 @@ extern "C" int odit_attn_fwd(const void* q, const void* k, const void* v, void* 
   p.scale = scale;
   p.scale_log2 = scale * 1.4426950408889634f;
 
-  int variant = 28;
+  int variant = 34;
   if (const char* e = getenv("ODIT_ATTN_VARIANT")) variant = atoi(e);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (variant == 38 || variant == 34) {
+    const int rc = launch_attn_dma(p, dtype, D, variant == 38 ? 8 : 4, st);
+    if (rc != ODIT_ENOTSUP) return rc;
+    variant = 28;  // tensors too large for 32-bit buffer offsets: pointer-addressed kernel
+  }
   if (dtype == ODIT_BF16) {
     return D == 128 ? dispatch_attn<bf16_t, 128>(p, variant, st)
                     : dispatch_attn<bf16_t, 64>(p, variant, st);

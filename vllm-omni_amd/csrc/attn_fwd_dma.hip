@@ -1,0 +1,342 @@
+// K1, production variant: software-pipelined flash attention whose K/V tiles go from global memory
+// straight into LDS (buffer_load ... lds), with no staging registers, no LDS store instructions and
+// no per-tile address arithmetic.
+//
+// Tile movement. A tile is 64 keys x D elements, row-major, unpadded (256 B rows for D = 128). One
+// `buffer_load_dwordx4 ... lds` of a wavefront fills 1 KB of LDS: lane l's 16 bytes land at
+// base + 16*l (measured), so the PLACE is fixed and the lane picks WHAT it fetches. Lane l therefore
+// fetches, for tile row r = 4*i + l/16 and physical 16-byte chunk pc = l%16, the logical chunk
+// pc ^ f(r): the swizzle lives in the global address. Per-lane byte offsets are computed once; the
+// tile index only moves a scalar offset. The buffer descriptor's size is the end of the last valid
+// key row, so rows past Sk read as zeros without any clamping.
+//   K:  f(r) = r % 16       a quarter-wave (16 key rows, one chunk column) of a ds_read_b128 covers
+//                           all 64 banks
+//   V:  f(r) = 4 * (r % 4)  the 4 keys x 4 eight-byte words of two ds_read_b64_tr_b16 groups cover
+//                           all 64 banks
+// Fragment addresses then are (per-lane base) XOR (a compile-time constant) plus an immediate.
+//
+// Everything else (transposed S^T = K Q^T / O^T = V^T P^T formulation, one query per lane, lazy
+// rescale, stage A = next-tile QK^T MFMAs interleaved with this tile's exp2 work, stage B = PV, one
+// barrier per tile, XCD-aware workgroup order) is as in attn_fwd_pipe_kernel.
+#include "attn_common.h"
+
+namespace odit {
+
+typedef short s16x4_d __attribute__((ext_vector_type(4)));
+typedef short s16x8_d __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4_d* lds_s16x4_p;
+typedef __attribute__((address_space(3))) void* lds_void_p;
+
+template <typename T, int D, int NW>
+__global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const AttnParams p) {
+  using M = Mma<T>;
+  using frag = typename M::frag;
+  constexpr int BN = 64;
+  constexpr int KS = D / 16;
+  constexpr int DT = D / 32;
+  constexpr int ROWB = D * 2;                 // bytes per tile row
+  constexpr int CPR = ROWB / 16;              // 16-byte chunks per row (16 for D=128, 8 for D=64)
+  constexpr int RPI = 64 / CPR;               // tile rows filled by one wave instruction (4 or 8)
+  constexpr int TILEB = BN * ROWB;            // bytes per tile
+  constexpr int NINST = BN / RPI;             // wave instructions per tile (16 or 8)
+  constexpr int IPW = (NINST + NW - 1) / NW;  // ... per wavefront
+  static_assert(NINST % NW == 0, "tile loads must divide evenly over the wavefronts");
+  constexpr int BM = NW * 32;
+
+  __shared__ __attribute__((aligned(1024))) char lds[4 * TILEB];  // K0 K1 V0 V1
+  char* const Kb = lds;
+  char* const Vb = lds + 2 * TILEB;
+
+  const int pid = xcd_remap(blockIdx.x, p.total_blocks);
+  const int qb = pid % p.n_qblocks;
+  const int bh = pid / p.n_qblocks;
+  const int h = bh % p.H;
+  const int b = bh / p.H;
+  const int hkv = h / (p.H / p.Hkv);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hh = lane >> 5;
+  const int q0 = qb * BM + wave * 32;
+
+  const T* qbase = static_cast<const T*>(p.q) + b * p.qs_b + h * p.qs_h;
+  const T* kbase = static_cast<const T*>(p.k) + b * p.ks_b + hkv * p.ks_h;
+  const T* vbase = static_cast<const T*>(p.v) + b * p.vs_b + hkv * p.vs_h;
+
+  // buffer descriptors end right after the last valid key row: later rows read as zeros
+  const uint32_t k_bytes = static_cast<uint32_t>(((p.Sk - 1) * p.ks_s + D) * 2);
+  const uint32_t v_bytes = static_cast<uint32_t>(((p.Sk - 1) * p.vs_s + D) * 2);
+  const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(kbase), 0, k_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(vbase), 0, v_bytes, 0x00020000);
+
+  // per-lane global byte offsets of the chunks this lane moves, relative to the tile's first row
+  uint32_t kvoff[IPW], vvoff[IPW];
+#pragma unroll
+  for (int i = 0; i < IPW; ++i) {
+    const int r = (wave * IPW + i) * RPI + lane / CPR;  // tile row
+    const int pc = lane % CPR;
+    kvoff[i] = static_cast<uint32_t>(r * p.ks_s * 2) + static_cast<uint32_t>(((pc ^ (r % 16)) % CPR) * 16);
+    vvoff[i] = static_cast<uint32_t>(r * p.vs_s * 2) + static_cast<uint32_t>(((pc ^ (4 * (r % 4))) % CPR) * 16);
+  }
+  const uint32_t k_tile_step = static_cast<uint32_t>(BN * p.ks_s * 2);
+  const uint32_t v_tile_step = static_cast<uint32_t>(BN * p.vs_s * 2);
+
+  auto dma_tile = [&](const __amdgpu_buffer_rsrc_t& rsrc, const uint32_t(&voff)[IPW], uint32_t soff, char* dst) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass cannot parse this builtin and would drop the kernel stub
+#pragma unroll
+    for (int i = 0; i < IPW; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_p)(dst + (wave * IPW + i) * 1024), 16, voff[i],
+                                               soff, 0, 0);
+#endif
+  };
+
+  // ---- Q fragments stay in registers ----
+  frag qf[KS];
+  {
+    int row = q0 + l32;
+    row = row < p.Sq ? row : p.Sq - 1;
+    const T* qp = qbase + row * p.qs_s + hh * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      qf[ks] = __builtin_bit_cast(frag, *reinterpret_cast<const u32x4_v*>(qp + ks * 16));
+  }
+
+  f32x16_v o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o[dt][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  const int n_tiles = (p.Sk + BN - 1) / BN;
+  const float c = p.scale_log2;
+  const uint8_t* mrow = p.mask ? p.mask + static_cast<int64_t>(b) * p.Sk : nullptr;
+
+  // K fragment (kt, ks): row kt*32 + l32, logical chunk 2*ks + hh  ->  chunk (2*ks) ^ (hh ^ l32 % 16)
+  const int k_lane = l32 * ROWB + ((((hh ^ (l32 % 16)) % CPR)) << 4);
+  // V transpose read, 16-lane group g = lane/16 (d half dh = g&1, key half = hh), lane s = lane%16:
+  // key 4*hh + s/4 (+ tile offsets), logical chunk 4*dt + 2*dh + (s%4)/2, 8-byte half (s%4)%2,
+  // physical chunk = logical ^ 4*(s/4)  ->  XOR of the dt field only
+  const int sq = (lane & 15) >> 2;
+  const int dh = (lane >> 4) & 1;
+  const int v_lane = (4 * hh + sq) * ROWB + ((((4 * sq) % CPR) ^ (2 * dh + ((lane & 3) >> 1))) << 4) + ((lane & 1) << 3);
+
+  auto qk_plain = [&](const char* kt_base, f32x16_v(&s)[2]) {
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s[kt][e] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+        const frag a = __builtin_bit_cast(
+            frag, *reinterpret_cast<const u32x4_v*>(kt_base + kt * 32 * ROWB + (k_lane ^ (ks * 32))));
+        s[kt] = M::run(a, qf[ks], s[kt]);
+      }
+  };
+
+  auto mask_and_max = [&](int j, f32x16_v(&s)[2]) -> float {
+    // branch-free selects: every lane rewrites all its scores, excluded ones with -inf
+    if (mrow != nullptr) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const int key = j * BN + kt * 32 + g * 8 + hh * 4 + t;
+            const int kc = key < p.Sk ? key : p.Sk - 1;
+            const bool live = (key < p.Sk) & (mrow[kc] != 0);
+            const float x = s[kt][g * 4 + t];
+            s[kt][g * 4 + t] = live ? x : -INFINITY;
+          }
+    } else if ((j + 1) * BN > p.Sk) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const int key = j * BN + kt * 32 + g * 8 + hh * 4 + t;
+            const float x = s[kt][g * 4 + t];
+            s[kt][g * 4 + t] = key < p.Sk ? x : -INFINITY;
+          }
+    }
+    float mx = s[0][0];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[kt][e]);
+    return mx;
+  };
+
+  auto settle_max = [&](float mx) {
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx);
+    if (__any((m_new - m_run) * c > 8.f)) {
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * c);
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[dt][e] *= alpha;
+      m_run = m_new;
+    }
+  };
+
+  auto tile = [&](int j, f32x16_v(&s_cur)[2], f32x16_v(&s_next)[2]) {
+    const int buf = j & 1;
+    const bool has_next = j + 1 < n_tiles;
+    // buffers K[buf] (held K(j), consumed last tile) and V[buf^1] (held V(j-1)) are free now
+    if (j + 2 < n_tiles) dma_tile(krsrc, kvoff, static_cast<uint32_t>(j + 2) * k_tile_step, Kb + buf * TILEB);
+    if (has_next) dma_tile(vrsrc, vvoff, static_cast<uint32_t>(j + 1) * v_tile_step, Vb + (buf ^ 1) * TILEB);
+
+    const float mc = (m_run == -INFINITY) ? 0.f : m_run * c;
+    uint32_t pf[2][2][4];
+    float psum = 0.f;
+    // ---- stage A ----
+    if (has_next) {
+      const char* kt_base = Kb + (buf ^ 1) * TILEB;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s_next[kt][e] = 0.f;
+      constexpr int KPF = 3;  // K fragments in flight ahead of the MFMA that consumes them
+      u32x4_v kfr[KPF + 1];
+      auto k_fetch = [&](int i) {
+        const int ks = i >> 1, kt = i & 1;
+        kfr[i % (KPF + 1)] = *reinterpret_cast<const u32x4_v*>(kt_base + kt * 32 * ROWB + (k_lane ^ (ks * 32)));
+      };
+#pragma unroll
+      for (int i = 0; i < KPF; ++i) k_fetch(i);
+#pragma unroll
+      for (int i = 0; i < 2 * KS; ++i) {
+        if (i + KPF < 2 * KS) k_fetch(i + KPF);
+        const int ks = i >> 1, kt = i & 1;
+        s_next[kt] = M::run(__builtin_bit_cast(frag, kfr[i % (KPF + 1)]), qf[ks], s_next[kt]);
+        constexpr int PAIRS = 16 / (2 * KS) > 0 ? 16 / (2 * KS) : 1;
+#pragma unroll
+        for (int q = 0; q < PAIRS; ++q) {
+          const int pi = i * PAIRS + q;
+          if (pi < 16) {
+            const int pkt = pi >> 3, e0 = (pi & 7) * 2;
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(s_cur[pkt][e0], c, -mc));
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(s_cur[pkt][e0 + 1], c, -mc));
+            psum += p0 + p1;
+            pf[pkt][(pi & 7) >> 2][pi & 3] = M::pack2(p0, p1);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);  // pin: fetch(i+KPF), MFMA(i), this step's exp2 work
+      }
+    } else {
+#pragma unroll
+      for (int pi = 0; pi < 16; ++pi) {
+        const int pkt = pi >> 3, e0 = (pi & 7) * 2;
+        const float p0 = __builtin_amdgcn_exp2f(fmaf(s_cur[pkt][e0], c, -mc));
+        const float p1 = __builtin_amdgcn_exp2f(fmaf(s_cur[pkt][e0 + 1], c, -mc));
+        psum += p0 + p1;
+        pf[pkt][(pi & 7) >> 2][pi & 3] = M::pack2(p0, p1);
+      }
+    }
+    l_run += psum;
+
+    // ---- stage B: O^T += V(j)^T P(j)^T ----
+    // 4*DT steps (dt, kt, g2); the two transpose reads of step n + PF are issued before the MFMA of
+    // step n, so LDS latency is covered by PF matrix instructions
+    const char* vt_base = Vb + buf * TILEB;
+    constexpr int NSTEP = 4 * DT;
+    constexpr int PF = 3;
+    s16x4_d vlo[PF + 1], vhi[PF + 1];
+    auto v_fetch = [&](int step) {
+      const int dt = step >> 2, kt = (step >> 1) & 1, g2 = step & 1;
+      const char* vp = vt_base + (kt * 32 + g2 * 16) * ROWB + (v_lane ^ ((dt * 64) % ROWB));
+      vlo[step % (PF + 1)] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_p)(vp));
+      vhi[step % (PF + 1)] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_p)(vp + 8 * ROWB));
+    };
+#pragma unroll
+    for (int st = 0; st < PF; ++st) v_fetch(st);
+#pragma unroll
+    for (int st = 0; st < NSTEP; ++st) {
+      if (st + PF < NSTEP) v_fetch(st + PF);
+      const int dt = st >> 2, kt = (st >> 1) & 1, g2 = st & 1;
+      const s16x8_d av = __builtin_shufflevector(vlo[st % (PF + 1)], vhi[st % (PF + 1)], 0, 1, 2, 3, 4, 5, 6, 7);
+      u32x4_v pb;
+      pb.x = pf[kt][g2][0]; pb.y = pf[kt][g2][1]; pb.z = pf[kt][g2][2]; pb.w = pf[kt][g2][3];
+      o[dt] = M::run(__builtin_bit_cast(frag, av), __builtin_bit_cast(frag, pb), o[dt]);
+      __builtin_amdgcn_sched_barrier(0);  // keep the reads of step st+PF ahead of this MFMA
+    }
+
+    float mx = -INFINITY;
+    if (has_next) mx = mask_and_max(j + 1, s_next);
+    __builtin_amdgcn_s_waitcnt(0);  // this wave's tile loads have landed in LDS
+    __syncthreads();
+    if (has_next) settle_max(mx);
+  };
+
+  // ---- prologue ----
+  dma_tile(krsrc, kvoff, 0, Kb);
+  dma_tile(vrsrc, vvoff, 0, Vb);
+  if (n_tiles > 1) dma_tile(krsrc, kvoff, k_tile_step, Kb + TILEB);
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  f32x16_v sa[2], sb[2];
+  qk_plain(Kb, sa);
+  settle_max(mask_and_max(0, sa));
+
+  for (int j = 0; j < n_tiles; j += 2) {
+    tile(j, sa, sb);
+    if (j + 1 < n_tiles) tile(j + 1, sb, sa);
+  }
+
+  // ---- epilogue ----
+  T* obase = static_cast<T*>(p.o) + b * p.os_b + h * p.os_h;
+  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  const int row = q0 + l32;
+  if (row < p.Sq) {
+    T* op = obase + row * p.os_s;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2_v w;
+        w.x = M::pack2(o[dt][g * 4 + 0] * inv, o[dt][g * 4 + 1] * inv);
+        w.y = M::pack2(o[dt][g * 4 + 2] * inv, o[dt][g * 4 + 3] * inv);
+        *reinterpret_cast<u32x2_v*>(op + dt * 32 + g * 8 + hh * 4) = w;
+      }
+    if (p.lse != nullptr && hh == 0) {
+      const float lse = l_tot > 0.f ? m_run * p.scale + __logf(l_tot) : -INFINITY;
+      p.lse[(static_cast<int64_t>(b) * p.H + h) * p.Sq + row] = lse;
+    }
+  }
+}
+
+template <typename T, int D, int NW>
+static int launch_dma(AttnParams& p, hipStream_t stream) {
+  constexpr int BM = NW * 32;
+  p.n_qblocks = (p.Sq + BM - 1) / BM;
+  const int64_t total = static_cast<int64_t>(p.n_qblocks) * p.H * p.B;
+  if (total > 0x7fffffffll) {
+    set_error("odit_attn_fwd: grid of %lld workgroups is too large", static_cast<long long>(total));
+    return ODIT_EINVAL;
+  }
+  p.total_blocks = static_cast<int>(total);
+  hipLaunchKernelGGL((attn_fwd_dma_kernel<T, D, NW>), dim3(p.total_blocks), dim3(NW * 64), 0, stream, p);
+  return check_launch("odit_attn_fwd");
+}
+
+int launch_attn_dma(AttnParams& p, int dtype, int D, int nw, hipStream_t stream) {
+  // 32-bit buffer offsets: the whole key range of one (batch, head) must be addressable
+  const int64_t k_span = (static_cast<int64_t>(p.Sk) + 64) * p.ks_s * 2;
+  const int64_t v_span = (static_cast<int64_t>(p.Sk) + 64) * p.vs_s * 2;
+  if (k_span >= (1ll << 31) || v_span >= (1ll << 31) || p.ks_s < 0 || p.vs_s < 0) return ODIT_ENOTSUP;
+#define ODIT_DMA_GO(T)                                                                     \
+  if (D == 128) return nw == 8 ? launch_dma<T, 128, 8>(p, stream) : launch_dma<T, 128, 4>(p, stream); \
+  return nw == 8 ? launch_dma<T, 64, 8>(p, stream) : launch_dma<T, 64, 4>(p, stream);
+  if (dtype == ODIT_BF16) { ODIT_DMA_GO(bf16_t) }
+  ODIT_DMA_GO(f16_t)
+#undef ODIT_DMA_GO
+}
+
+}  // namespace odit

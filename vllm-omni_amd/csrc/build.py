@@ -21,7 +21,7 @@ PKG = CSRC.parent
 LIB_NAME = "libomni_dit_hip.so"
 LIB_PATH = PKG / LIB_NAME
 OBJ_DIR = CSRC / "build"
-HEADERS = [CSRC / "odit_common.h", PKG.parent / "include" / "omni_dit.h"]
+HEADERS = [CSRC / "odit_common.h", CSRC / "attn_common.h", PKG.parent / "include" / "omni_dit.h"]
 
 # (source file, extra defines, object stem)
 UNITS: list[tuple[str, list[str], str]] = [
@@ -33,6 +33,7 @@ UNITS: list[tuple[str, list[str], str]] = [
     ("qknorm_rope.hip", ["-DODIT_QK_TU=1"], "qknorm_rope_f16"),
     ("qknorm_rope.hip", ["-DODIT_QK_TU=2"], "qknorm_rope_f32"),
     ("attn_fwd.hip", [], "attn_fwd"),
+    ("attn_fwd_dma.hip", [], "attn_fwd_dma"),
 ]
 
 # -packed-fp32-ops is switched off on purpose: v_pk_*_f32 forms are not trusted on this target.
