@@ -170,8 +170,8 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
     return mx;
   };
 
+  // mx = row maximum over both lane halves
   auto settle_max = [&](float mx) {
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m_run, mx);
     if (__any((m_new - m_run) * c > 8.f)) {
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
@@ -242,33 +242,46 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
     l_run += psum;
 
     // ---- stage B: O^T += V(j)^T P(j)^T ----
-    // 4*DT steps (dt, kt, g2); the two transpose reads of step n + PF are issued before the MFMA of
-    // step n, so LDS latency is covered by PF matrix instructions
+    // 4*DT steps, head-dim tile innermost so that consecutive MFMAs hit different accumulators and one
+    // P fragment serves DT of them; the two transpose reads of step n + PF are issued before the MFMA
+    // of step n, so LDS latency is covered by PF matrix instructions. The in-lane row maximum of
+    // S(j+1) — vector work with nothing to wait for — is placed in the shadow of these MFMAs.
     const char* vt_base = Vb + buf * TILEB;
     constexpr int NSTEP = 4 * DT;
     constexpr int PF = 3;
     s16x4_d vlo[PF + 1], vhi[PF + 1];
     auto v_fetch = [&](int step) {
-      const int dt = step >> 2, kt = (step >> 1) & 1, g2 = step & 1;
+      const int dt = step % DT, kt = (step / DT) >> 1, g2 = (step / DT) & 1;
       const char* vp = vt_base + (kt * 32 + g2 * 16) * ROWB + (v_lane ^ ((dt * 64) % ROWB));
       vlo[step % (PF + 1)] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_p)(vp));
       vhi[step % (PF + 1)] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_p)(vp + 8 * ROWB));
     };
+    const bool plain_next = has_next && mrow == nullptr && (j + 2) * BN <= p.Sk;  // no exclusions in S(j+1)
+    float mx = -INFINITY;
 #pragma unroll
     for (int st = 0; st < PF; ++st) v_fetch(st);
 #pragma unroll
     for (int st = 0; st < NSTEP; ++st) {
       if (st + PF < NSTEP) v_fetch(st + PF);
-      const int dt = st >> 2, kt = (st >> 1) & 1, g2 = st & 1;
+      const int dt = st % DT, kt = (st / DT) >> 1, g2 = (st / DT) & 1;
       const s16x8_d av = __builtin_shufflevector(vlo[st % (PF + 1)], vhi[st % (PF + 1)], 0, 1, 2, 3, 4, 5, 6, 7);
       u32x4_v pb;
       pb.x = pf[kt][g2][0]; pb.y = pf[kt][g2][1]; pb.z = pf[kt][g2][2]; pb.w = pf[kt][g2][3];
       o[dt] = M::run(__builtin_bit_cast(frag, av), __builtin_bit_cast(frag, pb), o[dt]);
+      if (st == 1 && plain_next) {  // wave-uniform
+        float t = s_next[0][0];
+#pragma unroll
+        for (int kt2 = 0; kt2 < 2; ++kt2)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) t = fmaxf(t, s_next[kt2][e]);
+        mx = fmaxf(t, __shfl_xor(t, 32, 64));
+      }
       __builtin_amdgcn_sched_barrier(0);  // keep the reads of step st+PF ahead of this MFMA
     }
-
-    float mx = -INFINITY;
-    if (has_next) mx = mask_and_max(j + 1, s_next);
+    if (has_next && !plain_next) {
+      const float t = mask_and_max(j + 1, s_next);
+      mx = fmaxf(t, __shfl_xor(t, 32, 64));
+    }
     __builtin_amdgcn_s_waitcnt(0);  // this wave's tile loads have landed in LDS
     __syncthreads();
     if (has_next) settle_max(mx);
@@ -282,7 +295,10 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   __syncthreads();
   f32x16_v sa[2], sb[2];
   qk_plain(Kb, sa);
-  settle_max(mask_and_max(0, sa));
+  {
+    const float t = mask_and_max(0, sa);
+    settle_max(fmaxf(t, __shfl_xor(t, 32, 64)));
+  }
 
   for (int j = 0; j < n_tiles; j += 2) {
     tile(j, sa, sb);
