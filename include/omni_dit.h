@@ -73,6 +73,19 @@ int odit_attn_fwd(const void* q, const void* k, const void* v, void* o, const ui
                   const int64_t v_strides[3], const int64_t o_strides[3], float scale, int dtype,
                   void* stream);
 
+/* Same as odit_attn_fwd, with the output of the joint sequence split at a row: query rows
+ * [0, q_split) are written to `o` (row r -> o row r), rows [q_split, Sq) to `o_tail` (row r -> o_tail
+ * row r - q_split), each with its own (batch, seq, head) strides. Replaces the two slices
+ * joint_hidden_states[:, :seq_len_txt] / [:, seq_len_txt:] of qwen_image_transformer.py:654-656, whose
+ * strided views otherwise force a copy in front of each output projection. o_tail == NULL behaves
+ * exactly like odit_attn_fwd.
+ */
+int odit_attn_fwd_split(const void* q, const void* k, const void* v, void* o, void* o_tail, int q_split,
+                        const uint8_t* key_mask, float* lse, int B, int Sq, int Sk, int H, int Hkv,
+                        int D, const int64_t q_strides[3], const int64_t k_strides[3],
+                        const int64_t v_strides[3], const int64_t o_strides[3],
+                        const int64_t o_tail_strides[3], float scale, int dtype, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * K2  fused QK-RMSNorm + rotary embedding + scatter into the joint [txt;img] sequence.
  *

@@ -370,6 +370,27 @@ def test_attention_key_mask_equals_deleting_keys(gpu, monkeypatch, variant):
                        layer(q.to(gpu), k.to(gpu), v.to(gpu)).cpu())
 
 
+@pytest.mark.parametrize("variant", ["18", "28", "38", "34"])
+@pytest.mark.parametrize("split", [0, 1, 37, 64, 299, 300])
+def test_attention_split_output_equals_slices(gpu, monkeypatch, variant, split):
+    """Two dense outputs written by the kernel == slices of the single output, bit for bit."""
+    from vllm_omni_amd import kernels
+
+    monkeypatch.setenv("ODIT_ATTN_VARIANT", variant)
+    B, S, H, D = 2, 300, 3, 128
+    q, k, v = (t.to(gpu) for t in _attn_inputs(B, S, S, H, H, D, seed=77))
+    print(f"attn split variant={variant} split={split}", flush=True)
+    whole, lse = kernels.attn_fwd(q, k, v, 0.09, return_lse=True)
+    head, tail, lse2 = kernels.attn_fwd(q, k, v, 0.09, return_lse=True, split=split)
+    assert head.shape == (B, split, H, D) and tail.shape == (B, S - split, H, D)
+    assert head.is_contiguous() and tail.is_contiguous()
+    assert torch.equal(head.cpu(), whole[:, :split].cpu())
+    assert torch.equal(tail.cpu(), whole[:, split:].cpu())
+    assert torch.equal(lse.cpu(), lse2.cpu())
+    with pytest.raises(ValueError):
+        kernels.attn_fwd(q, k, v, 0.09, split=S + 1)
+
+
 def test_attention_fp32_goes_to_sdpa(gpu):
     from vllm_omni_amd.attention.layer import Attention
 

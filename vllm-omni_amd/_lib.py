@@ -30,6 +30,12 @@ _SIGNATURES = {
          C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
          _i64p, _i64p, _i64p, _i64p, C.c_float, C.c_int, C.c_void_p],
     ),
+    "odit_attn_fwd_split": (
+        C.c_int,
+        [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p,
+         C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
+         _i64p, _i64p, _i64p, _i64p, _i64p, C.c_float, C.c_int, C.c_void_p],
+    ),
     "odit_qknorm_rope": (
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,

@@ -50,7 +50,9 @@ class AttentionBackend(ABC):
 @dataclass
 class AttentionMetadata:
     """Per-call extras (abstract.py:54-66). ``attn_mask`` is a [B,Sk] key-padding mask; the joint_*
-    fields carry a replicated text segment for sequence-parallel strategies and are unused on one GPU."""
+    fields carry a replicated text segment for sequence-parallel strategies and are unused on one GPU.
+    ``output_split`` (not in the reference) asks the backend for two dense outputs, rows [0, s) and
+    [s, Sq) of the joint sequence, instead of one tensor the caller would slice and copy."""
 
     attn_mask: torch.Tensor | None = None
     joint_attn_mask: torch.Tensor | None = None
@@ -58,6 +60,7 @@ class AttentionMetadata:
     joint_key: torch.Tensor | None = None
     joint_value: torch.Tensor | None = None
     joint_strategy: str = "front"
+    output_split: int | None = None
 
 
 T = TypeVar("T", bound=AttentionMetadata)

@@ -43,6 +43,10 @@ class SDPAImpl(AttentionImpl):
         out = torch.nn.functional.scaled_dot_product_attention(
             q, k, v, attn_mask=mask, dropout_p=0.0, is_causal=self.causal, scale=self.softmax_scale,
             enable_gqa=k.shape[1] != q.shape[1])
-        return out.transpose(1, 2)
+        out = out.transpose(1, 2)
+        split = attn_metadata.output_split if attn_metadata else None
+        if split is not None:
+            return out[:, :split].contiguous(), out[:, split:].contiguous()
+        return out
 
     forward_cuda = forward_hip

@@ -188,15 +188,16 @@ class QwenImageCrossAttention(nn.Module):
         kernels.qknorm_rope(img_qkv[:, :, 0], img_qkv[:, :, 1], img_qkv[:, :, 2], jq, jk, jv,
                             self.norm_q.weight, self.norm_k.weight, tables.img_cos, tables.img_sin,
                             eps=self.eps, out_seq_offset=S_txt, norm_mode=ODIT_NORM_HEAD, ref_rounding=rr)
-        meta = None
+        # the backend writes the text and image rows of the output to two dense tensors
+        meta = AttentionMetadata(output_split=S_txt)
         if hidden_states_mask is not None or encoder_hidden_states_mask is not None:
             ones = lambda n: torch.ones((B, n), dtype=torch.bool, device=jq.device)  # noqa: E731
             txt_m = encoder_hidden_states_mask if encoder_hidden_states_mask is not None else ones(S_txt)
             img_m = hidden_states_mask if hidden_states_mask is not None else ones(S_img)
-            meta = AttentionMetadata(attn_mask=torch.cat([txt_m.bool(), img_m.bool()], dim=1))
-        joint = self.attn(jq, jk, jv, meta).flatten(2, 3)
-        img_out = self.to_out(joint[:, S_txt:, :])
-        txt_out = self.to_add_out(joint[:, :S_txt, :])
+            meta.attn_mask = torch.cat([txt_m.bool(), img_m.bool()], dim=1)
+        txt_attn, img_attn = self.attn(jq, jk, jv, meta)
+        img_out = self.to_out(img_attn.flatten(2, 3))
+        txt_out = self.to_add_out(txt_attn.flatten(2, 3))
         return img_out, txt_out
 
 

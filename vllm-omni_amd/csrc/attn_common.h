@@ -43,7 +43,18 @@ struct AttnParams {
   int64_t qs_b, qs_s, qs_h, ks_b, ks_s, ks_h, vs_b, vs_s, vs_h, os_b, os_s, os_h;
   float scale, scale_log2;
   int n_qblocks, total_blocks;
+  // optional second output: query rows >= q_split are written to o_tail[row - q_split]
+  void* o_tail; int q_split;
+  int64_t ts_b, ts_s, ts_h;
 };
+
+// address of output row `row` of (batch b, head h): head of the joint sequence in `o`, tail in `o_tail`
+template <typename T>
+__device__ __forceinline__ T* out_row_ptr(const AttnParams& p, int b, int h, int row) {
+  if (p.o_tail != nullptr && row >= p.q_split)
+    return static_cast<T*>(p.o_tail) + b * p.ts_b + h * p.ts_h + static_cast<int64_t>(row - p.q_split) * p.ts_s;
+  return static_cast<T*>(p.o) + b * p.os_b + h * p.os_h + static_cast<int64_t>(row) * p.os_s;
+}
 
 constexpr int kNumXcd = 8;
 

@@ -267,14 +267,13 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(const AttnParams p) {
   }
 
   // ---- epilogue: normalise and store O (and LSE) ----
-  T* obase = static_cast<T*>(p.o) + b * p.os_b + h * p.os_h;
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     const float l_tot = l_run[qt] + __shfl_xor(l_run[qt], 32, 64);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int row = q0 + qt * 32 + l32;
     if (row < p.Sq) {
-      T* op = obase + row * p.os_s;
+      T* op = out_row_ptr<T>(p, b, h, row);
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -548,12 +547,11 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_pipe_kernel(const At
   }
 
   // ---- epilogue ----
-  T* obase = static_cast<T*>(p.o) + b * p.os_b + h * p.os_h;
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   const int row = q0 + l32;
   if (row < p.Sq) {
-    T* op = obase + row * p.os_s;
+    T* op = out_row_ptr<T>(p, b, h, row);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -616,12 +614,36 @@ static int dispatch_attn(AttnParams& p, int variant, hipStream_t stream) {
 
 }  // namespace odit
 
+extern "C" int odit_attn_fwd_split(const void* q, const void* k, const void* v, void* o, void* o_tail,
+                                   int q_split, const uint8_t* key_mask, float* lse, int B, int Sq,
+                                   int Sk, int H, int Hkv, int D, const int64_t q_strides[3],
+                                   const int64_t k_strides[3], const int64_t v_strides[3],
+                                   const int64_t o_strides[3], const int64_t o_tail_strides[3],
+                                   float scale, int dtype, void* stream);
+
 extern "C" int odit_attn_fwd(const void* q, const void* k, const void* v, void* o,
                              const uint8_t* key_mask, float* lse, int B, int Sq, int Sk, int H,
                              int Hkv, int D, const int64_t q_strides[3], const int64_t k_strides[3],
                              const int64_t v_strides[3], const int64_t o_strides[3], float scale,
                              int dtype, void* stream) {
+  return odit_attn_fwd_split(q, k, v, o, nullptr, 0, key_mask, lse, B, Sq, Sk, H, Hkv, D, q_strides,
+                             k_strides, v_strides, o_strides, nullptr, scale, dtype, stream);
+}
+
+extern "C" int odit_attn_fwd_split(const void* q, const void* k, const void* v, void* o, void* o_tail,
+                                   int q_split, const uint8_t* key_mask, float* lse, int B, int Sq,
+                                   int Sk, int H, int Hkv, int D, const int64_t q_strides[3],
+                                   const int64_t k_strides[3], const int64_t v_strides[3],
+                                   const int64_t o_strides[3], const int64_t o_tail_strides[3],
+                                   float scale, int dtype, void* stream) {
   using namespace odit;
+  if (o_tail != nullptr) {
+    ODIT_CHECK_ARG(o_tail_strides != nullptr, "odit_attn_fwd_split: o_tail given without strides");
+    ODIT_CHECK_ARG(q_split >= 0 && q_split <= Sq, "odit_attn_fwd_split: q_split=%d outside [0, Sq=%d]", q_split, Sq);
+    ODIT_CHECK_ARG(aligned16(o_tail) && o_tail_strides[0] % 8 == 0 && o_tail_strides[1] % 8 == 0 &&
+                       o_tail_strides[2] % 8 == 0,
+                   "odit_attn_fwd_split: o_tail must be 16-byte aligned with strides multiple of 8");
+  }
   ODIT_CHECK_ARG(q && k && v && o, "odit_attn_fwd: q/k/v/o must not be null");
   ODIT_CHECK_ARG(q_strides && k_strides && v_strides && o_strides, "odit_attn_fwd: null strides");
   ODIT_CHECK_ARG(B >= 0 && Sq >= 0 && Sk >= 0 && H > 0 && Hkv > 0, "odit_attn_fwd: bad shape");
@@ -654,6 +676,8 @@ extern "C" int odit_attn_fwd(const void* q, const void* k, const void* v, void* 
   p.os_b = o_strides[0]; p.os_s = o_strides[1]; p.os_h = o_strides[2];
   p.scale = scale;
   p.scale_log2 = scale * 1.4426950408889634f;
+  p.o_tail = o_tail; p.q_split = q_split;
+  p.ts_b = o_tail ? o_tail_strides[0] : 0; p.ts_s = o_tail ? o_tail_strides[1] : 0; p.ts_h = o_tail ? o_tail_strides[2] : 0;
 
   int variant = 34;
   if (const char* e = getenv("ODIT_ATTN_VARIANT")) variant = atoi(e);

@@ -306,12 +306,11 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   }
 
   // ---- epilogue ----
-  T* obase = static_cast<T*>(p.o) + b * p.os_b + h * p.os_h;
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   const int row = q0 + l32;
   if (row < p.Sq) {
-    T* op = obase + row * p.os_s;
+    T* op = out_row_ptr<T>(p, b, h, row);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll

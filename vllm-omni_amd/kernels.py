@@ -69,11 +69,13 @@ def attn_fwd(
     scale: float,
     key_mask: torch.Tensor | None = None,
     return_lse: bool = False,
+    split: int | None = None,
 ):
     """softmax(q k^T * scale) v for q [B,Sq,H,D], k/v [B,Sk,Hkv,D] (BSHD, bf16/fp16).
 
     key_mask: optional [B,Sk] bool/uint8, False/0 = key excluded. Returns o [B,Sq,H,D]
-    (and lse [B,H,Sq] float32 when return_lse).
+    (and lse [B,H,Sq] float32 when return_lse). With ``split`` = s the output comes back as two dense
+    tensors (o[:, :s], o[:, s:]) written directly by the kernel.
     """
     _dev(q, k, v, key_mask)
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
@@ -90,7 +92,10 @@ def attn_fwd(
         return t if ok else t.contiguous()
 
     q, k, v = _prep(q), _prep(k), _prep(v)
-    o = torch.empty((B, Sq, H, D), dtype=q.dtype, device=q.device)
+    if split is not None and not 0 <= split <= Sq:
+        raise ValueError(f"split={split} outside [0, {Sq}]")
+    o = torch.empty((B, Sq if split is None else split, H, D), dtype=q.dtype, device=q.device)
+    o_tail = None if split is None else torch.empty((B, Sq - split, H, D), dtype=q.dtype, device=q.device)
     lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device) if return_lse else None
     mask_u8 = None
     if key_mask is not None:
@@ -98,15 +103,39 @@ def attn_fwd(
             raise ValueError(f"key_mask must be [B,Sk]={B, Sk}, got {tuple(key_mask.shape)}")
         mask_u8 = (key_mask != 0).to(torch.uint8).contiguous()
     lib = _lib.load()
-    rc = lib.odit_attn_fwd(
-        q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), _ptr(mask_u8), _ptr(lse),
-        B, Sq, Sk, H, Hkv, D,
+    if split is not None and split in (0, Sq):  # one side is empty: the plain entry point writes the other
+        full = o_tail if split == 0 else o
+        rc = lib.odit_attn_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), full.data_ptr(), _ptr(mask_u8), _ptr(lse),
+            B, Sq, Sk, H, Hkv, D,
+            _lib.i64_array(q.stride()[:3]), _lib.i64_array(k.stride()[:3]),
+            _lib.i64_array(v.stride()[:3]), _lib.i64_array((Sq * H * D, H * D, D)),
+            float(scale), _code(q), _stream(),
+        )
+        _lib.check(rc, "odit_attn_fwd")
+        return (o, o_tail, lse) if return_lse else (o, o_tail)
+    if split is None:
+        rc = lib.odit_attn_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), _ptr(mask_u8), _ptr(lse),
+            B, Sq, Sk, H, Hkv, D,
+            _lib.i64_array(q.stride()[:3]), _lib.i64_array(k.stride()[:3]),
+            _lib.i64_array(v.stride()[:3]), _lib.i64_array(o.stride()[:3]),
+            float(scale), _code(q), _stream(),
+        )
+        _lib.check(rc, "odit_attn_fwd")
+        return (o, lse) if return_lse else o
+    # dense [B, n, H, D] strides even when n == 0 or B == 1 (torch may report arbitrary ones there)
+    o_str = (split * H * D, H * D, D)
+    t_str = ((Sq - split) * H * D, H * D, D)
+    rc = lib.odit_attn_fwd_split(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), o_tail.data_ptr(), int(split),
+        _ptr(mask_u8), _ptr(lse), B, Sq, Sk, H, Hkv, D,
         _lib.i64_array(q.stride()[:3]), _lib.i64_array(k.stride()[:3]),
-        _lib.i64_array(v.stride()[:3]), _lib.i64_array(o.stride()[:3]),
+        _lib.i64_array(v.stride()[:3]), _lib.i64_array(o_str), _lib.i64_array(t_str),
         float(scale), _code(q), _stream(),
     )
-    _lib.check(rc, "odit_attn_fwd")
-    return (o, lse) if return_lse else o
+    _lib.check(rc, "odit_attn_fwd_split")
+    return (o, o_tail, lse) if return_lse else (o, o_tail)
 
 
 # --------------------------------------------------------------------------------------------- K2
