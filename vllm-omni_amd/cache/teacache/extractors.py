@@ -85,8 +85,41 @@ def extract_qwen_context(module: nn.Module, hidden_states: torch.Tensor,
                         run_transformer_blocks_rows=run_rows)
 
 
+def extract_flux_context(module: nn.Module, hidden_states: torch.Tensor,
+                         encoder_hidden_states: torch.Tensor | None = None,
+                         pooled_projections: torch.Tensor | None = None, timestep: torch.Tensor | None = None,
+                         img_ids: torch.Tensor | None = None, txt_ids: torch.Tensor | None = None,
+                         guidance: torch.Tensor | None = None,
+                         joint_attention_kwargs: dict[str, Any] | None = None, **kwargs: Any) -> CacheContext:
+    """Flux: stem, then block 0's norm1 (AdaLayerNormZero) on the x_embedder output is the decision
+    tensor — the recipe the reference sketches for this model (extractors.py:580, 597-613) with the
+    coefficients it already ships (config.py:11-17). ``module`` is this package's FluxTransformer2DModel."""
+    if not hasattr(module, "transformer_blocks") or len(module.transformer_blocks) == 0:
+        raise ValueError("Module must have transformer_blocks")
+    img, txt, temb, rotary = module.prepare(hidden_states, encoder_hidden_states, pooled_projections, timestep,
+                                            img_ids, txt_ids, guidance)
+    modulated = module.transformer_blocks[0].norm1(img, emb=temb)[0]
+    return_dict = kwargs.get("return_dict", True)
+
+    def run_rows(rows: list[int] | None):
+        if rows is None:
+            h, e, t = img, txt, temb
+        else:
+            idx = torch.as_tensor(rows, device=img.device)
+            h, e, t = img.index_select(0, idx), txt.index_select(0, idx), temb.index_select(0, idx)
+        return module.run_blocks(h, e, t, rotary, joint_attention_kwargs)
+
+    def postprocess(h):
+        return module.finish(h, temb, return_dict=return_dict)
+
+    return CacheContext(modulated_input=modulated, hidden_states=img, encoder_hidden_states=txt, temb=temb,
+                        run_transformer_blocks=lambda: run_rows(None), postprocess=postprocess,
+                        run_transformer_blocks_rows=run_rows)
+
+
 EXTRACTOR_REGISTRY: dict[str, Callable] = {
     "QwenImageTransformer2DModel": extract_qwen_context,
+    "FluxTransformer2DModel": extract_flux_context,
 }
 
 

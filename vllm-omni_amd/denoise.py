@@ -84,3 +84,27 @@ def diffuse(transformer, inp: DenoiseInputs, num_inference_steps: int, true_cfg_
         if on_step is not None:
             on_step(i, latents)
     return latents
+
+
+def diffuse_flux(transformer, latents: torch.Tensor, prompt_embeds: torch.Tensor, pooled_prompt_embeds: torch.Tensor,
+                 img_ids: torch.Tensor, txt_ids: torch.Tensor, num_inference_steps: int,
+                 guidance_scale: float | None = 3.5, on_step=None) -> torch.Tensor:
+    """Guidance-distilled Flux loop: one transformer call per step, no CFG pair
+    (vllm_omni/diffusion/models/flux/pipeline_flux.py denoising loop: timestep / 1000, embedded
+    guidance scale, flow-match Euler step)."""
+    transformer.do_true_cfg = False
+    transformer.cfg_batched_branches = None
+    nb = latents.shape[0]
+    sig = flow_match_sigmas(num_inference_steps, latents.shape[1])
+    guidance = None
+    if guidance_scale is not None and getattr(transformer, "guidance_embeds", True):
+        guidance = torch.full((nb,), float(guidance_scale), device=latents.device, dtype=torch.float32)
+    for i in range(num_inference_steps):
+        t = (torch.full((nb,), float(sig[i]) * 1000.0, device=latents.device, dtype=latents.dtype) / 1000)
+        noise = transformer(hidden_states=latents, encoder_hidden_states=prompt_embeds,
+                            pooled_projections=pooled_prompt_embeds, timestep=t, img_ids=img_ids, txt_ids=txt_ids,
+                            guidance=guidance, return_dict=False)[0]
+        latents = euler_step(latents, noise, float(sig[i]), float(sig[i + 1]))
+        if on_step is not None:
+            on_step(i, latents)
+    return latents
