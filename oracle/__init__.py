@@ -15,8 +15,13 @@ Parity status of arithmetic that lives in third-party wheels absent from the ref
   * ``rms_norm_head``      vllm RMSNorm cast order (fp32 normalise -> cast -> x weight); vllm==0.16.0 / 0.14.0+rocm700
   * ``ada_layer_norm_continuous``, ``timestep_embedding`` + ``TimestepEmbedding`` MLP,
     ``flow_match_euler_step`` / sigma shifting    diffusers>=0.36.0 (AdaLayerNormContinuous chunk
-    order scale,shift; FlowMatchEulerDiscreteScheduler). ``timestep_embedding`` itself IS pinned by the
-    in-tree duplicate at pipeline_qwen_image.py:141-190.
+    order scale,shift; FlowMatchEulerDiscreteScheduler). The sinusoid of ``timestep_embedding`` is pinned
+    by closed forms and, in its ``cast_freqs`` form, follows the in-tree function at
+    pipeline_qwen_image.py:141-190; that the transformers' ``Timesteps`` keeps fp32 frequencies is the
+    upstream convention.
+  * Flux: ``AdaLayerNormZero`` / ``AdaLayerNormZeroSingle`` chunk orders, the combined
+    timestep/guidance/pooled-text embedding, ``get_1d_rotary_pos_embed``; Wan: ``FP32LayerNorm``,
+    ``PixArtAlphaTextProjection`` (diffusers>=0.36.0; see ``oracle/flux.py``, ``oracle/wan.py``).
 Everything else (attention, interleaved/NeoX rotary, AdaLayerNorm, gated residual, rel-L1, TeaCache
 decision logic, Qwen rope tables, block wiring, CFG combine) follows code present in the reference.
 """

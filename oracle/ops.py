@@ -208,13 +208,18 @@ def poly_horner(coeffs, x: float) -> float:
 
 def timestep_embedding(t: torch.Tensor, dim: int = 256, flip_sin_to_cos: bool = True,
                        downscale_freq_shift: float = 0.0, scale: float = 1000.0,
-                       max_period: int = 10000) -> torch.Tensor:
-    """Sinusoidal embedding of fractional timesteps, fp32. In-tree statement:
-    models/qwen_image/pipeline_qwen_image.py:141-190; used through diffusers Timesteps at
-    models/qwen_image/qwen_image_transformer.py:163."""
+                       max_period: int = 10000, cast_freqs: bool = False) -> torch.Tensor:
+    """Sinusoidal embedding of (possibly fractional or integer) timesteps, fp32: what diffusers'
+    ``Timesteps`` module evaluates at models/qwen_image/qwen_image_transformer.py:163,
+    models/flux/flux_transformer.py:462-466 and models/wan2_2/wan2_2_transformer.py:265 (third-party:
+    frequencies stay fp32 and multiply ``t.float()``). ``cast_freqs=True`` is the variant of the in-tree
+    function models/qwen_image/pipeline_qwen_image.py:141-190, which first casts the frequencies to
+    t's dtype; no transformer on this path calls that one."""
     half = dim // 2
     freqs = torch.exp(-math.log(max_period) * torch.arange(half, dtype=torch.float32) / (half - downscale_freq_shift))
-    arg = scale * (t[:, None].float() * freqs[None, :].to(t.dtype))
+    if cast_freqs:
+        freqs = freqs.to(t.dtype)
+    arg = scale * (t[:, None].float() * freqs[None, :])
     emb = torch.cat((torch.sin(arg), torch.cos(arg)), dim=-1)
     if flip_sin_to_cos:
         emb = torch.cat((emb[:, half:], emb[:, :half]), dim=-1)

@@ -1,0 +1,151 @@
+"""Wan blocks on the GPU: a tiny video DiT (2 blocks, hidden 256 = 4 heads x 64, FFN 640) built from
+the HIP kernels in bf16 against the fp32 CPU oracle, per block (max-abs <= 2e-2, cosine >= 0.9995), on a
+ragged 3x5x7 patch grid with 13 text tokens; plus one block at the Wan2.1-14B width (hidden 5120 =
+40 heads x 128, FFN 13824) on a short sequence against the oracle, and size-independent properties of
+that block at a long sequence."""
+
+import pytest
+import torch
+
+from oracle import wan as ow
+
+pytestmark = pytest.mark.gpu
+
+
+def _cosine(a, b):
+    a, b = a.float().flatten().cpu(), b.float().flatten().cpu()
+    return float(torch.dot(a, b) / (a.norm() * b.norm()))
+
+
+def _model(gpu, cfg, w_lp, dtype=torch.bfloat16):
+    from vllm_omni_amd.attention.selector import get_attn_backend
+    from vllm_omni_amd.blocks.wan import WanTransformer3DModel
+
+    get_attn_backend.cache_clear()
+    model = WanTransformer3DModel(
+        patch_size=cfg.patch_size, num_attention_heads=cfg.num_heads, attention_head_dim=cfg.head_dim,
+        in_channels=cfg.in_channels, out_channels=cfg.out_channels, text_dim=cfg.text_dim, freq_dim=cfg.freq_dim,
+        ffn_dim=cfg.ffn_dim, num_layers=cfg.num_layers, cross_attn_norm=cfg.cross_attn_norm, eps=cfg.eps,
+        rope_max_seq_len=cfg.rope_max_seq_len).to(gpu).to(dtype)
+    model.load_flat_state(w_lp)
+    return model
+
+
+@pytest.mark.parametrize("fhw,n_txt,B", [((3, 10, 14), 13, 2), ((1, 16, 16), 32, 1)])
+def test_tiny_wan_per_block_parity(gpu, fhw, n_txt, B):
+    cfg = ow.tiny_config()
+    w32 = ow.init_params(cfg, seed=0, bias_std=0.02, norm_jitter=0.1)
+    w = {k: v.bfloat16() for k, v in w32.items()}
+    model = _model(gpu, cfg, w)
+    g = torch.Generator().manual_seed(1)
+    video = torch.randn(B, cfg.in_channels, *fhw, generator=g).bfloat16()
+    text = torch.randn(B, n_txt, cfg.text_dim, generator=g).bfloat16()
+    t = torch.tensor([731.0, 204.0][:B])
+    wf = {k: v.float() for k, v in w.items()}
+    want, per_block = ow.transformer_forward(wf, cfg, video.float(), t, text.float(), collect_blocks=True)
+    with torch.inference_mode():
+        x, ctx, temb, tproj, rot = model.prepare(video.to(gpu), t.to(gpu), text.to(gpu))
+        for i, block in enumerate(model.blocks):
+            x = block(x, ctx, tproj, rot)
+            err = (x.float().cpu() - per_block[i]).abs().max().item()
+            cos = _cosine(x, per_block[i])
+            print(f"wan block {i}: max-abs {err:.4f} cosine {cos:.6f}", flush=True)
+            assert err <= 2e-2 and cos >= 0.9995, (i, err, cos)
+        grid = (fhw[0], fhw[1] // 2, fhw[2] // 2)
+        out = model.finish(x, temb, grid, return_dict=False)[0]
+        out2 = model(video.to(gpu), t.to(gpu), text.to(gpu)).sample
+    assert out.shape == video.shape
+    assert (out.float().cpu() - want).abs().max().item() <= 2e-2 and _cosine(out, want) >= 0.9995
+    # forward() forms all blocks' modulation rows in one op: same values, same result
+    assert torch.equal(out2, out)
+
+
+def test_unbuilt_variants_raise(gpu):
+    from vllm_omni_amd.blocks.wan import WanTransformer3DModel, WanTransformerBlock
+
+    with pytest.raises(NotImplementedError):
+        WanTransformerBlock(256, 640, 4, added_kv_proj_dim=128)
+    with pytest.raises(NotImplementedError):
+        WanTransformer3DModel(num_attention_heads=4, attention_head_dim=64, ffn_dim=640, num_layers=1, image_dim=64)
+
+
+def _wide_block(gpu, seed=0):
+    """One block at the 14B width with synthetic weights, and the same weights for the oracle."""
+    from vllm_omni_amd.attention.selector import get_attn_backend
+    from vllm_omni_amd.blocks.wan import WanTransformerBlock
+
+    get_attn_backend.cache_clear()
+    cfg = ow.WanConfig(num_layers=1)
+    g = torch.Generator().manual_seed(seed)
+    w = {}
+    for n, s in ow.block_param_shapes(cfg).items():
+        if n.endswith("scale_shift_table"):
+            t = torch.randn(s, generator=g) / s[-1] ** 0.5
+        elif n.endswith(("norm_q.weight", "norm_k.weight", "norm2.weight")):
+            t = 1 + 0.1 * torch.randn(s, generator=g)
+        elif n.endswith(".bias"):
+            t = 0.02 * torch.randn(s, generator=g)
+        else:
+            t = 0.02 * torch.randn(s, generator=g)
+        w["blocks.0." + n] = t.bfloat16()
+    blk = WanTransformerBlock(cfg.dim, cfg.ffn_dim, cfg.num_heads, cfg.eps, None, True).to(gpu).bfloat16()
+    with torch.no_grad():
+        for k, p in blk.named_parameters():
+            p.copy_(w["blocks.0." + k].to(gpu))
+    return cfg, w, blk
+
+
+def test_wan_14b_width_block_against_oracle(gpu):
+    """hidden 5120, 40 heads x 128, FFN 13824, 2 x (2x6x8 = 96 video tokens), 24 text tokens."""
+    cfg, w, blk = _wide_block(gpu)
+    g = torch.Generator().manual_seed(3)
+    B, fhw, T = 2, (2, 6, 8), 24
+    S = fhw[0] * fhw[1] * fhw[2]
+    x = torch.randn(B, S, cfg.dim, generator=g).bfloat16()
+    ctx = torch.randn(B, T, cfg.dim, generator=g).bfloat16()
+    temb6 = (0.5 * torch.randn(B, 6, cfg.dim, generator=g)).bfloat16()
+    cos, sin = ow.wan_rope_tables(cfg, *fhw)
+    want = ow.block_forward({k: v.float() for k, v in w.items()}, 0, cfg, x.float(), ctx.float(), temb6.float(),
+                            cos, sin)
+    with torch.inference_mode():
+        got = blk(x.to(gpu), ctx.to(gpu), temb6.to(gpu), (cos.to(gpu), sin.to(gpu)))
+    err = (got.float().cpu() - want).abs().max().item()
+    cs = _cosine(got, want)
+    print(f"wan 14B-width block: max-abs {err:.4f} cosine {cs:.6f} (|x| max {want.abs().max():.2f})", flush=True)
+    # outputs reach |x| ~ 5: the bf16 ulp there is 3e-2, so the absolute bound scales with magnitude
+    assert err <= 2e-2 * max(1.0, want.abs().max().item() / 2) and cs >= 0.9995
+
+
+def test_wan_14b_width_block_long_sequence_properties(gpu):
+    """A 21x12x13 = 3276-token grid per sample (a tenth of the 81-frame 480x832 grid, same kernels and
+    dispatch): closing both gates leaves x + cross-attention only, and that remainder does not depend on
+    the rotary tables; permuting video tokens with their table rows permutes the output."""
+    cfg, w, blk = _wide_block(gpu, seed=1)
+    g = torch.Generator().manual_seed(4)
+    B, fhw, T = 2, (21, 12, 13), 512
+    S = fhw[0] * fhw[1] * fhw[2]
+    x = torch.randn(B, S, cfg.dim, generator=g).bfloat16().to(gpu)
+    ctx = torch.randn(B, T, cfg.dim, generator=g).bfloat16().to(gpu)
+    temb6 = (0.5 * torch.randn(B, 6, cfg.dim, generator=g)).bfloat16().to(gpu)
+    cos, sin = (t.to(gpu) for t in ow.wan_rope_tables(cfg, *fhw))
+    with torch.inference_mode():
+        base = blk(x, ctx, temb6, (cos, sin))
+        assert torch.isfinite(base.float()).all()
+        p = torch.randperm(S, generator=g).to(gpu)
+        perm = blk(x[:, p].contiguous(), ctx, temb6, (cos[:, p].contiguous(), sin[:, p].contiguous()))
+        d = (perm.float() - base[:, p].float()).abs().max().item()
+        print(f"token-permutation equivariance, S={S}: max diff {d:.4f}", flush=True)
+        # key order changes the summation order inside attention: allow two bf16 ulps at the output's scale
+        assert d <= base.float().abs().max().item() * 2 ** -6 and _cosine(perm, base[:, p]) >= 0.99999
+        # gates closed: mod = table + temb with rows 2 and 5 (the gates) forced to zero
+        mod = blk.scale_shift_table.float() + temb6.float()
+        mod[:, 2] = 0
+        mod[:, 5] = 0
+        closed = blk(x, ctx, None, (cos, sin), mod=mod)
+        closed_norope = blk(x, ctx, None, None, mod=mod)
+        assert torch.equal(closed, closed_norope)
+        from vllm_omni_amd import kernels
+        lw, lb = blk._norm2_affine()
+        n = kernels.adaln_modulate(x, None, None, eps=cfg.eps, ln_weight=lw, ln_bias=lb)
+        want = x + blk.attn2(n, ctx)
+        assert torch.equal(closed, want)

@@ -245,3 +245,13 @@ def test_timestep_embedding_layout():
     # last channel has frequency max_period^(-(127/128))
     f = math.exp(-math.log(10000) * 127 / 128)
     assert math.isclose(e[2, 127].item(), math.cos(1000.0 * f), abs_tol=1e-4)
+    # integer timesteps (Wan passes them raw, scale 1) keep fractional frequencies
+    ei = ops.timestep_embedding(torch.tensor([500]), scale=1.0)
+    assert math.isclose(ei[0, 127].item(), math.cos(500.0 * f), abs_tol=1e-4)
+    # 16-bit timesteps: frequencies stay fp32 unless the in-tree variant is asked for
+    tb = torch.tensor([0.3]).bfloat16()
+    e32 = ops.timestep_embedding(tb)
+    assert math.isclose(e32[0, 127].item(), math.cos(1000.0 * f * float(tb[0])), abs_tol=1e-4)
+    ecast = ops.timestep_embedding(tb, cast_freqs=True)
+    fb = float(torch.tensor(f).bfloat16())
+    assert math.isclose(ecast[0, 127].item(), math.cos(1000.0 * fb * float(tb[0])), abs_tol=1e-4)

@@ -1,0 +1,127 @@
+"""Pins for the Wan oracle that do not retype its formulas: a library routine for the patch embedding
+and its inverse, invariances of the architecture (token permutation with the rotary tables carried
+along, text-token permutation, zero gates), the relative-position property of the 3D rotary tables,
+and fp32-vs-fp64 agreement."""
+
+import torch
+
+from oracle import ops
+from oracle import wan as ow
+
+
+def _setup(seed=0, B=1, fhw=(2, 4, 6), n_txt=5, dtype=torch.float64):
+    cfg = ow.tiny_config()
+    w = {k: v.to(dtype) for k, v in ow.init_params(cfg, seed=seed, std=0.05, bias_std=0.05, norm_jitter=0.1).items()}
+    g = torch.Generator().manual_seed(seed + 1)
+    video = torch.randn(B, cfg.in_channels, *fhw, generator=g, dtype=dtype)
+    text = torch.randn(B, n_txt, cfg.text_dim, generator=g, dtype=dtype)
+    t = torch.tensor([417.0, 902.0][:B], dtype=dtype)
+    return cfg, w, video, text, t
+
+
+def test_rope_table_layout_and_relative_position():
+    cfg = ow.tiny_config()
+    D = cfg.head_dim
+    cos, sin = ow.wan_rope_tables(cfg, 3, 4, 5)
+    assert cos.shape == (1, 60, 1, D) and cos.dtype == torch.float32
+    # each value appears twice along D; widths per axis are (D - 4*(D//6), 2*(D//6), 2*(D//6))
+    assert torch.equal(cos[..., 0::2], cos[..., 1::2]) and torch.equal(sin[..., 0::2], sin[..., 1::2])
+    wt = D - 4 * (D // 6)
+    tok = lambda f, h, w: (f * 4 + h) * 5 + w  # noqa: E731
+    # the frame slice depends on f only, the height slice on h only, the width slice on w only
+    assert torch.equal(cos[0, tok(1, 0, 0), 0, :wt], cos[0, tok(1, 3, 4), 0, :wt])
+    assert torch.equal(cos[0, tok(0, 2, 0), 0, wt:wt + 2 * (D // 6)], cos[0, tok(2, 2, 3), 0, wt:wt + 2 * (D // 6)])
+    assert torch.equal(cos[0, tok(0, 0, 3), 0, wt + 2 * (D // 6):], cos[0, tok(2, 1, 3), 0, wt + 2 * (D // 6):])
+    assert torch.all(cos[0, 0] == 1) and torch.all(sin[0, 0] == 0)
+    # scores depend on grid offsets only: compare pairs with equal (df, dh, dw)
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(1, 1, 1, D, generator=g, dtype=torch.float64)
+    k = torch.randn(1, 1, 1, D, generator=g, dtype=torch.float64)
+
+    def score(a, b):
+        qa = ops.apply_rotary_wan(q, cos[:, a:a + 1].double(), sin[:, a:a + 1].double())
+        kb = ops.apply_rotary_wan(k, cos[:, b:b + 1].double(), sin[:, b:b + 1].double())
+        return (qa * kb).sum()
+
+    torch.testing.assert_close(score(tok(0, 1, 1), tok(1, 3, 2)), score(tok(1, 0, 2), tok(2, 2, 3)), atol=1e-6, rtol=0)
+    assert abs(score(tok(0, 1, 1), tok(1, 3, 2)) - score(tok(0, 1, 1), tok(1, 3, 3))) > 1e-4
+
+
+def test_patch_embedding_is_a_linear_over_patches():
+    """The stem's Conv3d (library routine) equals gathering each (C_in, 1, 2, 2) patch into a row and
+    multiplying by the flattened kernel — the form the product uses."""
+    cfg, w, video, text, t = _setup(B=2)
+    x, _, _, _ = ow.stem(w, cfg, video, t, text)
+    B, Cin, nf, hh, ww = video.shape
+    rows = video.view(B, Cin, nf, 1, hh // 2, 2, ww // 2, 2).permute(0, 2, 4, 6, 1, 3, 5, 7).reshape(B, -1, Cin * 4)
+    want = rows @ w["patch_embedding.weight"].view(cfg.dim, -1).t() + w["patch_embedding.bias"]
+    torch.testing.assert_close(x, want, atol=1e-12, rtol=0)
+
+
+def test_unpatchify_inverts_patchify_layout():
+    """head() with an identity-like projection puts token (f,h,w)'s (p_t,p_h,p_w,c) block back at
+    video[c, f*p_t.., h*p_h.., w*p_w..]."""
+    cfg = ow.tiny_config()
+    grid, B = (2, 3, 4), 1
+    n_out = cfg.out_channels * 4
+    w = {"output_scale_shift_prepare.scale_shift_table": torch.zeros(1, 2, cfg.dim, dtype=torch.float64),
+         "proj_out.weight": torch.zeros(n_out, cfg.dim, dtype=torch.float64),
+         "proj_out.bias": torch.zeros(n_out, dtype=torch.float64)}
+    w["proj_out.weight"][:, :n_out] = torch.eye(n_out, dtype=torch.float64)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(B, 24, cfg.dim, generator=g, dtype=torch.float64)
+    out = ow.head(w, cfg, x, torch.zeros(B, cfg.dim, dtype=torch.float64), grid, B)
+    assert out.shape == (B, cfg.out_channels, 2, 6, 8)
+    xn = torch.nn.functional.layer_norm(x, (cfg.dim,), eps=cfg.eps)
+    f, h, ww_, ph, pw, c = 1, 2, 3, 1, 0, 5
+    tok = (f * 3 + h) * 4 + ww_
+    # projection output channel order is (p_t, p_h, p_w, c)
+    assert torch.isclose(out[0, c, f, h * 2 + ph, ww_ * 2 + pw], xn[0, tok, (ph * 2 + pw) * cfg.out_channels + c])
+
+
+def test_token_permutation_equivariance_of_a_block():
+    cfg, w, video, text, t = _setup(seed=3)
+    x, temb, temb6, ctx = ow.stem(w, cfg, video, t, text)
+    cos, sin = ow.wan_rope_tables(cfg, 2, 2, 3)
+    base = ow.block_forward(w, 0, cfg, x, ctx, temb6, cos, sin)
+    g = torch.Generator().manual_seed(5)
+    p = torch.randperm(x.shape[1], generator=g)
+    pt = torch.randperm(ctx.shape[1], generator=g)
+    out = ow.block_forward(w, 0, cfg, x[:, p], ctx, temb6, cos[:, p], sin[:, p])
+    torch.testing.assert_close(out, base[:, p], atol=2e-6, rtol=0)
+    out_t = ow.block_forward(w, 0, cfg, x, ctx[:, pt], temb6, cos, sin)
+    torch.testing.assert_close(out_t, base, atol=2e-6, rtol=0)
+    out_bad = ow.block_forward(w, 0, cfg, x[:, p], ctx, temb6, cos, sin)
+    assert (out_bad - base[:, p]).abs().max() > 1e-3
+
+
+def test_gates_and_plain_cross_attention_residual():
+    """table + temb = 0 closes both gates: what is left is exactly x + cross_attention(norm2(x)) —
+    the cross-attention residual carries no gate."""
+    cfg, w, video, text, t = _setup(seed=4)
+    x, temb, temb6, ctx = ow.stem(w, cfg, video, t, text)
+    cos, sin = ow.wan_rope_tables(cfg, 2, 2, 3)
+    w = dict(w)
+    w["blocks.0.scale_shift_table"] = -temb6[:1].clone()
+    out = ow.block_forward(w, 0, cfg, x, ctx, temb6[:1], cos, sin)
+    n = torch.nn.functional.layer_norm(x, (cfg.dim,), w["blocks.0.norm2.weight"], w["blocks.0.norm2.bias"], cfg.eps)
+    want = x + ow.cross_attention(w, "blocks.0.attn2.", cfg, n, ctx)
+    torch.testing.assert_close(out, want, atol=2e-6, rtol=0)  # the block's LayerNorms are fp32
+    # opening only the self-attention gate (3rd of the 6 rows) adds attn1 of the unmodulated LayerNorm
+    tbl = -temb6[:1].clone()
+    tbl[:, 2] += 1.0
+    w["blocks.0.scale_shift_table"] = tbl
+    out = ow.block_forward(w, 0, cfg, x, ctx, temb6[:1], cos, sin)
+    x1 = x + ow.self_attention(w, "blocks.0.attn1.", cfg, torch.nn.functional.layer_norm(x, (cfg.dim,), eps=cfg.eps),
+                               cos, sin)
+    n = torch.nn.functional.layer_norm(x1, (cfg.dim,), w["blocks.0.norm2.weight"], w["blocks.0.norm2.bias"], cfg.eps)
+    torch.testing.assert_close(out, x1 + ow.cross_attention(w, "blocks.0.attn2.", cfg, n, ctx), atol=2e-6, rtol=0)
+
+
+def test_fp32_agrees_with_fp64():
+    cfg, w, video, text, t = _setup(seed=6, B=2)
+    want = ow.transformer_forward(w, cfg, video, t, text)
+    w32 = {k: v.float() for k, v in w.items()}
+    got = ow.transformer_forward(w32, cfg, video.float(), t.float(), text.float())
+    assert got.shape == video.shape
+    torch.testing.assert_close(got.double(), want, atol=5e-4, rtol=1e-3)

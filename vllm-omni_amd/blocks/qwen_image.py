@@ -14,6 +14,7 @@ qit.py:1073-1113). Differences are all below the module interfaces:
 
 from __future__ import annotations
 
+import math
 from functools import lru_cache
 from typing import Any
 
@@ -282,11 +283,11 @@ class QwenTimestepProjEmbeddings(nn.Module):
 
     @staticmethod
     def time_proj(t: torch.Tensor, dim: int = 256, max_period: int = 10000, scale: float = 1000.0):
+        """diffusers ``Timesteps(dim, flip_sin_to_cos=True, downscale_freq_shift=0, scale)``: fp32
+        frequencies times ``t.float()``, cosines first."""
         half = dim // 2
-        import math
-
         freqs = torch.exp(-math.log(max_period) * torch.arange(half, dtype=torch.float32, device=t.device) / half)
-        arg = scale * (t[:, None].float() * freqs[None, :].to(t.dtype))
+        arg = scale * (t[:, None].float() * freqs[None, :])
         return torch.cat((torch.cos(arg), torch.sin(arg)), dim=-1)
 
     def forward(self, timestep: torch.Tensor, hidden_states: torch.Tensor, addition_t_cond=None):
