@@ -6,6 +6,7 @@ steps/s, the attention kernel's live-measured roofline fraction (bf16 MFMA), per
 TFLOP/s for the other kernels on the path, and the CPU oracle timed on the host cores.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--blocks N] [--no-cpu] [--no-kernels]
+  python bench.py --workload flux|wan [--steps K] [--warmup W]     (the other block families, same protocol)
 """
 
 from __future__ import annotations
@@ -57,6 +58,7 @@ class AttnTimer:
         self.torch, self.kernels = torch, kernels
         self.orig = kernels.attn_fwd
         self.pairs = []
+        self.flops = []
         self.active = False
 
     def __enter__(self):
@@ -67,7 +69,9 @@ class AttnTimer:
             s.record()
             out = self.orig(*a, **kw)
             e.record()
+            q, k = a[0], a[1]
             self.pairs.append((s, e))
+            self.flops.append(4.0 * q.shape[0] * q.shape[2] * q.shape[1] * k.shape[1] * q.shape[3])
             return out
 
         self.kernels.attn_fwd = timed
@@ -78,6 +82,12 @@ class AttnTimer:
 
     def mean_ms(self):
         return sum(s.elapsed_time(e) for s, e in self.pairs) / max(len(self.pairs), 1)
+
+    def dominant(self):
+        """(mean ms, flop per launch, launches) of the launches with the largest flop count."""
+        top = max(self.flops)
+        ms = [s.elapsed_time(e) for (s, e), f in zip(self.pairs, self.flops) if f == top]
+        return sum(ms) / len(ms), top, len(ms)
 
 
 def build_model(torch, layers):
@@ -103,6 +113,127 @@ def build_model(torch, layers):
                 p.normal_(0.0, 0.02, generator=g)
     model.fuse_modulation()
     return model.eval()
+
+
+def _init_synthetic(torch, model, seed=0):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if name.endswith(("norm_q.weight", "norm_k.weight", "norm2.weight", "txt_norm.weight")):
+                p.fill_(1.0)
+            elif name.endswith(".bias"):
+                p.zero_()
+            elif name.endswith("scale_shift_table"):
+                p.normal_(0.0, p.shape[-1] ** -0.5, generator=g)
+            else:
+                p.normal_(0.0, 0.02, generator=g)
+
+
+def flux_workload(torch, layers=None):
+    """BASELINE.json configs[4]: Flux shape, 19 dual + 38 single blocks, B=1, 512 text + 4096 image tokens."""
+    from vllm_omni_amd.blocks.flux import FluxTransformer2DModel
+    from vllm_omni_amd.denoise import euler_step, flow_match_sigmas
+
+    n_dual, n_single = (19, 38) if layers is None else (max(layers // 3, 1), max(layers - layers // 3, 1))
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device("cuda"):
+            model = FluxTransformer2DModel(num_layers=n_dual, num_single_layers=n_single)
+    finally:
+        torch.set_default_dtype(prev)
+    _init_synthetic(torch, model)
+    model.fuse_modulation()
+    model.eval()
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cuda").manual_seed(1)
+    s_txt, side = 512, 64
+    lat0 = torch.randn(1, side * side, 64, device=dev, generator=g).bfloat16()
+    text = torch.randn(1, s_txt, 4096, device=dev, generator=g).bfloat16()
+    pooled = torch.randn(1, 768, device=dev, generator=g).bfloat16()
+    ids = torch.zeros(side, side, 3, device=dev)
+    ids[..., 1] += torch.arange(side, device=dev)[:, None]
+    ids[..., 2] += torch.arange(side, device=dev)[None, :]
+    img_ids, txt_ids = ids.reshape(-1, 3), torch.zeros(s_txt, 3, device=dev)
+    guidance = torch.full((1,), 3.5, device=dev)
+    sig = flow_match_sigmas(28, side * side)
+
+    def step(i, lat):
+        t = torch.full((1,), float(sig[i % 28]), device=dev, dtype=torch.bfloat16)
+        out = model(hidden_states=lat, encoder_hidden_states=text, pooled_projections=pooled, timestep=t,
+                    img_ids=img_ids, txt_ids=txt_ids, guidance=guidance, return_dict=False)[0]
+        return euler_step(lat, out, float(sig[i % 28]), float(sig[i % 28 + 1]))
+
+    Cf, S = 3072, s_txt + side * side
+    gemm = 2.0 * S * Cf * Cf * (n_dual * (3 + 1 + 8) + n_single * (3 + 4 + 5))
+    name = (f"Flux-shape MMDiT denoise step: {n_dual} dual + {n_single} single blocks, hidden 3072, 24 heads x 128, "
+            f"{s_txt} text + {side * side} image tokens, batch 1 (guidance-distilled), random weights N(0,0.02)")
+    return model, step, lat0, name, gemm, (n_dual, n_single) == (19, 38)
+
+
+def wan_workload(torch, layers=None):
+    """BASELINE.json configs[3]: Wan2.1-14B shape, 40 blocks, B=2, 21x30x52 = 32760 video tokens, 512 text tokens."""
+    from vllm_omni_amd.blocks.wan import WanTransformer3DModel
+    from vllm_omni_amd.denoise import combine_cfg_noise, euler_step
+
+    n = 40 if layers is None else layers
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device("cuda"):
+            model = WanTransformer3DModel(num_layers=n)
+    finally:
+        torch.set_default_dtype(prev)
+    _init_synthetic(torch, model)
+    model.eval()
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cuda").manual_seed(1)
+    lat0 = torch.randn(1, 16, 21, 60, 104, device=dev, generator=g).bfloat16()
+    text = torch.randn(2, 512, 4096, device=dev, generator=g).bfloat16()
+
+    def step(i, lat):
+        t = torch.full((2,), 900.0 - 40.0 * i, device=dev)
+        out = model(lat.expand(2, -1, -1, -1, -1), t, text, return_dict=False)[0]
+        noise = combine_cfg_noise(out[0:1], out[1:2], 5.0, False)
+        return euler_step(lat, noise, 1.0 - 0.04 * i, 1.0 - 0.04 * (i + 1))
+
+    Cw, Fw, S, T = 5120, 13824, 32760, 512
+    gemm = n * 2.0 * 2 * (S * (3 * Cw * Cw + Cw * Cw + Cw * Cw + Cw * Cw + 2 * Cw * Fw) + T * 2 * Cw * Cw)
+    name = (f"Wan2.1-14B-shape video DiT denoise step: {n} blocks, hidden 5120, 40 heads x 128, FFN 13824, "
+            "21x30x52 = 32760 video tokens, 512 text tokens, CFG batch 2, random weights N(0,0.02)")
+    return model, step, lat0, name, gemm, n == 40
+
+
+def run_secondary(torch, kernels, args):
+    """Flux / Wan shapes: same timing protocol as the headline line, one JSON line, no CPU leg."""
+    make = flux_workload if args.workload == "flux" else wan_workload
+    model, step, lat, name, gemm_flop, valid = make(torch, None if args.blocks == LAYERS else args.blocks)
+    with torch.inference_mode(), AttnTimer(torch, kernels) as timer:
+        for i in range(args.warmup):
+            lat = step(i, lat)
+        torch.cuda.synchronize()
+        timer.active = True
+        t0 = time.perf_counter()
+        for i in range(args.warmup, args.warmup + args.steps):
+            lat = step(i, lat)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        timer.active = False
+    assert bool(torch.isfinite(lat.float()).all()), "non-finite latents"
+    ms, flop, n = timer.dominant()
+    tf = flop / ms / 1e9
+    attn_total = sum(timer.flops) / args.steps
+    print(json.dumps({
+        "metric": f"DiT denoise steps/s, {args.workload} shape (1 GPU)", "value": args.steps / elapsed,
+        "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": elapsed * 1e3 / args.steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic", "config": {"workload": name, "valid": valid},
+        "roofline": {"kernel": "attn_fwd (largest attention shape of the step)", "bound": "mfma", "achieved": tf,
+                     "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tf / PEAK_MFMA_BF16_TFLOPS,
+                     "traffic": None, "launches_timed": n, "avg_ms": ms, "flop_per_launch": flop},
+        "step_flop": {"gemm": gemm_flop, "attention": attn_total,
+                      "achieved_TFLOP/s": (gemm_flop + attn_total) / (elapsed / args.steps) / 1e12},
+    }))
 
 
 def _time_rot(torch, fns, iters=40, warmup=4):
@@ -196,12 +327,16 @@ def cpu_baseline(torch):
     vf, tf = oq.qwen_rope_freqs(cfg, *IMG_SHAPE, txt_len=S_TXT)
     with torch.inference_mode():
         oq.block_forward(w, 0, cfg, img[:, :256], txt, temb, vf[:256], tf)  # page in / warm threads
-        t0 = time.perf_counter()
-        oq.block_forward(w, 0, cfg, img, txt, temb, vf, tf)
-        dt = time.perf_counter() - t0
+        reps, t0 = 0, time.perf_counter()
+        while reps < 3 or (time.perf_counter() - t0 < 12.0 and reps < 12):  # about 12-20 s of CPU work
+            oq.block_forward(w, 0, cfg, img, txt, temb, vf, tf)
+            reps += 1
+        total = time.perf_counter() - t0
+    dt = total / reps
     return {"value": 1.0 / (dt * LAYERS), "unit": "steps/s", "cores": cores, "kind": "port",
             "sample": f"1 of {LAYERS} blocks at the full B=2, 4096+256-token shape, fp32 torch on {cores} threads, "
-                      f"{dt:.2f} s measured; step time extrapolated as {LAYERS} x block (stem/head < 0.5%)",
+                      f"{reps} repetitions in {total:.1f} s; step time extrapolated as {LAYERS} x block "
+                      "(stem/head < 0.5%)",
             "block_seconds": dt}
 
 
@@ -211,6 +346,8 @@ def main():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--blocks", type=int, default=LAYERS, help="debug only: fewer blocks (result is then marked invalid)")
+    ap.add_argument("--workload", choices=("qwen", "flux", "wan"), default="qwen",
+                    help="qwen = the headline metric; flux / wan = the other block families at their config shapes")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
     args = ap.parse_args()
@@ -231,6 +368,8 @@ def main():
     tuned = gemm_tuning.enable()  # hipBLASLt solution ids picked offline for this model's GEMM shapes
     torch.cuda.set_device(0)
     dev = torch.device("cuda:0")
+    if args.workload != "qwen":
+        return run_secondary(torch, kernels, args)
     model = build_model(torch, args.blocks)
     g = torch.Generator(device="cuda").manual_seed(1)
     latents = torch.randn(1, S_IMG, IN_CH, device=dev, generator=g).bfloat16()

@@ -73,18 +73,32 @@ int odit_attn_fwd(const void* q, const void* k, const void* v, void* o, const ui
                   const int64_t v_strides[3], const int64_t o_strides[3], float scale, int dtype,
                   void* stream);
 
-/* Same as odit_attn_fwd, with the output of the joint sequence split at a row: query rows
- * [0, q_split) are written to `o` (row r -> o row r), rows [q_split, Sq) to `o_tail` (row r -> o_tail
- * row r - q_split), each with its own (batch, seq, head) strides. Replaces the two slices
- * joint_hidden_states[:, :seq_len_txt] / [:, seq_len_txt:] of qwen_image_transformer.py:654-656, whose
- * strided views otherwise force a copy in front of each output projection. o_tail == NULL behaves
- * exactly like odit_attn_fwd.
+/* Extended form of odit_attn_fwd with two optional additions.
+ *
+ * Two outputs: with o_tail != NULL, query rows [0, q_split) are written to `o` (row r -> o row r) and
+ * rows [q_split, Sq) to `o_tail` (row r -> o_tail row r - q_split), each with its own (batch, seq,
+ * head) strides. Replaces the two slices joint_hidden_states[:, :seq_len_txt] / [:, seq_len_txt:] of
+ * qwen_image_transformer.py:654-656 (flux_transformer.py:217-219), whose strided views otherwise force
+ * a copy in front of each output projection.
+ *
+ * Scratch: `workspace` (device memory, 16-byte aligned, workspace_bytes >=
+ * odit_attn_fwd_workspace_bytes for the same shape, contents irrelevant before and after) lets the
+ * kernel cut the last, partly filled round of workgroups into key ranges that run side by side and
+ * are merged by a second launch; without it a shape whose workgroup count is not a multiple of what
+ * the GPU runs at once idles part of the GPU for a whole round. NULL = never split. Results with and
+ * without scratch agree to rounding (the merge re-associates the key sum); for given shapes and device
+ * the partition is fixed, so repeated calls are bit-identical. No counterpart in the reference.
+ *
+ * o_tail == NULL and workspace == NULL behaves exactly like odit_attn_fwd.
  */
-int odit_attn_fwd_split(const void* q, const void* k, const void* v, void* o, void* o_tail, int q_split,
-                        const uint8_t* key_mask, float* lse, int B, int Sq, int Sk, int H, int Hkv,
-                        int D, const int64_t q_strides[3], const int64_t k_strides[3],
-                        const int64_t v_strides[3], const int64_t o_strides[3],
-                        const int64_t o_tail_strides[3], float scale, int dtype, void* stream);
+int odit_attn_fwd_ex(const void* q, const void* k, const void* v, void* o, void* o_tail, int q_split,
+                     const uint8_t* key_mask, float* lse, int B, int Sq, int Sk, int H, int Hkv, int D,
+                     const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                     const int64_t o_strides[3], const int64_t o_tail_strides[3], float scale, int dtype,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* Scratch bytes odit_attn_fwd_ex can use for this shape on the current device (0 = none needed). */
+size_t odit_attn_fwd_workspace_bytes(int B, int Sq, int Sk, int H, int D);
 
 /* ---------------------------------------------------------------------------------------------
  * K2  fused QK-RMSNorm + rotary embedding + scatter into the joint [txt;img] sequence.

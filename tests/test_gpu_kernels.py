@@ -391,6 +391,75 @@ def test_attention_split_output_equals_slices(gpu, monkeypatch, variant, split):
         kernels.attn_fwd(q, k, v, 0.09, split=S + 1)
 
 
+KEY_SPLIT_SHAPES = [
+    # B, Sq, Sk, H, Hkv, D: few workgroups, many key tiles -> the last (only) round is cut along the keys
+    (1, 300, 1100, 3, 3, 128),    # ragged queries and keys; ranges of 10 + 8 tiles
+    (2, 64, 4352, 8, 8, 64),      # one q block per head, 68 tiles in up to 8 ranges
+    (1, 130, 2048, 4, 2, 128),    # grouped KV heads, second q block almost empty
+    (1, 1, 1030, 1, 1, 128),      # a single query row, 17 tiles in two ranges
+]
+
+
+@pytest.mark.parametrize("variant", ["34", "38"])
+@pytest.mark.parametrize("shape", KEY_SPLIT_SHAPES)
+def test_attention_key_split_tail(gpu, monkeypatch, variant, shape):
+    """The launch that cuts its last round of workgroups into key ranges and merges them must agree with
+    the single-pass launch and with the oracle: plain, with a key mask, with LSE and with two outputs."""
+    from vllm_omni_amd import _lib, kernels
+
+    monkeypatch.setenv("ODIT_ATTN_VARIANT", variant)
+    B, Sq, Sk, H, Hkv, D = shape
+    assert _lib.load().odit_attn_fwd_workspace_bytes(B, Sq, Sk, H, D) > 0, "shape does not exercise the key split"
+    q, k, v = _attn_inputs(B, Sq, Sk, H, Hkv, D, seed=5)
+    scale = 1.0 / math.sqrt(D)
+    print(f"attn key-split variant={variant} shape={shape}", flush=True)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    one, lse1 = kernels.attn_fwd(qg, kg, vg, scale, return_lse=True, use_workspace=False)
+    two, lse2 = kernels.attn_fwd(qg, kg, vg, scale, return_lse=True)
+    torch.cuda.synchronize()
+    want = ops.sdpa(q.float(), k.float(), v.float(), scale)
+    _close(two, want, atol=2e-2, rtol=2e-2, what="key-split attention vs oracle")
+    assert _cosine(two, want) >= 0.9995
+    _close(two, one, atol=8e-3, rtol=8e-3, what="key-split vs single pass")   # one bf16 ulp of O(1) values
+    _close(lse2, lse1, atol=1e-4, rtol=1e-5, what="lse")
+    again = kernels.attn_fwd(qg, kg, vg, scale)
+    assert torch.equal(again, two), "the partition is fixed: repeated calls are bit-identical"
+    # key mask: scattered, plus one whole key range excluded (its partial must get weight zero)
+    g = torch.Generator().manual_seed(8)
+    m = torch.rand(B, Sk, generator=g) > 0.3
+    m[:, : min(Sk // 2, 640)] = False
+    m[:, -1] = True
+    got_m = kernels.attn_fwd(qg, kg, vg, scale, key_mask=m.to(gpu))
+    _close(got_m, ops.sdpa(q.float(), k.float(), v.float(), scale, key_mask=m), atol=2e-2, rtol=2e-2,
+           what="key-split with mask")
+    if Sq > 2:
+        cut = Sq // 3
+        head, tail = kernels.attn_fwd(qg, kg, vg, scale, split=cut)
+        assert torch.equal(head, two[:, :cut]) and torch.equal(tail, two[:, cut:])
+
+
+def test_attention_workspace_too_small_is_an_error(gpu):
+    from vllm_omni_amd import _lib
+
+    lib = _lib.load()
+    B, Sq, Sk, H, D = 1, 128, 2048, 2, 128
+    need = lib.odit_attn_fwd_workspace_bytes(B, Sq, Sk, H, D)
+    assert need > 0
+    q = torch.zeros(B, Sq, H, D, device=gpu, dtype=torch.bfloat16)
+    o = torch.empty_like(q)
+    ws = torch.empty(need, device=gpu, dtype=torch.uint8)
+    st = _lib.i64_array(q.stride()[:3])
+    rc = lib.odit_attn_fwd_ex(q.data_ptr(), q.data_ptr(), q.data_ptr(), o.data_ptr(), None, 0, None, None,
+                              B, Sq, Sk if False else Sq, H, H, D, st, st, st, st, None, 0.1, 0, ws.data_ptr(), 16, None)
+    assert rc == 0  # Sk = 128: nothing to split, any workspace size is fine
+    k = torch.zeros(B, Sk, H, D, device=gpu, dtype=torch.bfloat16)
+    sk = _lib.i64_array(k.stride()[:3])
+    rc = lib.odit_attn_fwd_ex(q.data_ptr(), k.data_ptr(), k.data_ptr(), o.data_ptr(), None, 0, None, None,
+                              B, Sq, Sk, H, H, D, st, sk, sk, st, None, 0.1, 0, ws.data_ptr(), need - 1, None)
+    assert rc == -4 and b"workspace" in lib.odit_last_error()
+    torch.cuda.synchronize()
+
+
 def test_attention_fp32_goes_to_sdpa(gpu):
     from vllm_omni_amd.attention.layer import Attention
 

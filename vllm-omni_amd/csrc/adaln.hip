@@ -38,7 +38,10 @@ __device__ __forceinline__ void load_params(const TP* p, float fill, float (&dst
 // read-once / write-once pass near the HBM rate. The two LayerNorm moments are taken in one sweep
 // about the row's first element (a shift every wave can fetch by itself) and combined across the W
 // waves through 2*W floats of LDS.
-template <typename T, typename TM, int W, int NVL, bool REF_ROUND>
+// PLAIN = the per-block call of the DiT step (shift and scale given, no per-token index, no LayerNorm
+// affine): the optional operands cost registers and address arithmetic even when absent, and this
+// pass lives on how many rows a CU keeps in flight.
+template <typename T, typename TM, int W, int NVL, bool REF_ROUND, bool PLAIN>
 __global__ __launch_bounds__(W * 64) void adaln_rows_kernel(
     const T* __restrict__ x, T* __restrict__ out, const TM* __restrict__ shift,
     const TM* __restrict__ scale, const int32_t* __restrict__ index,
@@ -46,9 +49,9 @@ __global__ __launch_bounds__(W * 64) void adaln_rows_kernel(
     int64_t xs_b, int64_t xs_s, int64_t os_b, int64_t os_s, int64_t mod_stride_b, float eps) {
   constexpr int EPV = Vec16<T>::N;
   const int tid = threadIdx.x;
-  const int64_t row = blockIdx.x;
-  const int b = static_cast<int>(row / S);
-  const int s = static_cast<int>(row - static_cast<int64_t>(b) * S);
+  const unsigned row = blockIdx.x;  // the launcher keeps B*S below 2^31
+  const int b = static_cast<int>(row / static_cast<unsigned>(S));
+  const int s = static_cast<int>(row - static_cast<unsigned>(b) * static_cast<unsigned>(S));
   const T* xr = x + b * xs_b + s * xs_s;
   T* orow = out + b * os_b + s * os_s;
 
@@ -56,7 +59,8 @@ __global__ __launch_bounds__(W * 64) void adaln_rows_kernel(
 #pragma unroll
   for (int i = 0; i < NVL; ++i) {
     const int c0 = (i * (W * 64) + tid) * EPV;
-    raw[i] = c0 < C ? load_raw(xr + c0) : u32x4{0u, 0u, 0u, 0u};
+    // the row is consumed once: keep it out of the way of the [B,C] modulation rows in L2
+    raw[i] = c0 < C ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xr + c0)) : u32x4{0u, 0u, 0u, 0u};
   }
   const float k0 = to_float(xr[0]);  // same address for the whole workgroup: one broadcast load
   float s1 = 0.f, s2 = 0.f;
@@ -88,9 +92,9 @@ __global__ __launch_bounds__(W * 64) void adaln_rows_kernel(
   const float rstd = rsqrtf(fmaxf(s2 * inv_c - m1 * m1, 0.f) + eps);
 
   int mrow = b;
-  if (index != nullptr && index[static_cast<int64_t>(b) * S + s] != 0) mrow = b + B;
-  const TM* sh = shift ? shift + mrow * mod_stride_b : nullptr;
-  const TM* sc = scale ? scale + mrow * mod_stride_b : nullptr;
+  if (!PLAIN && index != nullptr && index[static_cast<int64_t>(b) * S + s] != 0) mrow = b + B;
+  const TM* sh = (PLAIN || shift) ? shift + mrow * mod_stride_b : nullptr;
+  const TM* sc = (PLAIN || scale) ? scale + mrow * mod_stride_b : nullptr;
 
 #pragma unroll
   for (int i = 0; i < NVL; ++i) {
@@ -99,14 +103,16 @@ __global__ __launch_bounds__(W * 64) void adaln_rows_kernel(
       float scl_v[EPV], shf_v[EPV], lw_v[EPV], lb_v[EPV];
       load_params<TM, EPV>(sc ? sc + c0 : nullptr, 0.f, scl_v);
       load_params<TM, EPV>(sh ? sh + c0 : nullptr, 0.f, shf_v);
-      load_params<float, EPV>(ln_w ? ln_w + c0 : nullptr, 1.f, lw_v);
-      load_params<float, EPV>(ln_b ? ln_b + c0 : nullptr, 0.f, lb_v);
+      if (!PLAIN) {
+        load_params<float, EPV>(ln_w ? ln_w + c0 : nullptr, 1.f, lw_v);
+        load_params<float, EPV>(ln_b ? ln_b + c0 : nullptr, 0.f, lb_v);
+      }
       float r[EPV];
 #pragma unroll
       for (int j = 0; j < EPV; ++j) {
         float y = (Raw<T>::get(raw[i], j) - mean) * rstd;
-        if (ln_w) y *= lw_v[j];
-        if (ln_b) y += lb_v[j];
+        if (!PLAIN && ln_w) y *= lw_v[j];
+        if (!PLAIN && ln_b) y += lb_v[j];
         if (REF_ROUND) {
           // torch path: LN -> T, (1 + scale) -> T, product -> T, sum -> T
           r[j] = round_to<T>(round_to<T>(y) * round_to<T>(1.f + scl_v[j])) + shf_v[j];
@@ -177,11 +183,15 @@ static int launch_adaln(const void* x, void* out, const void* shift, const void*
                       aligned16(shift) && aligned16(scale) && mod_stride_b % EPM == 0 &&
                       aligned16(ln_w) && aligned16(ln_b);
   const int nvec = (C + EPV - 1) / EPV;  // 16-byte vectors per row
+  const bool plain = shift && scale && !index && !ln_w && !ln_b;
+#define ODIT_ADALN_LAUNCH(WW, NVLL, PL)                                                            \
+  hipLaunchKernelGGL((adaln_rows_kernel<T, TM, WW, NVLL, REF_ROUND, PL>),                          \
+                     dim3(static_cast<unsigned>(rows)), dim3(WW * 64), 0, stream,                  \
+                     static_cast<const T*>(x), static_cast<T*>(out), static_cast<const TM*>(shift), \
+                     static_cast<const TM*>(scale), index, ln_w, ln_b, B, S, C, xs[0], xs[1],      \
+                     os[0], os[1], mod_stride_b, eps)
 #define ODIT_ADALN_CASE(WW, NVLL)                                                                  \
-  hipLaunchKernelGGL((adaln_rows_kernel<T, TM, WW, NVLL, REF_ROUND>), dim3(static_cast<unsigned>(rows)), \
-                     dim3(WW * 64), 0, stream, static_cast<const T*>(x), static_cast<T*>(out),     \
-                     static_cast<const TM*>(shift), static_cast<const TM*>(scale), index, ln_w,    \
-                     ln_b, B, S, C, xs[0], xs[1], os[0], os[1], mod_stride_b, eps)
+  do { if (plain) ODIT_ADALN_LAUNCH(WW, NVLL, true); else ODIT_ADALN_LAUNCH(WW, NVLL, false); } while (0)
   if (vec_ok && nvec <= 8 * 64 * 2 && rows <= 0x7fffffffll) {
     if (nvec <= 64) ODIT_ADALN_CASE(1, 1);
     else if (nvec <= 128) ODIT_ADALN_CASE(2, 1);
@@ -198,6 +208,7 @@ static int launch_adaln(const void* x, void* out, const void* shift, const void*
                        ln_b, B, S, C, xs[0], xs[1], os[0], os[1], mod_stride_b, eps);
   }
 #undef ODIT_ADALN_CASE
+#undef ODIT_ADALN_LAUNCH
   return check_launch("odit_adaln_modulate");
 }
 

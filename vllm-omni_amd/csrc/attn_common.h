@@ -11,6 +11,7 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_v;
 typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2_v;
 typedef uint32_t u32x4_v __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_v __attribute__((ext_vector_type(2)));
+typedef float f32x4_v __attribute__((ext_vector_type(4)));
 typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_v;
 typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_v;
 
@@ -46,6 +47,11 @@ struct AttnParams {
   // optional second output: query rows >= q_split are written to o_tail[row - q_split]
   void* o_tail; int q_split;
   int64_t ts_b, ts_s, ts_h;
+  // key-split tail (attn_fwd_dma.hip): workgroup ids < n_full own a whole (q-block, head, batch) unit;
+  // the remaining units are cut into key_chunks ranges of tiles_per_chunk key tiles each, one
+  // workgroup per range, which leave unnormalised partial results in `ws` for the merge kernel
+  int n_full, key_chunks, tiles_per_chunk;
+  float* ws;
 };
 
 // address of output row `row` of (batch b, head h): head of the joint sequence in `o`, tail in `o_tail`
@@ -69,6 +75,11 @@ __device__ __forceinline__ int xcd_remap(int bid, int total) {
 
 // software-pipelined kernel with direct global->LDS tile loads (attn_fwd_dma.hip); returns
 // ODIT_ENOTSUP when the tensors cannot be addressed with 32-bit buffer offsets
-int launch_attn_dma(AttnParams& p, int dtype, int D, int nw, hipStream_t stream);
+// `ws` (may be null) is scratch for the key-split tail; see attn_dma_workspace_bytes.
+int launch_attn_dma(AttnParams& p, int dtype, int D, int nw, hipStream_t stream, void* ws, size_t ws_bytes);
+
+// bytes of scratch with which launch_attn_dma can split the last, partly filled round of workgroups
+// along the keys (0 when this shape gains nothing from it)
+size_t attn_dma_workspace_bytes(int B, int Sq, int Sk, int H, int D, int nw);
 
 }  // namespace odit

@@ -614,35 +614,48 @@ static int dispatch_attn(AttnParams& p, int variant, hipStream_t stream) {
 
 }  // namespace odit
 
-extern "C" int odit_attn_fwd_split(const void* q, const void* k, const void* v, void* o, void* o_tail,
-                                   int q_split, const uint8_t* key_mask, float* lse, int B, int Sq,
-                                   int Sk, int H, int Hkv, int D, const int64_t q_strides[3],
-                                   const int64_t k_strides[3], const int64_t v_strides[3],
-                                   const int64_t o_strides[3], const int64_t o_tail_strides[3],
-                                   float scale, int dtype, void* stream);
+static int attn_variant() {
+  int variant = 34;
+  if (const char* e = getenv("ODIT_ATTN_VARIANT")) variant = atoi(e);
+  return variant;
+}
+
+extern "C" int odit_attn_fwd_ex(const void* q, const void* k, const void* v, void* o, void* o_tail,
+                                int q_split, const uint8_t* key_mask, float* lse, int B, int Sq, int Sk,
+                                int H, int Hkv, int D, const int64_t q_strides[3],
+                                const int64_t k_strides[3], const int64_t v_strides[3],
+                                const int64_t o_strides[3], const int64_t o_tail_strides[3], float scale,
+                                int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 extern "C" int odit_attn_fwd(const void* q, const void* k, const void* v, void* o,
                              const uint8_t* key_mask, float* lse, int B, int Sq, int Sk, int H,
                              int Hkv, int D, const int64_t q_strides[3], const int64_t k_strides[3],
                              const int64_t v_strides[3], const int64_t o_strides[3], float scale,
                              int dtype, void* stream) {
-  return odit_attn_fwd_split(q, k, v, o, nullptr, 0, key_mask, lse, B, Sq, Sk, H, Hkv, D, q_strides,
-                             k_strides, v_strides, o_strides, nullptr, scale, dtype, stream);
+  return odit_attn_fwd_ex(q, k, v, o, nullptr, 0, key_mask, lse, B, Sq, Sk, H, Hkv, D, q_strides, k_strides,
+                          v_strides, o_strides, nullptr, scale, dtype, nullptr, 0, stream);
 }
 
-extern "C" int odit_attn_fwd_split(const void* q, const void* k, const void* v, void* o, void* o_tail,
-                                   int q_split, const uint8_t* key_mask, float* lse, int B, int Sq,
-                                   int Sk, int H, int Hkv, int D, const int64_t q_strides[3],
-                                   const int64_t k_strides[3], const int64_t v_strides[3],
-                                   const int64_t o_strides[3], const int64_t o_tail_strides[3],
-                                   float scale, int dtype, void* stream) {
+extern "C" size_t odit_attn_fwd_workspace_bytes(int B, int Sq, int Sk, int H, int D) {
+  const int variant = attn_variant();
+  if (variant != 34 && variant != 38) return 0;
+  if (D != 64 && D != 128) return 0;
+  return odit::attn_dma_workspace_bytes(B, Sq, Sk, H, D, variant == 38 ? 8 : 4);
+}
+
+extern "C" int odit_attn_fwd_ex(const void* q, const void* k, const void* v, void* o, void* o_tail,
+                                int q_split, const uint8_t* key_mask, float* lse, int B, int Sq, int Sk,
+                                int H, int Hkv, int D, const int64_t q_strides[3],
+                                const int64_t k_strides[3], const int64_t v_strides[3],
+                                const int64_t o_strides[3], const int64_t o_tail_strides[3], float scale,
+                                int dtype, void* workspace, size_t workspace_bytes, void* stream) {
   using namespace odit;
   if (o_tail != nullptr) {
-    ODIT_CHECK_ARG(o_tail_strides != nullptr, "odit_attn_fwd_split: o_tail given without strides");
-    ODIT_CHECK_ARG(q_split >= 0 && q_split <= Sq, "odit_attn_fwd_split: q_split=%d outside [0, Sq=%d]", q_split, Sq);
+    ODIT_CHECK_ARG(o_tail_strides != nullptr, "odit_attn_fwd_ex: o_tail given without strides");
+    ODIT_CHECK_ARG(q_split >= 0 && q_split <= Sq, "odit_attn_fwd_ex: q_split=%d outside [0, Sq=%d]", q_split, Sq);
     ODIT_CHECK_ARG(aligned16(o_tail) && o_tail_strides[0] % 8 == 0 && o_tail_strides[1] % 8 == 0 &&
                        o_tail_strides[2] % 8 == 0,
-                   "odit_attn_fwd_split: o_tail must be 16-byte aligned with strides multiple of 8");
+                   "odit_attn_fwd_ex: o_tail must be 16-byte aligned with strides multiple of 8");
   }
   ODIT_CHECK_ARG(q && k && v && o, "odit_attn_fwd: q/k/v/o must not be null");
   ODIT_CHECK_ARG(q_strides && k_strides && v_strides && o_strides, "odit_attn_fwd: null strides");
@@ -679,11 +692,12 @@ extern "C" int odit_attn_fwd_split(const void* q, const void* k, const void* v, 
   p.o_tail = o_tail; p.q_split = q_split;
   p.ts_b = o_tail ? o_tail_strides[0] : 0; p.ts_s = o_tail ? o_tail_strides[1] : 0; p.ts_h = o_tail ? o_tail_strides[2] : 0;
 
-  int variant = 34;
-  if (const char* e = getenv("ODIT_ATTN_VARIANT")) variant = atoi(e);
+  p.n_full = 0; p.key_chunks = 1; p.tiles_per_chunk = 0; p.ws = nullptr;
+
+  int variant = attn_variant();
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (variant == 38 || variant == 34) {
-    const int rc = launch_attn_dma(p, dtype, D, variant == 38 ? 8 : 4, st);
+    const int rc = launch_attn_dma(p, dtype, D, variant == 38 ? 8 : 4, st, workspace, workspace_bytes);
     if (rc != ODIT_ENOTSUP) return rc;
     variant = 28;  // tensors too large for 32-bit buffer offsets: pointer-addressed kernel
   }

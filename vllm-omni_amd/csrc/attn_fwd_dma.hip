@@ -27,7 +27,12 @@ typedef short s16x8_d __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) s16x4_d* lds_s16x4_p;
 typedef __attribute__((address_space(3))) void* lds_void_p;
 
-template <typename T, int D, int NW>
+// TAIL = false: workgroup i owns unit i (a q block of one head of one batch row), all keys.
+// TAIL = true:  launched after the full rounds for the units that are left over: workgroup i owns key
+//               tiles [jt0, n_tiles) of unit n_full + i / key_chunks and leaves an unnormalised partial
+//               result in scratch for attn_merge_kernel. A separate instantiation, so the extra
+//               bookkeeping cannot disturb the register allocation of the main kernel.
+template <typename T, int D, int NW, bool TAIL>
 __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const AttnParams p) {
   using M = Mma<T>;
   using frag = typename M::frag;
@@ -47,7 +52,16 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   char* const Kb = lds;
   char* const Vb = lds + 2 * TILEB;
 
-  const int pid = xcd_remap(blockIdx.x, p.total_blocks);
+  const int n_tiles_all = (p.Sk + BN - 1) / BN;
+  int pid, jt0 = 0, n_tiles = n_tiles_all;
+  const int part = blockIdx.x;
+  if constexpr (!TAIL) {
+    pid = xcd_remap(blockIdx.x, p.n_full);
+  } else {  // this workgroup covers key tiles [jt0, n_tiles) of unit pid (jt0 is even)
+    pid = p.n_full + part / p.key_chunks;
+    jt0 = (part % p.key_chunks) * p.tiles_per_chunk;
+    n_tiles = jt0 + p.tiles_per_chunk < n_tiles_all ? jt0 + p.tiles_per_chunk : n_tiles_all;
+  }
   const int qb = pid % p.n_qblocks;
   const int bh = pid / p.n_qblocks;
   const int h = bh % p.H;
@@ -107,7 +121,6 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
     for (int e = 0; e < 16; ++e) o[dt][e] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  const int n_tiles = (p.Sk + BN - 1) / BN;
   const float c = p.scale_log2;
   const uint8_t* mrow = p.mask ? p.mask + static_cast<int64_t>(b) * p.Sk : nullptr;
 
@@ -287,26 +300,45 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
     if (has_next) settle_max(mx);
   };
 
-  // ---- prologue ----
-  dma_tile(krsrc, kvoff, 0, Kb);
-  dma_tile(vrsrc, vvoff, 0, Vb);
-  if (n_tiles > 1) dma_tile(krsrc, kvoff, k_tile_step, Kb + TILEB);
+  // ---- prologue (jt0 is even, so tile j always lives in buffer j & 1) ----
+  dma_tile(krsrc, kvoff, static_cast<uint32_t>(jt0) * k_tile_step, Kb);
+  dma_tile(vrsrc, vvoff, static_cast<uint32_t>(jt0) * v_tile_step, Vb);
+  if (jt0 + 1 < n_tiles) dma_tile(krsrc, kvoff, static_cast<uint32_t>(jt0 + 1) * k_tile_step, Kb + TILEB);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   f32x16_v sa[2], sb[2];
   qk_plain(Kb, sa);
   {
-    const float t = mask_and_max(0, sa);
+    const float t = mask_and_max(jt0, sa);
     settle_max(fmaxf(t, __shfl_xor(t, 32, 64)));
   }
 
-  for (int j = 0; j < n_tiles; j += 2) {
+  for (int j = jt0; j < n_tiles; j += 2) {
     tile(j, sa, sb);
     if (j + 1 < n_tiles) tile(j + 1, sb, sa);
   }
 
   // ---- epilogue ----
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  if constexpr (TAIL) {
+    // partial result of a key range: unnormalised O (fp32, [BM][D] per part) and the row's (m, l)
+    float* wo = p.ws + (static_cast<int64_t>(part) * BM + wave * 32 + l32) * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4_v w4;
+        w4.x = o[dt][g * 4 + 0]; w4.y = o[dt][g * 4 + 1]; w4.z = o[dt][g * 4 + 2]; w4.w = o[dt][g * 4 + 3];
+        *reinterpret_cast<f32x4_v*>(wo + dt * 32 + g * 8 + hh * 4) = w4;
+      }
+    if (hh == 0) {
+      float* ml = p.ws + static_cast<int64_t>(gridDim.x) * BM * D +
+                  (static_cast<int64_t>(part) * BM + wave * 32 + l32) * 2;
+      ml[0] = m_run;
+      ml[1] = l_tot;
+    }
+    return;
+  }
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   const int row = q0 + l32;
   if (row < p.Sq) {
@@ -327,28 +359,149 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   }
 }
 
+// Merge of the key-split tail: one wavefront per query row adds the row's key_chunks partial results,
+//   O = sum_c 2^((m_c - m) c) O_c / sum_c 2^((m_c - m) c) l_c,   m = max_c m_c,
+// and writes the row (and its log-sum-exp) where the unsplit kernel would have.
+template <typename T, int D, int BM>
+__global__ __launch_bounds__(256) void attn_merge_kernel(const AttnParams p, int n_parts) {
+  using M = Mma<T>;
+  const int lane = threadIdx.x & 63;
+  const int64_t gr = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);  // (tail unit, row in unit)
+  const int unit = static_cast<int>(gr / BM), r = static_cast<int>(gr % BM);
+  if (unit >= n_parts / p.key_chunks) return;
+  const int pid = p.n_full + unit;
+  const int qb = pid % p.n_qblocks, bh = pid / p.n_qblocks;
+  const int h = bh % p.H, b = bh / p.H;
+  const int row = qb * BM + r;
+  if (row >= p.Sq) return;
+  const float* ml = p.ws + static_cast<int64_t>(n_parts) * BM * D;
+  float m = -INFINITY;
+  for (int cidx = 0; cidx < p.key_chunks; ++cidx)
+    m = fmaxf(m, ml[(static_cast<int64_t>(unit * p.key_chunks + cidx) * BM + r) * 2]);
+  const float m_safe = m == -INFINITY ? 0.f : m;
+  constexpr int EPL = D / 64;  // consecutive elements per lane
+  float acc[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
+  float l = 0.f;
+  for (int cidx = 0; cidx < p.key_chunks; ++cidx) {
+    const int64_t pr = static_cast<int64_t>(unit * p.key_chunks + cidx) * BM + r;
+    const float wgt = __builtin_amdgcn_exp2f((ml[pr * 2] - m_safe) * p.scale_log2);  // 0 for an empty range
+    l = fmaf(wgt, ml[pr * 2 + 1], l);
+    const float* src = p.ws + pr * D + lane * EPL;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) acc[e] = fmaf(wgt, src[e], acc[e]);
+  }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  T* op = out_row_ptr<T>(p, b, h, row) + lane * EPL;
+  if constexpr (EPL == 2) {
+    *reinterpret_cast<uint32_t*>(op) = M::pack2(acc[0] * inv, acc[1] * inv);
+  } else {
+    op[0] = from_float<T>(acc[0] * inv);
+  }
+  if (p.lse != nullptr && lane == 0)
+    p.lse[(static_cast<int64_t>(b) * p.H + h) * p.Sq + row] = l > 0.f ? m * p.scale + __logf(l) : -INFINITY;
+}
+
+// How the last round of workgroups is cut along the keys. `slots` workgroups run at once; after
+// `units / slots` full rounds, `rem` units are left: when they would leave at least half the slots
+// idle, each is cut into as many key ranges as fit the idle slots (ranges of an even number of tiles,
+// at least kMinTilesPerChunk), so the tail takes 1/key_chunks of a round instead of a whole one.
+struct TailPlan { int rem, key_chunks, tiles_per_chunk; };
+constexpr int kMinTilesPerChunk = 8;
+constexpr int kMaxKeyChunks = 16;
+
+static int device_slots(int nw) {
+  static int cus[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256 * (8 / nw);
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev] = n;
+  }
+  return cus[dev] * (8 / nw);
+}
+
+static TailPlan plan_tail(int64_t units, int n_tiles, int slots) {
+  TailPlan t{0, 1, n_tiles};
+  const int rem = static_cast<int>(units % slots);
+  if (rem == 0 || 2 * rem > slots) return t;
+  int kc = slots / rem;
+  if (kc > kMaxKeyChunks) kc = kMaxKeyChunks;
+  if (kc > n_tiles / kMinTilesPerChunk) kc = n_tiles / kMinTilesPerChunk;
+  if (kc < 2) return t;
+  int tpc = (n_tiles + kc - 1) / kc;
+  tpc += tpc & 1;                      // even, so a tile's LDS buffer is still (tile index & 1)
+  kc = (n_tiles + tpc - 1) / tpc;      // drop ranges that the rounding emptied
+  if (kc < 2) return t;
+  t.rem = rem; t.key_chunks = kc; t.tiles_per_chunk = tpc;
+  return t;
+}
+
+static size_t tail_ws_bytes(const TailPlan& t, int bm, int D) {
+  return t.rem == 0 ? 0 : static_cast<size_t>(t.rem) * t.key_chunks * bm * (D + 2) * sizeof(float);
+}
+
 template <typename T, int D, int NW>
-static int launch_dma(AttnParams& p, hipStream_t stream) {
+static int launch_dma(AttnParams& p, hipStream_t stream, void* ws, size_t ws_bytes) {
   constexpr int BM = NW * 32;
   p.n_qblocks = (p.Sq + BM - 1) / BM;
   const int64_t total = static_cast<int64_t>(p.n_qblocks) * p.H * p.B;
-  if (total > 0x7fffffffll) {
+  if (total > 0x3fffffffll) {
     set_error("odit_attn_fwd: grid of %lld workgroups is too large", static_cast<long long>(total));
     return ODIT_EINVAL;
   }
   p.total_blocks = static_cast<int>(total);
-  hipLaunchKernelGGL((attn_fwd_dma_kernel<T, D, NW>), dim3(p.total_blocks), dim3(NW * 64), 0, stream, p);
-  return check_launch("odit_attn_fwd");
+  p.n_full = p.total_blocks; p.key_chunks = 1; p.tiles_per_chunk = 0; p.ws = nullptr;
+  TailPlan t{0, 1, 0};
+  if (ws != nullptr) {
+    t = plan_tail(total, (p.Sk + 63) / 64, device_slots(NW));
+    if (t.rem > 0) {
+      if (ws_bytes < tail_ws_bytes(t, BM, D)) {
+        set_error("odit_attn_fwd: workspace of %zu bytes given, %zu needed", ws_bytes, tail_ws_bytes(t, BM, D));
+        return ODIT_EWORKSPACE;
+      }
+      if ((reinterpret_cast<uintptr_t>(ws) & 15) != 0) {
+        set_error("odit_attn_fwd: workspace must be 16-byte aligned");
+        return ODIT_EINVAL;
+      }
+      p.n_full = p.total_blocks - t.rem; p.key_chunks = t.key_chunks; p.tiles_per_chunk = t.tiles_per_chunk;
+      p.ws = static_cast<float*>(ws);
+    }
+  }
+  const int n_parts = t.rem * t.key_chunks;
+  int rc = ODIT_OK;
+  if (p.n_full > 0) {
+    hipLaunchKernelGGL((attn_fwd_dma_kernel<T, D, NW, false>), dim3(p.n_full), dim3(NW * 64), 0, stream, p);
+    rc = check_launch("odit_attn_fwd");
+  }
+  if (rc != ODIT_OK || n_parts == 0) return rc;
+  // stream order puts these after the full rounds, when every slot is free again
+  hipLaunchKernelGGL((attn_fwd_dma_kernel<T, D, NW, true>), dim3(n_parts), dim3(NW * 64), 0, stream, p);
+  rc = check_launch("odit_attn_fwd (key-split tail)");
+  if (rc != ODIT_OK) return rc;
+  const int64_t rows = static_cast<int64_t>(t.rem) * BM;
+  hipLaunchKernelGGL((attn_merge_kernel<T, D, BM>), dim3(static_cast<unsigned>((rows + 3) / 4)), dim3(256), 0,
+                     stream, p, n_parts);
+  return check_launch("odit_attn_fwd (merge)");
 }
 
-int launch_attn_dma(AttnParams& p, int dtype, int D, int nw, hipStream_t stream) {
+size_t attn_dma_workspace_bytes(int B, int Sq, int Sk, int H, int D, int nw) {
+  if (B <= 0 || Sq <= 0 || Sk <= 0 || H <= 0) return 0;
+  const int bm = nw * 32;
+  const int64_t units = static_cast<int64_t>((Sq + bm - 1) / bm) * H * B;
+  return tail_ws_bytes(plan_tail(units, (Sk + 63) / 64, device_slots(nw)), bm, D);
+}
+
+int launch_attn_dma(AttnParams& p, int dtype, int D, int nw, hipStream_t stream, void* ws, size_t ws_bytes) {
   // 32-bit buffer offsets: the whole key range of one (batch, head) must be addressable
   const int64_t k_span = (static_cast<int64_t>(p.Sk) + 64) * p.ks_s * 2;
   const int64_t v_span = (static_cast<int64_t>(p.Sk) + 64) * p.vs_s * 2;
   if (k_span >= (1ll << 31) || v_span >= (1ll << 31) || p.ks_s < 0 || p.vs_s < 0) return ODIT_ENOTSUP;
 #define ODIT_DMA_GO(T)                                                                     \
-  if (D == 128) return nw == 8 ? launch_dma<T, 128, 8>(p, stream) : launch_dma<T, 128, 4>(p, stream); \
-  return nw == 8 ? launch_dma<T, 64, 8>(p, stream) : launch_dma<T, 64, 4>(p, stream);
+  if (D == 128) return nw == 8 ? launch_dma<T, 128, 8>(p, stream, ws, ws_bytes) : launch_dma<T, 128, 4>(p, stream, ws, ws_bytes); \
+  return nw == 8 ? launch_dma<T, 64, 8>(p, stream, ws, ws_bytes) : launch_dma<T, 64, 4>(p, stream, ws, ws_bytes);
   if (dtype == ODIT_BF16) { ODIT_DMA_GO(bf16_t) }
   ODIT_DMA_GO(f16_t)
 #undef ODIT_DMA_GO

@@ -186,10 +186,10 @@ __global__ __launch_bounds__(256) void qknorm_row_kernel(
   constexpr int EPV = Vec16<T>::N;
   const int lane = threadIdx.x & 63;
   const int kind = blockIdx.y == 0 ? 0 : (blockIdx.y == 1 && k_in != nullptr ? 1 : 2);
-  const int64_t tok = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (tok >= static_cast<int64_t>(B) * S) return;  // wave-uniform
-  const int b = static_cast<int>(tok / S);
-  const int s = static_cast<int>(tok - static_cast<int64_t>(b) * S);
+  const unsigned tok = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);  // B*S < 2^31 (checked by the caller)
+  if (tok >= static_cast<unsigned>(B) * static_cast<unsigned>(S)) return;  // wave-uniform
+  const int b = static_cast<int>(tok / static_cast<unsigned>(S));
+  const int s = static_cast<int>(tok - static_cast<unsigned>(b) * static_cast<unsigned>(S));
   const T* in = (kind == 0 ? q_in : (kind == 1 ? k_in : v_in)) + b * is_b + s * is_s;
   T* out = (kind == 0 ? q_out : (kind == 1 ? k_out : v_out)) +
            (static_cast<int64_t>(b) * S_total + out_seq_offset + s) * HD;
@@ -368,6 +368,7 @@ extern "C" int odit_qknorm_rope(const void* q_in, const void* k_in, const void* 
     return ODIT_ENOTSUP;
   }
   if (B == 0 || S == 0) return ODIT_OK;
+  ODIT_CHECK_ARG(static_cast<int64_t>(B) * S <= 0x7fffffffll, "odit_qknorm_rope: B*S exceeds 2^31 - 1 rows");
   QkArgs a;
   a.q_in = q_in; a.k_in = k_in; a.v_in = v_in;
   a.q_out = q_out; a.k_out = k_out; a.v_out = v_out;

@@ -70,12 +70,14 @@ def attn_fwd(
     key_mask: torch.Tensor | None = None,
     return_lse: bool = False,
     split: int | None = None,
+    use_workspace: bool = True,
 ):
     """softmax(q k^T * scale) v for q [B,Sq,H,D], k/v [B,Sk,Hkv,D] (BSHD, bf16/fp16).
 
     key_mask: optional [B,Sk] bool/uint8, False/0 = key excluded. Returns o [B,Sq,H,D]
     (and lse [B,H,Sq] float32 when return_lse). With ``split`` = s the output comes back as two dense
-    tensors (o[:, :s], o[:, s:]) written directly by the kernel.
+    tensors (o[:, :s], o[:, s:]) written directly by the kernel. ``use_workspace=False`` keeps the launch
+    from cutting its last round of workgroups along the keys (no scratch buffer, one kernel).
     """
     _dev(q, k, v, key_mask)
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
@@ -103,39 +105,45 @@ def attn_fwd(
             raise ValueError(f"key_mask must be [B,Sk]={B, Sk}, got {tuple(key_mask.shape)}")
         mask_u8 = (key_mask != 0).to(torch.uint8).contiguous()
     lib = _lib.load()
-    if split is not None and split in (0, Sq):  # one side is empty: the plain entry point writes the other
-        full = o_tail if split == 0 else o
-        rc = lib.odit_attn_fwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), full.data_ptr(), _ptr(mask_u8), _ptr(lse),
-            B, Sq, Sk, H, Hkv, D,
-            _lib.i64_array(q.stride()[:3]), _lib.i64_array(k.stride()[:3]),
-            _lib.i64_array(v.stride()[:3]), _lib.i64_array((Sq * H * D, H * D, D)),
-            float(scale), _code(q), _stream(),
-        )
-        _lib.check(rc, "odit_attn_fwd")
-        return (o, o_tail, lse) if return_lse else (o, o_tail)
-    if split is None:
-        rc = lib.odit_attn_fwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), _ptr(mask_u8), _ptr(lse),
-            B, Sq, Sk, H, Hkv, D,
-            _lib.i64_array(q.stride()[:3]), _lib.i64_array(k.stride()[:3]),
-            _lib.i64_array(v.stride()[:3]), _lib.i64_array(o.stride()[:3]),
-            float(scale), _code(q), _stream(),
-        )
-        _lib.check(rc, "odit_attn_fwd")
-        return (o, lse) if return_lse else o
     # dense [B, n, H, D] strides even when n == 0 or B == 1 (torch may report arbitrary ones there)
-    o_str = (split * H * D, H * D, D)
-    t_str = ((Sq - split) * H * D, H * D, D)
-    rc = lib.odit_attn_fwd_split(
-        q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), o_tail.data_ptr(), int(split),
+    if split is None or split == Sq:
+        head_t, tail_t, cut = o, None, 0
+    elif split == 0:  # the first output is empty: everything goes to the second
+        head_t, tail_t, cut = o_tail, None, 0
+    else:
+        head_t, tail_t, cut = o, o_tail, int(split)
+    n_head = head_t.shape[1]
+    o_str = (n_head * H * D, H * D, D)
+    t_str = None if tail_t is None else _lib.i64_array(((Sq - cut) * H * D, H * D, D))
+    ws = _attn_workspace(lib, q.device, B, Sq, Sk, H, D) if use_workspace else None
+    rc = lib.odit_attn_fwd_ex(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), head_t.data_ptr(), _ptr(tail_t), cut,
         _ptr(mask_u8), _ptr(lse), B, Sq, Sk, H, Hkv, D,
         _lib.i64_array(q.stride()[:3]), _lib.i64_array(k.stride()[:3]),
-        _lib.i64_array(v.stride()[:3]), _lib.i64_array(o_str), _lib.i64_array(t_str),
-        float(scale), _code(q), _stream(),
+        _lib.i64_array(v.stride()[:3]), _lib.i64_array(o_str), t_str,
+        float(scale), _code(q), _ptr(ws), 0 if ws is None else ws.numel(), _stream(),
     )
-    _lib.check(rc, "odit_attn_fwd_split")
+    _lib.check(rc, "odit_attn_fwd_ex")
+    if split is None:
+        return (o, lse) if return_lse else o
     return (o, o_tail, lse) if return_lse else (o, o_tail)
+
+
+_ATTN_SCRATCH: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def _attn_workspace(lib, device: torch.device, B: int, Sq: int, Sk: int, H: int, D: int) -> torch.Tensor | None:
+    """Scratch for the key-split tail of the attention launch, one growing buffer per (device, stream):
+    launches on one stream are ordered, so they can share it."""
+    need = int(lib.odit_attn_fwd_workspace_bytes(B, Sq, Sk, H, D))
+    if need == 0:
+        return None
+    key = (device.index or 0, _stream())
+    ws = _ATTN_SCRATCH.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.empty(need, dtype=torch.uint8, device=device)
+        _ATTN_SCRATCH[key] = ws
+    return ws
 
 
 # --------------------------------------------------------------------------------------------- K2
