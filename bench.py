@@ -24,6 +24,10 @@ if ROOT not in sys.path:
 
 PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, vendor figure
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E, vendor figure
+# HBM bytes of one attention launch at the headline shape, from rocprofv3 FETCH_SIZE / WRITE_SIZE passes
+# over `bench.py --traffic-probe`, each scaled by what the same counter reads for a 512 MiB copy
+# (FETCH_SIZE x2.0, WRITE_SIZE x1.0): 228.0 MB fetched + 53.5 MB written.
+ATTN_TRAFFIC_BYTES = 281.5e6
 
 # Qwen-Image shape at 1024x1024 (BASELINE.json configs[2])
 LAYERS, HEADS, HEAD_DIM, MLP_RATIO = 60, 24, 128, 4
@@ -348,6 +352,9 @@ def main():
     ap.add_argument("--blocks", type=int, default=LAYERS, help="debug only: fewer blocks (result is then marked invalid)")
     ap.add_argument("--workload", choices=("qwen", "flux", "wan"), default="qwen",
                     help="qwen = the headline metric; flux / wan = the other block families at their config shapes")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="launch only the headline attention shape and a plain 512 MiB copy, a few times each: the "
+                         "program to run under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
     args = ap.parse_args()
@@ -368,6 +375,19 @@ def main():
     tuned = gemm_tuning.enable()  # hipBLASLt solution ids picked offline for this model's GEMM shapes
     torch.cuda.set_device(0)
     dev = torch.device("cuda:0")
+    if args.traffic_probe:
+        S = S_IMG + S_TXT
+        q = torch.randn(B, S, HEADS, HEAD_DIM, device=dev, dtype=torch.bfloat16)
+        k, v = torch.randn_like(q), torch.randn_like(q)
+        src = torch.empty(512 << 20, device=dev, dtype=torch.uint8).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            kernels.attn_fwd(q, k, v, 1.0 / math.sqrt(HEAD_DIM))
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": "attention B=2 S=4352 24x128 bf16 x4, copy 512 MiB x4",
+                          "attention_min_bytes": 4 * q.numel() * 2, "copy_bytes_each_way": src.numel()}))
+        return
     if args.workload != "qwen":
         return run_secondary(torch, kernels, args)
     model = build_model(torch, args.blocks)
@@ -422,7 +442,8 @@ def main():
                    "valid": args.blocks == LAYERS, "gemm": "hipBLASLt via torch" + (" (tuned solution table)" if tuned else "")},
         "roofline": {"kernel": "attn_fwd_kernel (joint attention, B=2, 24x128, S=4352)", "bound": "mfma",
                      "achieved": attn_tflops, "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": attn_tflops / PEAK_MFMA_BF16_TFLOPS, "traffic": None,
+                     "frac": attn_tflops / PEAK_MFMA_BF16_TFLOPS,
+                     "traffic": ATTN_TRAFFIC_BYTES if args.blocks == LAYERS else None,
                      "launches_timed": n_attn, "avg_ms": attn_ms, "flop_per_launch": attn_flop},
         "step_flop": None,
     }

@@ -84,8 +84,8 @@ int odit_attn_fwd(const void* q, const void* k, const void* v, void* o, const ui
  * Scratch: `workspace` (device memory, 16-byte aligned, workspace_bytes >=
  * odit_attn_fwd_workspace_bytes for the same shape, contents irrelevant before and after) lets the
  * kernel cut the last, partly filled round of workgroups into key ranges that run side by side and
- * are merged by a second launch; without it a shape whose workgroup count is not a multiple of what
- * the GPU runs at once idles part of the GPU for a whole round. NULL = never split. Results with and
+ * are merged by a second launch; it is used when that last round would fill at most an eighth of the
+ * GPU (few heads x query blocks, many keys), where the unsplit launch leaves most of the GPU idle. NULL = never split. Results with and
  * without scratch agree to rounding (the merge re-associates the key sum); for given shapes and device
  * the partition is fixed, so repeated calls are bit-identical. No counterpart in the reference.
  *

@@ -188,3 +188,77 @@ def test_cfg_combine_and_euler_closed_forms():
     for i in range(6):
         x = denoise.euler_step(x, x / float(sig[i]), float(sig[i]), float(sig[i + 1]))
         assert torch.allclose(x, torch.full_like(x, float(sig[i + 1])), atol=1e-5)
+
+
+# ----------------------------------------------------------------------------- checkpoint loading
+def _split_qkv(flat, fused_suffix, names):
+    """Turn fused [q;k;v] entries of a flat state into three separately stored tensors."""
+    out = {}
+    for k, v in flat.items():
+        hit = next((f for f in fused_suffix if f in k), None)
+        if hit is None:
+            out[k] = v
+            continue
+        for part, t in zip(names[hit], v.chunk(3, dim=0)):
+            out[k.replace(hit, part)] = t
+    return out
+
+
+def test_load_weights_stacks_qkv_and_renames_like_the_reference():
+    from oracle import flux as ofx
+    from oracle import qwen_image as oq
+    from oracle import wan as ow
+    from vllm_omni_amd.blocks.flux import FluxTransformer2DModel
+    from vllm_omni_amd.blocks.qwen_image import QwenImageTransformer2DModel
+    from vllm_omni_amd.blocks.wan import WanTransformer3DModel
+
+    joint = {".to_qkv.": (".to_q.", ".to_k.", ".to_v."),
+             ".add_kv_proj.": (".add_q_proj.", ".add_k_proj.", ".add_v_proj.")}
+    # Qwen-Image: diffusers stores attn.to_out.0
+    cfg = oq.tiny_config()
+    flat = oq.init_params(cfg, seed=3, bias_std=0.02)
+    stored = {k.replace(".attn.to_out.", ".attn.to_out.0."): v for k, v in _split_qkv(flat, list(joint), joint).items()}
+    m = QwenImageTransformer2DModel(in_channels=cfg.in_channels, out_channels=cfg.out_channels,
+                                    num_layers=cfg.num_layers, attention_head_dim=cfg.head_dim,
+                                    num_attention_heads=cfg.num_heads, joint_attention_dim=cfg.joint_attention_dim,
+                                    axes_dims_rope=cfg.axes_dims_rope)
+    loaded = m.load_weights(stored.items())
+    assert set(stored) <= loaded
+    for k, p in m.named_parameters():
+        assert torch.equal(p, flat[k]), k
+    # Flux
+    fcfg = ofx.tiny_config()
+    fflat = ofx.init_params(fcfg, seed=4, bias_std=0.02)
+    fm = FluxTransformer2DModel(in_channels=fcfg.in_channels, out_channels=fcfg.out_channels,
+                                num_layers=fcfg.num_layers, num_single_layers=fcfg.num_single_layers,
+                                attention_head_dim=fcfg.head_dim, num_attention_heads=fcfg.num_heads,
+                                joint_attention_dim=fcfg.joint_attention_dim,
+                                pooled_projection_dim=fcfg.pooled_projection_dim, axes_dims_rope=fcfg.axes_dims_rope)
+    fm.load_weights(_split_qkv(fflat, list(joint), joint).items())
+    for k, p in fm.named_parameters():
+        assert torch.equal(p, fflat[k]), k
+    # Wan: only attn1 is fused; ffn.net.N and the top-level scale_shift_table are renamed; extras are skipped
+    wcfg = ow.tiny_config()
+    wflat = ow.init_params(wcfg, seed=5, bias_std=0.02, norm_jitter=0.1)
+    a1 = {".attn1.to_qkv.": (".attn1.to_q.", ".attn1.to_k.", ".attn1.to_v.")}
+    wstored = {}
+    for k, v in _split_qkv(wflat, list(a1), a1).items():
+        k = k.replace(".ffn.net_0.", ".ffn.net.0.").replace(".ffn.net_2.", ".ffn.net.2.")
+        k = k.replace(".to_out.", ".to_out.0.")
+        if k == "output_scale_shift_prepare.scale_shift_table":
+            k = "scale_shift_table"
+        wstored[k] = v
+    wstored["not.a.parameter"] = torch.zeros(1)
+    wm = WanTransformer3DModel(patch_size=wcfg.patch_size, num_attention_heads=wcfg.num_heads,
+                               attention_head_dim=wcfg.head_dim, in_channels=wcfg.in_channels,
+                               out_channels=wcfg.out_channels, text_dim=wcfg.text_dim, ffn_dim=wcfg.ffn_dim,
+                               num_layers=wcfg.num_layers, rope_max_seq_len=wcfg.rope_max_seq_len)
+    loaded = wm.load_weights(wstored.items())
+    assert "not.a.parameter" not in loaded
+    for k, p in wm.named_parameters():
+        assert torch.equal(p, wflat[k]), k
+    # a shard of the wrong size is an error, not a silent partial copy
+    with pytest.raises(ValueError):
+        m.load_weights([("transformer_blocks.0.attn.to_q.weight", torch.zeros(3, cfg.dim))])
+    with pytest.raises(KeyError):
+        m.load_weights([("transformer_blocks.0.nothing.weight", torch.zeros(1))])

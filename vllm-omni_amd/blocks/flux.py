@@ -394,6 +394,12 @@ class FluxTransformer2DModel(nn.Module):
         return self.finish(img, temb, return_dict=return_dict)
 
     # -- weights --------------------------------------------------------------------------------
+    def load_weights(self, weights) -> set[str]:
+        """Load a diffusers-layout checkpoint stream, stacking separate q/k/v projections (flux.py:588-628)."""
+        from .weights import QKV_JOINT_MAPPING, load_stacked_weights
+
+        return load_stacked_weights(self, weights, QKV_JOINT_MAPPING, substring_renames=((".to_out.0.", ".to_out."),))
+
     def load_flat_state(self, weights: dict[str, torch.Tensor]) -> None:
         """Load a flat name->tensor dict keyed with the reference's parameter names."""
         own = dict(self.named_parameters())

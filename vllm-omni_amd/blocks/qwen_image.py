@@ -400,6 +400,13 @@ class QwenImageTransformer2DModel(nn.Module):
         return self.finish(img, temb, return_dict=return_dict)
 
     # -- weights --------------------------------------------------------------------------------
+    def load_weights(self, weights) -> set[str]:
+        """Load a diffusers-layout checkpoint stream: separate to_q/to_k/to_v and add_*_proj tensors are
+        stacked into the fused projections, ``attn.to_out.0`` maps to ``attn.to_out`` (qit.py:1073-1113)."""
+        from .weights import QKV_JOINT_MAPPING, load_stacked_weights
+
+        return load_stacked_weights(self, weights, QKV_JOINT_MAPPING, substring_renames=((".to_out.0.", ".to_out."),))
+
     def load_flat_state(self, weights: dict[str, torch.Tensor]) -> None:
         """Load a flat name->tensor dict keyed with the reference's parameter names."""
         own = dict(self.named_parameters())

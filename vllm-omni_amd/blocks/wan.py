@@ -372,6 +372,19 @@ class WanTransformer3DModel(nn.Module):
         x = self.run_blocks(x, ctx, tproj, rotary)
         return self.finish(x, temb, (nf // p_t, hh // p_h, ww // p_w), return_dict=return_dict)
 
+    def load_weights(self, weights) -> set[str]:
+        """Load a diffusers-layout checkpoint stream (wan.py:907-990): attn1 q/k/v are stacked, attn2's
+        stay separate, ``ffn.net.N`` maps to ``ffn.net_N``, ``to_out.0`` to ``to_out``, the top-level
+        ``scale_shift_table`` to ``output_scale_shift_prepare.scale_shift_table``; unknown names are skipped."""
+        from .weights import load_stacked_weights
+
+        mapping = [(".attn1.to_qkv", ".attn1.to_q", "q"), (".attn1.to_qkv", ".attn1.to_k", "k"),
+                   (".attn1.to_qkv", ".attn1.to_v", "v")]
+        renames = ((".ffn.net.0.", ".ffn.net_0."), (".ffn.net.2.", ".ffn.net_2."), (".to_out.0.", ".to_out."))
+        return load_stacked_weights(self, weights, mapping, substring_renames=renames,
+                                    exact_renames={"scale_shift_table": "output_scale_shift_prepare.scale_shift_table"},
+                                    skip_unknown=True)
+
     def load_flat_state(self, weights: dict[str, torch.Tensor]) -> None:
         """Load a flat name->tensor dict keyed with the reference's parameter names."""
         own = dict(self.named_parameters())

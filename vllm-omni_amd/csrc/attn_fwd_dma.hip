@@ -404,9 +404,12 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const AttnParams p, int
 }
 
 // How the last round of workgroups is cut along the keys. `slots` workgroups run at once; after
-// `units / slots` full rounds, `rem` units are left: when they would leave at least half the slots
-// idle, each is cut into as many key ranges as fit the idle slots (ranges of an even number of tiles,
-// at least kMinTilesPerChunk), so the tail takes 1/key_chunks of a round instead of a whole one.
+// `units / slots` full rounds, `rem` units are left: when they would occupy at most an eighth of the
+// slots, each is cut into as many key ranges as fit the slots (ranges of an even number of tiles, at
+// least kMinTilesPerChunk), so the tail takes 1/key_chunks of a round instead of most of one. Measured
+// at rem = 96 of 512 slots (the 4352-token, 48-head shape): the unsplit tail costs 0.7 of a round, the
+// split one 0.2 of a round plus two more launches and 130 MB of partial results - no gain, hence the
+// threshold.
 struct TailPlan { int rem, key_chunks, tiles_per_chunk; };
 constexpr int kMinTilesPerChunk = 8;
 constexpr int kMaxKeyChunks = 16;
@@ -426,7 +429,7 @@ static int device_slots(int nw) {
 static TailPlan plan_tail(int64_t units, int n_tiles, int slots) {
   TailPlan t{0, 1, n_tiles};
   const int rem = static_cast<int>(units % slots);
-  if (rem == 0 || 2 * rem > slots) return t;
+  if (rem == 0 || 8 * rem > slots) return t;
   int kc = slots / rem;
   if (kc > kMaxKeyChunks) kc = kMaxKeyChunks;
   if (kc > n_tiles / kMinTilesPerChunk) kc = n_tiles / kMinTilesPerChunk;
