@@ -94,7 +94,7 @@ class AttnTimer:
         return sum(ms) / len(ms), top, len(ms)
 
 
-def build_model(torch, layers):
+def build_model(torch, layers, fuse_epilogues=True):
     from vllm_omni_amd.blocks.qwen_image import QwenImageTransformer2DModel
 
     prev = torch.get_default_dtype()
@@ -103,7 +103,8 @@ def build_model(torch, layers):
         with torch.device("cuda"):
             model = QwenImageTransformer2DModel(num_layers=layers, attention_head_dim=HEAD_DIM,
                                                 num_attention_heads=HEADS, joint_attention_dim=TEXT_DIM,
-                                                in_channels=IN_CH, out_channels=16, mlp_ratio=MLP_RATIO)
+                                                in_channels=IN_CH, out_channels=16, mlp_ratio=MLP_RATIO,
+                                                fuse_epilogues=fuse_epilogues)
     finally:
         torch.set_default_dtype(prev)
     g = torch.Generator(device="cuda").manual_seed(0)
@@ -213,6 +214,10 @@ def run_secondary(torch, kernels, args):
     make = flux_workload if args.workload == "flux" else wan_workload
     model, step, lat, name, gemm_flop, valid = make(torch, None if args.blocks == LAYERS else args.blocks)
     with torch.inference_mode(), AttnTimer(torch, kernels) as timer:
+        if args.autotune > 0:
+            kernels.set_linear_autotune(args.autotune)
+            step(0, lat)
+            kernels.set_linear_autotune(0)
         for i in range(args.warmup):
             lat = step(i, lat)
         torch.cuda.synchronize()
@@ -355,6 +360,10 @@ def main():
     ap.add_argument("--traffic-probe", action="store_true",
                     help="launch only the headline attention shape and a plain 512 MiB copy, a few times each: the "
                          "program to run under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`")
+    ap.add_argument("--unfused-epilogues", action="store_true",
+                    help="A/B switch: GELU and gated residuals as separate kernels after plain GEMMs")
+    ap.add_argument("--autotune", type=int, default=0,
+                    help="time the library's kernels for each fused-epilogue GEMM in an untimed first step")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
     args = ap.parse_args()
@@ -390,7 +399,7 @@ def main():
         return
     if args.workload != "qwen":
         return run_secondary(torch, kernels, args)
-    model = build_model(torch, args.blocks)
+    model = build_model(torch, args.blocks, fuse_epilogues=not args.unfused_epilogues)
     g = torch.Generator(device="cuda").manual_seed(1)
     latents = torch.randn(1, S_IMG, IN_CH, device=dev, generator=g).bfloat16()
     text = torch.randn(B, S_TXT, TEXT_DIM, device=dev, generator=g).bfloat16()
@@ -406,6 +415,10 @@ def main():
 
     with torch.inference_mode(), AttnTimer(torch, kernels) as timer:
         lat = latents
+        if args.autotune > 0:   # untimed: pick the library kernel for each fused-epilogue GEMM
+            kernels.set_linear_autotune(args.autotune)
+            step(0, lat)
+            kernels.set_linear_autotune(0)
         for i in range(args.warmup):
             lat = step(i, lat)
         torch.cuda.synchronize()
@@ -439,7 +452,9 @@ def main():
         "config": {"workload": f"Qwen-Image-shape MMDiT denoise step: {args.blocks} dual-stream blocks, hidden {C}, "
                                f"{HEADS} heads x {HEAD_DIM}, MLP {MLP_RATIO * C}, {S_IMG} image + {S_TXT} text tokens, "
                                "CFG batch 2, random weights N(0,0.02)",
-                   "valid": args.blocks == LAYERS, "gemm": "hipBLASLt via torch" + (" (tuned solution table)" if tuned else "")},
+                   "valid": args.blocks == LAYERS, "gemm": "hipBLASLt via torch" + (" (tuned solution table)" if tuned else "") +
+                           ("; GELU and gated residuals as separate kernels" if args.unfused_epilogues else
+                            "; GELU and gated residuals in the GEMM epilogues (odit_linear)")},
         "roofline": {"kernel": "attn_fwd_kernel (joint attention, B=2, 24x128, S=4352)", "bound": "mfma",
                      "achieved": attn_tflops, "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": attn_tflops / PEAK_MFMA_BF16_TFLOPS,

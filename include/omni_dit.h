@@ -199,6 +199,59 @@ int odit_rel_l1(const void* cur, const void* prev, double* sums, void* workspace
 int odit_gelu_tanh(const void* x, void* out, int64_t n, int dtype, void* stream);
 int odit_silu(const void* x, void* out, int64_t n, int dtype, void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Dense projection with the elementwise work done in the GEMM's epilogue:
+ *     ODIT_EPI_NONE / ODIT_EPI_BIAS        out = x W^T (+ bias)
+ *     ODIT_EPI_(BIAS_)GELU_TANH            out = gelu_tanh(x W^T (+ bias))
+ *     ODIT_EPI_GATED_RESIDUAL              out = residual + gate * (x W^T + bias)
+ *     ODIT_EPI_GATED_RESIDUAL_PRE          out = residual + gate * (x W^T) + bias, with float32 `gate` and a
+ *                                          float32 `bias` the caller has already multiplied by the gate
+ *                                          (NULL = none): no helper launch; for callers that form the
+ *                                          gates of all blocks of a step at once
+ *
+ * Replaces, as one launch each (plus a [N]-sized helper launch for the gated form):
+ *   ColumnParallelLinear + F.gelu(approximate="tanh")     qwen_image_transformer.py:399-424,
+ *                                                          flux_transformer.py:30-45, wan2_2_transformer.py:92-109
+ *   RowParallelLinear followed by `h + gate * y`           qwen_image_transformer.py:794-795, 801, 806,
+ *                                                          flux_transformer.py:288-309, wan2_2_transformer.py:661, 673
+ * The contraction runs on hipBLASLt's MFMA kernels (it is a plain dense GEMM); this entry point sets the
+ * problem up so that bias, activation, gate and residual ride in that kernel's epilogue.
+ *
+ * x [M,K] (row stride ldx), W [N,K] (row stride ldw: torch's nn.Linear weight, or a column range of
+ * one), bias [N] or NULL, out [M,N] (row stride ldo). Gated form: residual [M,N] (row stride ldr; may be
+ * `out` itself), gate [N] of `dtype` or float32 (gate_dtype), NULL = ones: one call per batch row when
+ * the gate differs per batch row. dtype: ODIT_BF16, ODIT_F16 or ODIT_F32 (fp32 accumulation always).
+ * workspace: device scratch, 256-byte aligned, for the library's split-K kernels and, in the gated
+ * form, two float[N] vectors; odit_linear_workspace_bytes() is a size that suits every kernel. NULL
+ * restricts the choice to kernels that need none (not allowed for the gated form).
+ *
+ * odit_linear_tune launches every kernel the library offers for the problem on the given buffers
+ * (`out` is overwritten; this call synchronises with the stream), keeps the fastest for later
+ * odit_linear calls with the same shape, strides, epilogue and dtype FROM THE SAME HOST THREAD, and
+ * reports its time. `flush` (optional device buffer, ideally larger than the last-level cache) is
+ * overwritten before every timed launch so that each one starts from cold caches, as a projection
+ * with its own weights does inside a model. Without tuning the library's own first choice is used.
+ */
+enum odit_epilogue {
+  ODIT_EPI_NONE = 0,
+  ODIT_EPI_BIAS = 1,
+  ODIT_EPI_GELU_TANH = 2,
+  ODIT_EPI_BIAS_GELU_TANH = 3,
+  ODIT_EPI_GATED_RESIDUAL = 4,
+  ODIT_EPI_GATED_RESIDUAL_PRE = 5
+};
+
+size_t odit_linear_workspace_bytes(void);
+
+int odit_linear(const void* x, const void* w, const void* bias, void* out, const void* residual,
+                const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int64_t ldr,
+                int epilogue, int gate_dtype, int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+int odit_linear_tune(const void* x, const void* w, const void* bias, void* out, const void* residual,
+                     const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int64_t ldr,
+                     int epilogue, int gate_dtype, int dtype, void* workspace, size_t workspace_bytes,
+                     void* stream, int iters, void* flush, size_t flush_bytes, float* best_us);
+
 #ifdef __cplusplus
 }
 #endif

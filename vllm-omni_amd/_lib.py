@@ -18,6 +18,8 @@ ODIT_BF16, ODIT_F16, ODIT_F32 = 0, 1, 2
 ODIT_FLAG_REF_ROUNDING = 1
 ODIT_FLAG_NEOX = 2
 ODIT_NORM_NONE, ODIT_NORM_HEAD, ODIT_NORM_ROW = 0, 1, 2
+ODIT_EPI_NONE, ODIT_EPI_BIAS, ODIT_EPI_GELU_TANH, ODIT_EPI_BIAS_GELU_TANH, ODIT_EPI_GATED_RESIDUAL = 0, 1, 2, 3, 4
+ODIT_EPI_GATED_RESIDUAL_PRE = 5
 
 # every symbol include/omni_dit.h declares: (name, restype, argtypes)
 _i64p = C.POINTER(C.c_int64)
@@ -60,6 +62,18 @@ _SIGNATURES = {
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int64,
          C.c_int64, C.c_int64, C.c_int, C.c_uint, C.c_void_p],
+    ),
+    "odit_linear_workspace_bytes": (C.c_size_t, []),
+    "odit_linear": (
+        C.c_int,
+        [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
+         C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p],
+    ),
+    "odit_linear_tune": (
+        C.c_int,
+        [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
+         C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p,
+         C.c_int, C.c_void_p, C.c_size_t, C.POINTER(C.c_float)],
     ),
     "odit_gelu_tanh": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p]),
     "odit_silu": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p]),

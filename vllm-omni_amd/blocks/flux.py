@@ -32,7 +32,7 @@ from ..attention.layer import Attention
 from ..layers.rmsnorm import RMSNorm
 from ..layers.rope import RotaryEmbedding
 from .qwen_image import (AdaLayerNormContinuous, FeedForward, QwenTimestepProjEmbeddings, TimestepEmbedding,
-                         Transformer2DModelOutput)
+                         Transformer2DModelOutput, project_residual)
 
 
 class FluxRotary:
@@ -117,7 +117,9 @@ class FluxAttention(nn.Module):
         self.ref_rounding = ref_rounding
 
     def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor | None = None,
-                image_rotary_emb=None, **kwargs):
+                image_rotary_emb=None, residuals=None, **kwargs):
+        """``residuals`` = (residual, gate, context_residual, context_gate) (dual blocks only): return
+        residual + gate * projection for both streams instead of the bare projections."""
         rot = _rotary(image_rotary_emb)
         B, S_x, _ = hidden_states.shape
         H, D = self.heads, self.head_dim
@@ -147,6 +149,10 @@ class FluxAttention(nn.Module):
                             self.norm_k.weight, ic, isn, eps=self.eps, out_seq_offset=S_c,
                             norm_mode=ODIT_NORM_HEAD, ref_rounding=rr)
         ctx_attn, x_attn = self.attn(jq, jk, jv, AttentionMetadata(output_split=S_c))
+        if residuals is not None:
+            res, gate, c_res, c_gate = residuals
+            return (project_residual(self.to_out[0], x_attn.flatten(2, 3), res, gate, ref_rounding=rr),
+                    project_residual(self.to_add_out, ctx_attn.flatten(2, 3), c_res, c_gate, ref_rounding=rr))
         return self.to_out[0](x_attn.flatten(2, 3)), self.to_add_out(ctx_attn.flatten(2, 3))
 
 
@@ -163,9 +169,9 @@ class FluxTransformerBlock(nn.Module):
                                   heads=num_attention_heads, out_dim=dim, context_pre_only=False, bias=True,
                                   eps=eps, ref_rounding=rr)
         self.norm2 = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
-        self.ff = FeedForward(dim=dim, dim_out=dim)
+        self.ff = FeedForward(dim=dim, dim_out=dim, fused=not rr)
         self.norm2_context = nn.LayerNorm(dim, elementwise_affine=False, eps=1e-6)
-        self.ff_context = FeedForward(dim=dim, dim_out=dim)
+        self.ff_context = FeedForward(dim=dim, dim_out=dim, fused=not rr)
         self.ref_rounding = rr
 
     def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, temb: torch.Tensor,
@@ -178,20 +184,17 @@ class FluxTransformerBlock(nn.Module):
         n_x, gate_msa, shift_mlp, scale_mlp, gate_mlp = self.norm1(hidden_states, emb=temb, mod=m_x)
         n_c, c_gate_msa, c_shift_mlp, c_scale_mlp, c_gate_mlp = self.norm1_context(encoder_hidden_states,
                                                                                    emb=temb, mod=m_c)
-        attn_output, context_attn_output = self.attn(hidden_states=n_x, encoder_hidden_states=n_c,
-                                                     image_rotary_emb=image_rotary_emb,
-                                                     **(joint_attention_kwargs or {}))
-        # inputs are never written: callers (TeaCache) keep them to form residuals
-        hidden_states = kernels.gated_residual(hidden_states, attn_output, gate_msa, ref_rounding=rr)
+        # inputs are never written (callers such as TeaCache keep them to form residuals): the attention
+        # residuals land in new tensors, the feed-forward residuals then update those in place
+        hidden_states, encoder_hidden_states = self.attn(
+            hidden_states=n_x, encoder_hidden_states=n_c, image_rotary_emb=image_rotary_emb,
+            residuals=(hidden_states, gate_msa, encoder_hidden_states, c_gate_msa), **(joint_attention_kwargs or {}))
         n2 = kernels.adaln_modulate(hidden_states, shift_mlp, scale_mlp, eps=self.norm2.eps, ref_rounding=rr)
-        hidden_states = kernels.gated_residual(hidden_states, self.ff(n2), gate_mlp, out=hidden_states,
-                                               ref_rounding=rr)
-        encoder_hidden_states = kernels.gated_residual(encoder_hidden_states, context_attn_output, c_gate_msa,
-                                                       ref_rounding=rr)
+        hidden_states = self.ff.forward_residual(n2, hidden_states, gate_mlp, out=hidden_states, ref_rounding=rr)
         c2 = kernels.adaln_modulate(encoder_hidden_states, c_shift_mlp, c_scale_mlp, eps=self.norm2_context.eps,
                                     ref_rounding=rr)
-        encoder_hidden_states = kernels.gated_residual(encoder_hidden_states, self.ff_context(c2), c_gate_mlp,
-                                                       out=encoder_hidden_states, ref_rounding=rr)
+        encoder_hidden_states = self.ff_context.forward_residual(c2, encoder_hidden_states, c_gate_mlp,
+                                                                 out=encoder_hidden_states, ref_rounding=rr)
         if encoder_hidden_states.dtype == torch.float16:
             encoder_hidden_states = encoder_hidden_states.clip(-65504, 65504)
         return encoder_hidden_states, hidden_states
@@ -218,15 +221,24 @@ class FluxSingleTransformerBlock(nn.Module):
                       mod: torch.Tensor | None = None, in_place: bool = False) -> torch.Tensor:
         B, S, C = x.shape
         n, gate = self.norm(x, emb=temb, mod=mod)
-        mlp = self.proj_mlp(n)
-        mlp = kernels.gelu_tanh(mlp, out=mlp)
+        fused = not self.ref_rounding and x.dtype != torch.float32
+        if fused:
+            mlp = kernels.linear(n, self.proj_mlp.weight, self.proj_mlp.bias, activation="gelu_tanh")
+        else:
+            mlp = self.proj_mlp(n)
+            mlp = kernels.gelu_tanh(mlp, out=mlp)
         att = self.attn(hidden_states=n, image_rotary_emb=image_rotary_emb)
-        # proj_out(cat([att, mlp], -1)) as two GEMMs over the two column ranges of the weight
+        # gate * proj_out(cat([att, mlp], -1)) + x as two GEMMs over the two column ranges of the weight,
+        # each accumulating onto the residual stream through its epilogue
         w = self.proj_out.weight
-        y = F.linear(mlp.view(B * S, -1), w[:, C:], self.proj_out.bias)
-        y.addmm_(att.reshape(B * S, C), w[:, :C].t())
-        out = kernels.gated_residual(x, y.view(B, S, C), gate, out=x if in_place else None,
-                                     ref_rounding=self.ref_rounding)
+        if fused:
+            out = kernels.linear(mlp, w[:, C:], self.proj_out.bias, residual=x, gate=gate, out=x if in_place else None)
+            out = kernels.linear(att, w[:, :C], None, residual=out, gate=gate, out=out)
+        else:
+            y = F.linear(mlp.view(B * S, -1), w[:, C:], self.proj_out.bias)
+            y.addmm_(att.reshape(B * S, C), w[:, :C].t())
+            out = kernels.gated_residual(x, y.view(B, S, C), gate, out=x if in_place else None,
+                                         ref_rounding=self.ref_rounding)
         if out.dtype == torch.float16:
             out = out.clip(-65504, 65504)
         return out

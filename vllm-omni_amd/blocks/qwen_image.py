@@ -47,13 +47,18 @@ class SiLU(nn.Module):
 
 
 class ApproxGELU(nn.Module):
-    """Linear + GELU(tanh) (qit.py:399-424); the activation overwrites the projection output."""
+    """Linear + GELU(tanh) (qit.py:399-424) as one GEMM whose epilogue applies bias and activation.
+    ``fused = False`` runs the projection and then the activation in place on its output, which rounds
+    the pre-activation to the tensor dtype like the reference's two ops do."""
 
-    def __init__(self, dim_in: int, dim_out: int, bias: bool = True):
+    def __init__(self, dim_in: int, dim_out: int, bias: bool = True, fused: bool = True):
         super().__init__()
         self.proj = nn.Linear(dim_in, dim_out, bias=bias)
+        self.fused = fused
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self.fused and x.dtype != torch.float32 and x.is_contiguous():
+            return kernels.linear(x, self.proj.weight, self.proj.bias, activation="gelu_tanh")
         y = self.proj(x)
         return kernels.gelu_tanh(y, out=y)
 
@@ -62,16 +67,40 @@ class FeedForward(nn.Module):
     """net.0 = Linear+GELU(tanh), net.1 = placeholder, net.2 = Linear (qit.py:427-466)."""
 
     def __init__(self, dim: int, dim_out: int | None = None, mult: int = 4, inner_dim: int | None = None,
-                 bias: bool = True):
+                 bias: bool = True, fused: bool = True):
         super().__init__()
         inner = inner_dim or dim * mult
-        self.net = nn.ModuleList([ApproxGELU(dim, inner, bias=bias), nn.Identity(),
+        self.net = nn.ModuleList([ApproxGELU(dim, inner, bias=bias, fused=fused), nn.Identity(),
                                   nn.Linear(inner, dim_out or dim, bias=bias)])
+        self.fused = fused
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         for m in self.net:
             x = m(x)
         return x
+
+    def forward_residual(self, x: torch.Tensor, residual: torch.Tensor, gate: torch.Tensor | None,
+                         out: torch.Tensor | None = None, ref_rounding: bool = False, pre=None) -> torch.Tensor:
+        """residual + gate * FF(x): with ``fused`` the down-projection's epilogue adds the gated result
+        onto the residual; otherwise the projection is followed by the gated-residual kernel."""
+        return project_residual(self.net[2], self.net[0](x), residual, gate, out=out,
+                                fused=self.fused, ref_rounding=ref_rounding, pre=pre)
+
+
+def project_residual(lin: nn.Linear, x: torch.Tensor, residual: torch.Tensor, gate: torch.Tensor | None,
+                     out: torch.Tensor | None = None, fused: bool = True, ref_rounding: bool = False,
+                     pre: tuple[torch.Tensor, torch.Tensor | None] | None = None) -> torch.Tensor:
+    """residual + gate * lin(x) (gate [B,N] or [B,1,N], None = plain add) in one GEMM, or, unfused, as
+    projection + gated-residual kernel (qit.py:794-806). ``pre`` = (float32 gate [B,N], float32
+    gate * bias [B,N] or None) made by the caller for all blocks at once replaces ``gate`` on the fused path."""
+    per_token_gate = gate is not None and gate.dim() == 3 and gate.shape[1] != 1
+    if (fused and not ref_rounding and not per_token_gate and x.dtype != torch.float32 and x.is_contiguous()
+            and residual.is_contiguous()):
+        if pre is not None:
+            return kernels.linear(x, lin.weight, None, residual=residual, gate=pre[0], gate_bias=pre[1],
+                                  prescaled=True, out=out)
+        return kernels.linear(x, lin.weight, lin.bias, residual=residual, gate=gate, out=out)
+    return kernels.gated_residual(residual, lin(x), gate, out=out, ref_rounding=ref_rounding)
 
 
 class QwenEmbedRope(nn.Module):
@@ -149,9 +178,10 @@ class QwenImageCrossAttention(nn.Module):
     """Joint text+image attention of one block (qit.py:469-661)."""
 
     def __init__(self, dim: int, num_heads: int, head_dim: int, added_kv_proj_dim: int,
-                 out_bias: bool = True, eps: float = 1e-6, ref_rounding: bool = False):
+                 out_bias: bool = True, eps: float = 1e-6, ref_rounding: bool = False, fused: bool = True):
         super().__init__()
         assert dim % num_heads == 0
+        self.fused = fused
         self.dim, self.head_dim, self.total_num_heads, self.eps = dim, head_dim, num_heads, eps
         inner = head_dim * num_heads
         self.inner_dim = inner
@@ -171,7 +201,10 @@ class QwenImageCrossAttention(nn.Module):
 
     def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, vid_freqs, txt_freqs=None,
                 hidden_states_mask: torch.Tensor | None = None,
-                encoder_hidden_states_mask: torch.Tensor | None = None):
+                encoder_hidden_states_mask: torch.Tensor | None = None, residuals=None):
+        """``residuals`` = (img_residual, img_gate, txt_residual, txt_gate[, img_pre, txt_pre]): return
+        residual + gate * projection for both streams (new tensors) instead of the bare projections;
+        the ``*_pre`` pairs are caller-made float32 (gate, gate * bias) rows (see project_residual)."""
         tables = vid_freqs if isinstance(vid_freqs, RotaryTables) else RotaryTables(vid_freqs, txt_freqs)
         B, S_img, _ = hidden_states.shape
         S_txt = encoder_hidden_states.shape[1]
@@ -197,6 +230,14 @@ class QwenImageCrossAttention(nn.Module):
             img_m = hidden_states_mask if hidden_states_mask is not None else ones(S_img)
             meta.attn_mask = torch.cat([txt_m.bool(), img_m.bool()], dim=1)
         txt_attn, img_attn = self.attn(jq, jk, jv, meta)
+        if residuals is not None:
+            img_res, img_gate, txt_res, txt_gate = residuals[:4]
+            img_pre, txt_pre = residuals[4:] if len(residuals) == 6 else (None, None)
+            img_out = project_residual(self.to_out, img_attn.flatten(2, 3), img_res, img_gate,
+                                       fused=self.fused, ref_rounding=rr, pre=img_pre)
+            txt_out = project_residual(self.to_add_out, txt_attn.flatten(2, 3), txt_res, txt_gate,
+                                       fused=self.fused, ref_rounding=rr, pre=txt_pre)
+            return img_out, txt_out
         img_out = self.to_out(img_attn.flatten(2, 3))
         txt_out = self.to_add_out(txt_attn.flatten(2, 3))
         return img_out, txt_out
@@ -206,20 +247,22 @@ class QwenImageTransformerBlock(nn.Module):
     """One dual-stream block (qit.py:664-814); returns (encoder_hidden_states, hidden_states)."""
 
     def __init__(self, dim: int, num_attention_heads: int, attention_head_dim: int, eps: float = 1e-6,
-                 zero_cond_t: bool = False, mlp_ratio: int = 4, ref_rounding: bool = False):
+                 zero_cond_t: bool = False, mlp_ratio: int = 4, ref_rounding: bool = False,
+                 fuse_epilogues: bool = True):
         super().__init__()
         self.dim = dim
+        fused = fuse_epilogues and not ref_rounding
         self.num_attention_heads, self.attention_head_dim = num_attention_heads, attention_head_dim
         self.img_mod = nn.Sequential(SiLU(), nn.Linear(dim, 6 * dim, bias=True))
         self.img_norm1 = AdaLayerNorm(dim, elementwise_affine=False, eps=eps, ref_rounding=ref_rounding)
         self.attn = QwenImageCrossAttention(dim=dim, num_heads=num_attention_heads, head_dim=attention_head_dim,
-                                            added_kv_proj_dim=dim, eps=eps, ref_rounding=ref_rounding)
+                                            added_kv_proj_dim=dim, eps=eps, ref_rounding=ref_rounding, fused=fused)
         self.img_norm2 = AdaLayerNorm(dim, elementwise_affine=False, eps=eps, ref_rounding=ref_rounding)
-        self.img_mlp = FeedForward(dim=dim, dim_out=dim, mult=mlp_ratio)
+        self.img_mlp = FeedForward(dim=dim, dim_out=dim, mult=mlp_ratio, fused=fused)
         self.txt_mod = nn.Sequential(SiLU(), nn.Linear(dim, 6 * dim, bias=True))
         self.txt_norm1 = AdaLayerNorm(dim, elementwise_affine=False, eps=eps, ref_rounding=ref_rounding)
         self.txt_norm2 = AdaLayerNorm(dim, elementwise_affine=False, eps=eps, ref_rounding=ref_rounding)
-        self.txt_mlp = FeedForward(dim=dim, dim_out=dim, mult=mlp_ratio)
+        self.txt_mlp = FeedForward(dim=dim, dim_out=dim, mult=mlp_ratio, fused=fused)
         self.zero_cond_t = zero_cond_t
         self.ref_rounding = ref_rounding
 
@@ -227,9 +270,15 @@ class QwenImageTransformerBlock(nn.Module):
                 encoder_hidden_states_mask: torch.Tensor | None, temb: torch.Tensor, image_rotary_emb,
                 joint_attention_kwargs: dict[str, Any] | None = None, modulate_index: torch.Tensor | None = None,
                 hidden_states_mask: torch.Tensor | None = None,
-                mod_params: tuple[torch.Tensor, torch.Tensor] | None = None):
+                mod_params: tuple[torch.Tensor, torch.Tensor] | None = None,
+                gate_rows: tuple[torch.Tensor, torch.Tensor] | None = None):
         """``mod_params`` = (img [B,6C], txt [B,6C]) computed by the caller for all blocks at once
-        (they depend on ``temb`` only); when absent they are computed here as in the reference."""
+        (they depend on ``temb`` only); when absent they are computed here as in the reference.
+        ``gate_rows`` = float32 (gates, gates * biases), each [B, 2 (img, txt), 2 (attention, MLP), C],
+        likewise made once per step: the fused output projections then need no per-call set-up."""
+        pre = [[None, None], [None, None]]
+        if gate_rows is not None and modulate_index is None:
+            pre = [[(gate_rows[0][:, s, j], gate_rows[1][:, s, j]) for j in range(2)] for s in range(2)]
         rr = self.ref_rounding
         if mod_params is not None:
             img_mod_params, txt_mod_params = mod_params
@@ -244,19 +293,19 @@ class QwenImageTransformerBlock(nn.Module):
         img_modulated, img_gate1 = self.img_norm1(hidden_states, img_mod1, modulate_index)
         txt_modulated, txt_gate1 = self.txt_norm1(encoder_hidden_states, txt_mod1)
         tables = image_rotary_emb if isinstance(image_rotary_emb, RotaryTables) else RotaryTables(*image_rotary_emb)
-        img_attn, txt_attn = self.attn(img_modulated, txt_modulated, tables,
-                                       hidden_states_mask=hidden_states_mask,
-                                       encoder_hidden_states_mask=encoder_hidden_states_mask)
-        # the block's inputs are never written: callers (TeaCache) keep them to form residuals
-        hidden_states = kernels.gated_residual(hidden_states, img_attn, img_gate1, ref_rounding=rr)
-        encoder_hidden_states = kernels.gated_residual(encoder_hidden_states, txt_attn, txt_gate1, ref_rounding=rr)
+        # the block's inputs are never written (callers such as TeaCache keep them to form residuals):
+        # the attention residuals land in new tensors, the MLP residuals then update those in place
+        hidden_states, encoder_hidden_states = self.attn(
+            img_modulated, txt_modulated, tables, hidden_states_mask=hidden_states_mask,
+            encoder_hidden_states_mask=encoder_hidden_states_mask,
+            residuals=(hidden_states, img_gate1, encoder_hidden_states, txt_gate1, pre[0][0], pre[1][0]))
 
         img_modulated2, img_gate2 = self.img_norm2(hidden_states, img_mod2, modulate_index)
-        hidden_states = kernels.gated_residual(hidden_states, self.img_mlp(img_modulated2), img_gate2,
-                                               out=hidden_states, ref_rounding=rr)
+        hidden_states = self.img_mlp.forward_residual(img_modulated2, hidden_states, img_gate2, out=hidden_states,
+                                                      ref_rounding=rr, pre=pre[0][1])
         txt_modulated2, txt_gate2 = self.txt_norm2(encoder_hidden_states, txt_mod2)
-        encoder_hidden_states = kernels.gated_residual(encoder_hidden_states, self.txt_mlp(txt_modulated2),
-                                                       txt_gate2, out=encoder_hidden_states, ref_rounding=rr)
+        encoder_hidden_states = self.txt_mlp.forward_residual(txt_modulated2, encoder_hidden_states, txt_gate2,
+                                                              out=encoder_hidden_states, ref_rounding=rr, pre=pre[1][1])
         if encoder_hidden_states.dtype == torch.float16:
             encoder_hidden_states = encoder_hidden_states.clip(-65504, 65504)
         if hidden_states.dtype == torch.float16:
@@ -317,7 +366,7 @@ class QwenImageTransformer2DModel(nn.Module):
     def __init__(self, patch_size: int = 2, in_channels: int = 64, out_channels: int | None = 16,
                  num_layers: int = 60, attention_head_dim: int = 128, num_attention_heads: int = 24,
                  joint_attention_dim: int = 3584, axes_dims_rope: tuple[int, int, int] = (16, 56, 56),
-                 mlp_ratio: int = 4, ref_rounding: bool = False):
+                 mlp_ratio: int = 4, ref_rounding: bool = False, fuse_epilogues: bool = True):
         super().__init__()
         self.in_channels = in_channels
         self.out_channels = out_channels or in_channels
@@ -329,7 +378,7 @@ class QwenImageTransformer2DModel(nn.Module):
         self.txt_in = nn.Linear(joint_attention_dim, self.inner_dim)
         self.transformer_blocks = nn.ModuleList([
             QwenImageTransformerBlock(self.inner_dim, num_attention_heads, attention_head_dim,
-                                      mlp_ratio=mlp_ratio, ref_rounding=ref_rounding)
+                                      mlp_ratio=mlp_ratio, ref_rounding=ref_rounding, fuse_epilogues=fuse_epilogues)
             for _ in range(num_layers)])
         self.norm_out = AdaLayerNormContinuous(self.inner_dim, self.inner_dim, eps=1e-6)
         self.proj_out = nn.Linear(self.inner_dim, patch_size * patch_size * self.out_channels, bias=True)
@@ -365,6 +414,20 @@ class QwenImageTransformer2DModel(nn.Module):
                     lin.weight.data = w_all[i, j]
                     lin.bias.data = b_all[i, j]
         self._mod_weight, self._mod_bias = w_all, b_all
+        # biases of the four gated output projections of every block, float32 [L, 2 (img, txt), 2, C]
+        self._res_bias = torch.stack([
+            torch.stack([torch.stack([blk.attn.to_out.bias, blk.img_mlp.net[2].bias]),
+                         torch.stack([blk.attn.to_add_out.bias, blk.txt_mlp.net[2].bias])])
+            for blk in self.transformer_blocks]).detach().float()
+
+    def all_gate_rows(self, mods: torch.Tensor | None):
+        """float32 (gates, gates * biases) [B, L, 2, 2, C] of the four gated projections of every block,
+        from the stacked modulation parameters: two small elementwise ops per step."""
+        if mods is None or getattr(self, "_res_bias", None) is None:
+            return None
+        B, L, C = mods.shape[0], mods.shape[1], self.inner_dim
+        gates = mods.view(B, L, 2, 2, 3 * C)[..., 2 * C:].float()
+        return gates, gates * self._res_bias
 
     def all_modulations(self, temb: torch.Tensor) -> torch.Tensor | None:
         """[B, L, 2, 6C] modulation parameters of every block, or None when not fused."""
@@ -380,11 +443,13 @@ class QwenImageTransformer2DModel(nn.Module):
         if mask is not None and bool(mask.all()):
             mask = None  # all-true masks are dropped (qit.py:1044-1048)
         mods = self.all_modulations(temb)
+        rows = self.all_gate_rows(mods)
         for i, block in enumerate(self.transformer_blocks):
             mp = (mods[:, i, 0], mods[:, i, 1]) if mods is not None else None
+            gr = (rows[0][:, i], rows[1][:, i]) if rows is not None else None
             txt, img = block(hidden_states=img, encoder_hidden_states=txt, encoder_hidden_states_mask=mask,
                              temb=temb, image_rotary_emb=rotary, joint_attention_kwargs=attention_kwargs,
-                             mod_params=mp)
+                             mod_params=mp, gate_rows=gr)
         return img, txt
 
     def finish(self, img, temb, return_dict: bool = True):

@@ -33,7 +33,8 @@ import torch.nn.functional as F
 from .. import kernels
 from .._lib import ODIT_NORM_ROW
 from ..attention.layer import Attention
-from .qwen_image import ApproxGELU, TimestepEmbedding, Transformer2DModelOutput, QwenTimestepProjEmbeddings
+from .qwen_image import (ApproxGELU, QwenTimestepProjEmbeddings, TimestepEmbedding, Transformer2DModelOutput,
+                         project_residual)
 
 
 class DistributedRMSNorm(nn.Module):
@@ -141,7 +142,10 @@ class WanSelfAttention(nn.Module):
         self.attn = Attention(num_heads=num_heads, head_size=head_dim, num_kv_heads=num_heads,
                               softmax_scale=1.0 / (head_dim ** 0.5), causal=False)
 
-    def forward(self, hidden_states: torch.Tensor, rotary_emb=None) -> torch.Tensor:
+    def forward(self, hidden_states: torch.Tensor, rotary_emb=None, residual: torch.Tensor | None = None,
+                gate: torch.Tensor | None = None) -> torch.Tensor:
+        """With ``residual``: residual + gate * attention output (a new tensor), formed in the output
+        projection's epilogue."""
         rot = _rotary(rotary_emb)
         B, S, _ = hidden_states.shape
         H, D = self.num_heads, self.head_dim
@@ -151,7 +155,10 @@ class WanSelfAttention(nn.Module):
         cos, sin = (rot.cos32, rot.sin32) if rot is not None else (None, None)
         kernels.qknorm_rope(qkv[:, :, 0], qkv[:, :, 1], None, q, k, None, self.norm_q.weight, self.norm_k.weight,
                             cos, sin, eps=self.norm_q.eps, norm_mode=ODIT_NORM_ROW)
-        return self.to_out(self.attn(q, k, qkv[:, :, 2]).flatten(2, 3))
+        o = self.attn(q, k, qkv[:, :, 2]).flatten(2, 3)
+        if residual is not None:
+            return project_residual(self.to_out, o, residual, gate)
+        return self.to_out(o)
 
 
 class WanCrossAttention(nn.Module):
@@ -173,7 +180,9 @@ class WanCrossAttention(nn.Module):
         self.attn = Attention(num_heads=num_heads, head_size=head_dim, num_kv_heads=num_heads,
                               softmax_scale=1.0 / (head_dim ** 0.5), causal=False)
 
-    def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor) -> torch.Tensor:
+    def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor,
+                residual: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+        """With ``residual``: residual + attention output (written to ``out`` when given)."""
         B, S, _ = hidden_states.shape
         T = encoder_hidden_states.shape[1]
         H, D = self.num_heads, self.head_dim
@@ -185,7 +194,10 @@ class WanCrossAttention(nn.Module):
         kernels.qknorm_rope(k_in, None, None, k, None, None, self.norm_k.weight, None, None, None,
                             eps=self.norm_k.eps, norm_mode=ODIT_NORM_ROW)
         v = self.to_v(encoder_hidden_states).view(B, T, H, D)
-        return self.to_out(self.attn(q, k, v).flatten(2, 3))
+        o = self.attn(q, k, v).flatten(2, 3)
+        if residual is not None:
+            return project_residual(self.to_out, o, residual, None, out=out)
+        return self.to_out(o)
 
 
 class FP32LayerNorm(nn.LayerNorm):
@@ -229,15 +241,15 @@ class WanTransformerBlock(nn.Module):
         shift_msa, scale_msa, gate_msa, c_shift, c_scale, c_gate = (mod[:, i] for i in range(6))
         x = hidden_states
         n = kernels.adaln_modulate(x, shift_msa, scale_msa, eps=self.eps)
-        x = kernels.gated_residual(x, self.attn1(n, rotary_emb), gate_msa)   # new tensor: the input is not written
+        x = self.attn1(n, rotary_emb, residual=x, gate=gate_msa)   # new tensor: the input is not written
         if isinstance(self.norm2, nn.Identity):
             n = x
         else:
             lw, lb = self._norm2_affine()
             n = kernels.adaln_modulate(x, None, None, eps=self.eps, ln_weight=lw, ln_bias=lb, out=n)
-        x = kernels.gated_residual(x, self.attn2(n, encoder_hidden_states), None, out=x)
+        x = self.attn2(n, encoder_hidden_states, residual=x, out=x)
         n = kernels.adaln_modulate(x, c_shift, c_scale, eps=self.eps, out=n if n is not x else None)
-        return kernels.gated_residual(x, self.ffn(n), c_gate, out=x)
+        return project_residual(self.ffn.net_2, self.ffn.net_0(n), x, c_gate, out=x)
 
 
 class PixArtAlphaTextProjection(nn.Module):

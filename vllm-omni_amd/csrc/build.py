@@ -34,7 +34,11 @@ UNITS: list[tuple[str, list[str], str]] = [
     ("qknorm_rope.hip", ["-DODIT_QK_TU=2"], "qknorm_rope_f32"),
     ("attn_fwd.hip", [], "attn_fwd"),
     ("attn_fwd_dma.hip", [], "attn_fwd_dma"),
+    ("linear.hip", [], "linear"),
 ]
+
+# the dense projections call hipBLASLt (its MFMA GEMM kernels); everything else is self-contained
+LINK_LIBS = ["-L/opt/rocm/lib", "-lhipblaslt"]
 
 # -packed-fp32-ops is switched off on purpose: v_pk_*_f32 forms are not trusted on this target.
 HIPCC_FLAGS = [
@@ -91,7 +95,7 @@ def build(force: bool = False, jobs: int | None = None, verbose: bool = True) ->
         list(ex.map(_run, work))
     if work or force or not LIB_PATH.exists():
         tmp = LIB_PATH.with_suffix(".so.tmp")
-        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)])
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs), *LINK_LIBS])
         os.replace(tmp, LIB_PATH)
     if verbose:
         print(f"[omni_dit build] {LIB_PATH} ({LIB_PATH.stat().st_size} bytes)", flush=True)

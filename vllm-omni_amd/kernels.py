@@ -12,6 +12,12 @@ import torch
 
 from . import _lib
 from ._lib import (
+    ODIT_EPI_BIAS,
+    ODIT_EPI_BIAS_GELU_TANH,
+    ODIT_EPI_GATED_RESIDUAL,
+    ODIT_EPI_GATED_RESIDUAL_PRE,
+    ODIT_EPI_GELU_TANH,
+    ODIT_EPI_NONE,
     ODIT_BF16,
     ODIT_F16,
     ODIT_F32,
@@ -379,3 +385,168 @@ def gelu_tanh(x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
 
 def silu(x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     return _unary("odit_silu", x, out)
+
+
+# --------------------------------------------------------------------------------------------- GEMM
+_LINEAR_SCRATCH: dict[tuple[int, int], torch.Tensor] = {}
+_LINEAR_AUTOTUNE_ITERS = 0
+_LINEAR_TUNED: dict[tuple, float] = {}
+
+
+_FLUSH_BYTES = 512 << 20  # twice the 256 MB last-level cache
+_FLUSH: dict[int, torch.Tensor] = {}
+
+
+def _flush_buffer(device: torch.device) -> int:
+    """Device buffer the tuning call overwrites between timed launches; released by set_linear_autotune(0)."""
+    idx = device.index or 0
+    if idx not in _FLUSH:
+        _FLUSH[idx] = torch.empty(_FLUSH_BYTES, dtype=torch.uint8, device=device)
+    return _FLUSH[idx].data_ptr()
+
+
+def set_linear_autotune(iters: int) -> None:
+    """With iters > 0, the first ``linear`` call of every new problem (shape, strides, epilogue, dtype)
+    first times the library's kernels for it on scratch copies of the output operands (a blocking,
+    one-off cost of some tenths of a second) and keeps the fastest for the rest of the process. Meant to
+    be switched on around a warm-up pass and off again; 0 = use the library's own first choice for
+    problems not tuned yet."""
+    global _LINEAR_AUTOTUNE_ITERS
+    _LINEAR_AUTOTUNE_ITERS = int(iters)
+    if _LINEAR_AUTOTUNE_ITERS <= 0:
+        _FLUSH.clear()
+
+
+def linear_tuning_report() -> dict[tuple, float]:
+    """{problem key: best time in microseconds} of everything tuned so far in this process."""
+    return dict(_LINEAR_TUNED)
+
+
+def _linear_workspace(lib, device: torch.device) -> torch.Tensor:
+    key = (device.index or 0, _stream())
+    ws = _LINEAR_SCRATCH.get(key)
+    if ws is None:
+        ws = torch.empty(int(lib.odit_linear_workspace_bytes()), dtype=torch.uint8, device=device)
+        _LINEAR_SCRATCH[key] = ws
+    return ws
+
+
+def _rows2d(t: torch.Tensor, name: str) -> tuple[torch.Tensor, int]:
+    """View of t as rows of its last axis with one row stride; returns (2-D view, row stride)."""
+    if t.stride(-1) != 1:
+        raise ValueError(f"{name}: last dimension must be contiguous")
+    t2 = t.reshape(-1, t.shape[-1]) if t.is_contiguous() else (t if t.dim() == 2 else None)
+    if t2 is None:
+        raise ValueError(f"{name}: needs a contiguous tensor or a 2-D view with a row stride")
+    return t2, (t2.stride(0) if t2.shape[0] > 1 else t2.shape[1])
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *, activation: str | None = None,
+           residual: torch.Tensor | None = None, gate: torch.Tensor | None = None, out: torch.Tensor | None = None,
+           gate_bias: torch.Tensor | None = None, prescaled: bool = False, tune_iters: int = 0):
+    """x W^T (+ bias) with the elementwise tail inside the GEMM's epilogue.
+
+    activation="gelu_tanh": GELU(tanh) of the result. residual (same shape as the result) with optional
+    gate [B,N] / [B,1,N] / [N]: ``residual + gate * (x W^T + bias)``; one GEMM per batch row when the gate
+    differs per batch row. ``prescaled=True``: ``gate`` is float32 and ``gate_bias`` (float32, same shape, or
+    None) already holds gate * bias — nothing is derived per call (``bias`` is then ignored).
+    ``weight`` may be a column range of a Linear weight (row stride > K).
+    ``tune_iters`` > 0 first times the library's kernels for this problem (overwrites ``out``) and
+    returns the best time in microseconds instead of the result.
+    """
+    _dev(x, weight, bias, residual, gate, out)
+    if weight.dim() != 2 or weight.stride(1) != 1 or x.shape[-1] != weight.shape[1]:
+        raise ValueError(f"weight must be [N,K] rows with K = {x.shape[-1]}, got {tuple(weight.shape)}")
+    if x.dtype != weight.dtype or (bias is not None and bias.dtype != x.dtype):
+        raise TypeError("x, weight and bias must share a dtype")
+    N, K = weight.shape
+    x2, ldx = _rows2d(x, "x")
+    M = x2.shape[0]
+    out_shape = (*x.shape[:-1], N)
+    if out is None:
+        out = torch.empty(out_shape, dtype=x.dtype, device=x.device)
+    elif tuple(out.shape) != out_shape or out.dtype != x.dtype:
+        raise ValueError(f"out must be {out_shape} of {x.dtype}")
+    o2, ldo = _rows2d(out, "out")
+    if bias is not None and (bias.numel() != N or not bias.is_contiguous()):
+        raise ValueError(f"bias must be contiguous [{N}]")
+    lib = _lib.load()
+    ws = _linear_workspace(lib, x.device)
+    ldw = weight.stride(0) if N > 1 else K
+    best = _lib.C.c_float(0.0)
+
+    def call(xp, op, rp, gp, m, epi, gate_code, bp=_ptr(bias)):
+        if _LINEAR_AUTOTUNE_ITERS > 0 and tune_iters == 0:
+            key = (x.device.index or 0, m, N, K, epi, bp is not None, gp is not None, _code(x), ldx, ldw, ldo, ldr)
+            if key not in _LINEAR_TUNED:
+                # time the candidates on scratch output operands: tuning overwrites (and, for the residual
+                # forms, keeps accumulating into) whatever it is given
+                t_out = torch.empty((m, ldo), dtype=x.dtype, device=x.device)
+                t_res = torch.zeros((m, max(ldr, 1)), dtype=x.dtype, device=x.device) if rp is not None else None
+                t_best = _lib.C.c_float(0.0)
+                _lib.check(lib.odit_linear_tune(xp, weight.data_ptr(), bp, t_out.data_ptr(), _ptr(t_res), gp, m, N, K,
+                                                ldx, ldw, ldo, ldr, epi, gate_code, _code(x), ws.data_ptr(),
+                                                ws.numel(), _stream(), _LINEAR_AUTOTUNE_ITERS, _flush_buffer(x.device),
+                                                _FLUSH_BYTES, _lib.C.byref(t_best)),
+                           "odit_linear_tune")
+                _LINEAR_TUNED[key] = t_best.value
+        args = (xp, weight.data_ptr(), bp, op, rp, gp, m, N, K, ldx, ldw, ldo, ldr, epi, gate_code, _code(x),
+                ws.data_ptr(), ws.numel(), _stream())
+        if tune_iters > 0:
+            _lib.check(lib.odit_linear_tune(*args, int(tune_iters), _flush_buffer(x.device), _FLUSH_BYTES,
+                                            _lib.C.byref(best)), "odit_linear_tune")
+        else:
+            _lib.check(lib.odit_linear(*args), "odit_linear")
+
+    ldr = 0
+    if residual is None:
+        if gate is not None:
+            raise ValueError("gate needs a residual")
+        if activation is None:
+            epi = ODIT_EPI_BIAS if bias is not None else ODIT_EPI_NONE
+        elif activation == "gelu_tanh":
+            epi = ODIT_EPI_BIAS_GELU_TANH if bias is not None else ODIT_EPI_GELU_TANH
+        else:
+            raise ValueError(f"unknown activation {activation!r}")
+        call(x2.data_ptr(), o2.data_ptr(), None, None, M, epi, _code(x))
+        return best.value if tune_iters > 0 else out
+    if activation is not None:
+        raise ValueError("activation and residual cannot be combined")
+    if tuple(residual.shape) != out_shape or residual.dtype != x.dtype:
+        raise ValueError(f"residual must be {out_shape} of {x.dtype}")
+    r2, ldr = _rows2d(residual, "residual")
+    esz = x.element_size()
+    if gate is None or gate.dim() == 1:
+        groups, rows, g2 = 1, M, (None if gate is None else gate.reshape(1, N))
+    else:
+        B = x.shape[0]
+        g2 = gate.reshape(B, N) if gate.numel() == B * N else None
+        if g2 is None or x.dim() < 2:
+            raise ValueError(f"gate shape {tuple(gate.shape)} does not give one row of {N} per batch row")
+        groups, rows = B, M // B
+    if g2 is not None:
+        _last_contig(g2, "gate")
+        if g2.dtype not in (x.dtype, torch.float32):
+            raise TypeError("gate must have x's dtype or float32")
+    gb2 = None
+    if prescaled:
+        if g2 is None or g2.dtype != torch.float32:
+            raise TypeError("prescaled=True needs a float32 gate")
+        if gate_bias is not None:
+            gb2 = gate_bias.reshape(g2.shape)
+            _last_contig(gb2, "gate_bias")
+            if gb2.dtype != torch.float32:
+                raise TypeError("gate_bias must be float32")
+    for b in range(groups):
+        off = b * rows
+        xp, op, rp = (x2.data_ptr() + off * ldx * esz, o2.data_ptr() + off * ldo * esz,
+                      r2.data_ptr() + off * ldr * esz)
+        if prescaled:
+            call(xp, op, rp, g2[b].data_ptr(), rows, ODIT_EPI_GATED_RESIDUAL_PRE, ODIT_F32,
+                 None if gb2 is None else gb2[b].data_ptr())
+        else:
+            call(xp, op, rp, None if g2 is None else g2[b].data_ptr(), rows, ODIT_EPI_GATED_RESIDUAL,
+                 _code(x) if g2 is None else _code(g2))
+        if tune_iters > 0:
+            break  # every batch row is the same problem
+    return best.value if tune_iters > 0 else out
