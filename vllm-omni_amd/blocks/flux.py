@@ -118,8 +118,9 @@ class FluxAttention(nn.Module):
 
     def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor | None = None,
                 image_rotary_emb=None, residuals=None, **kwargs):
-        """``residuals`` = (residual, gate, context_residual, context_gate) (dual blocks only): return
-        residual + gate * projection for both streams instead of the bare projections."""
+        """``residuals`` = (residual, gate, context_residual, context_gate[, pre, context_pre]) (dual blocks
+        only): return residual + gate * projection for both streams instead of the bare projections; the
+        ``pre`` pairs are caller-made float32 (gate, gate * bias) rows."""
         rot = _rotary(image_rotary_emb)
         B, S_x, _ = hidden_states.shape
         H, D = self.heads, self.head_dim
@@ -150,9 +151,11 @@ class FluxAttention(nn.Module):
                             norm_mode=ODIT_NORM_HEAD, ref_rounding=rr)
         ctx_attn, x_attn = self.attn(jq, jk, jv, AttentionMetadata(output_split=S_c))
         if residuals is not None:
-            res, gate, c_res, c_gate = residuals
-            return (project_residual(self.to_out[0], x_attn.flatten(2, 3), res, gate, ref_rounding=rr),
-                    project_residual(self.to_add_out, ctx_attn.flatten(2, 3), c_res, c_gate, ref_rounding=rr))
+            res, gate, c_res, c_gate = residuals[:4]
+            pre, c_pre = residuals[4:] if len(residuals) == 6 else (None, None)
+            return (project_residual(self.to_out[0], x_attn.flatten(2, 3), res, gate, ref_rounding=rr, pre=pre),
+                    project_residual(self.to_add_out, ctx_attn.flatten(2, 3), c_res, c_gate, ref_rounding=rr,
+                                     pre=c_pre))
         return self.to_out[0](x_attn.flatten(2, 3)), self.to_add_out(ctx_attn.flatten(2, 3))
 
 
@@ -176,10 +179,15 @@ class FluxTransformerBlock(nn.Module):
 
     def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, temb: torch.Tensor,
                 image_rotary_emb=None, joint_attention_kwargs: dict[str, Any] | None = None,
-                mod_params: tuple[torch.Tensor, torch.Tensor] | None = None):
+                mod_params: tuple[torch.Tensor, torch.Tensor] | None = None,
+                gate_rows: tuple[torch.Tensor, torch.Tensor] | None = None):
         """``mod_params`` = (norm1 [B,6C], norm1_context [B,6C]) when the caller projected ``temb`` for
-        all blocks at once; otherwise they are computed here as in the reference."""
+        all blocks at once; otherwise they are computed here as in the reference. ``gate_rows`` = float32
+        (gates, gates * biases), each [B, 2 (hidden, context), 2 (attention, feed-forward), C]."""
         rr = self.ref_rounding
+        pre = [[None, None], [None, None]]
+        if gate_rows is not None:
+            pre = [[(gate_rows[0][:, s, j], gate_rows[1][:, s, j]) for j in range(2)] for s in range(2)]
         m_x, m_c = mod_params if mod_params is not None else (None, None)
         n_x, gate_msa, shift_mlp, scale_mlp, gate_mlp = self.norm1(hidden_states, emb=temb, mod=m_x)
         n_c, c_gate_msa, c_shift_mlp, c_scale_mlp, c_gate_mlp = self.norm1_context(encoder_hidden_states,
@@ -188,13 +196,16 @@ class FluxTransformerBlock(nn.Module):
         # residuals land in new tensors, the feed-forward residuals then update those in place
         hidden_states, encoder_hidden_states = self.attn(
             hidden_states=n_x, encoder_hidden_states=n_c, image_rotary_emb=image_rotary_emb,
-            residuals=(hidden_states, gate_msa, encoder_hidden_states, c_gate_msa), **(joint_attention_kwargs or {}))
+            residuals=(hidden_states, gate_msa, encoder_hidden_states, c_gate_msa, pre[0][0], pre[1][0]),
+            **(joint_attention_kwargs or {}))
         n2 = kernels.adaln_modulate(hidden_states, shift_mlp, scale_mlp, eps=self.norm2.eps, ref_rounding=rr)
-        hidden_states = self.ff.forward_residual(n2, hidden_states, gate_mlp, out=hidden_states, ref_rounding=rr)
+        hidden_states = self.ff.forward_residual(n2, hidden_states, gate_mlp, out=hidden_states, ref_rounding=rr,
+                                                 pre=pre[0][1])
         c2 = kernels.adaln_modulate(encoder_hidden_states, c_shift_mlp, c_scale_mlp, eps=self.norm2_context.eps,
                                     ref_rounding=rr)
         encoder_hidden_states = self.ff_context.forward_residual(c2, encoder_hidden_states, c_gate_mlp,
-                                                                 out=encoder_hidden_states, ref_rounding=rr)
+                                                                 out=encoder_hidden_states, ref_rounding=rr,
+                                                                 pre=pre[1][1])
         if encoder_hidden_states.dtype == torch.float16:
             encoder_hidden_states = encoder_hidden_states.clip(-65504, 65504)
         return encoder_hidden_states, hidden_states
@@ -218,7 +229,9 @@ class FluxSingleTransformerBlock(nn.Module):
         self.ref_rounding = ref_rounding
 
     def forward_joint(self, x: torch.Tensor, temb: torch.Tensor, image_rotary_emb=None,
-                      mod: torch.Tensor | None = None, in_place: bool = False) -> torch.Tensor:
+                      mod: torch.Tensor | None = None, in_place: bool = False,
+                      gate_rows: tuple[torch.Tensor, torch.Tensor] | None = None) -> torch.Tensor:
+        """``gate_rows`` = float32 (gate [B,C], gate * proj_out.bias [B,C]) made by the caller."""
         B, S, C = x.shape
         n, gate = self.norm(x, emb=temb, mod=mod)
         fused = not self.ref_rounding and x.dtype != torch.float32
@@ -231,7 +244,11 @@ class FluxSingleTransformerBlock(nn.Module):
         # gate * proj_out(cat([att, mlp], -1)) + x as two GEMMs over the two column ranges of the weight,
         # each accumulating onto the residual stream through its epilogue
         w = self.proj_out.weight
-        if fused:
+        if fused and gate_rows is not None:
+            out = kernels.linear(mlp, w[:, C:], None, residual=x, gate=gate_rows[0], gate_bias=gate_rows[1],
+                                 prescaled=True, out=x if in_place else None)
+            out = kernels.linear(att, w[:, :C], None, residual=out, gate=gate_rows[0], prescaled=True, out=out)
+        elif fused:
             out = kernels.linear(mlp, w[:, C:], self.proj_out.bias, residual=x, gate=gate, out=x if in_place else None)
             out = kernels.linear(att, w[:, :C], None, residual=out, gate=gate, out=out)
         else:
@@ -367,6 +384,29 @@ class FluxTransformer2DModel(nn.Module):
                 l.weight.data, l.bias.data = w_all[r:r + n], b_all[r:r + n]
                 r += n
         self._mod_weight, self._mod_bias = w_all, b_all
+        # float32 biases of the gated output projections: dual [L, 2 (hidden, context), 2, C], single [Ls, C]
+        self._res_bias_dual = torch.stack([
+            torch.stack([torch.stack([blk.attn.to_out[0].bias, blk.ff.net[2].bias]),
+                         torch.stack([blk.attn.to_add_out.bias, blk.ff_context.net[2].bias])])
+            for blk in self.transformer_blocks]).detach().float() if len(self.transformer_blocks) else None
+        self._res_bias_single = torch.stack([blk.proj_out.bias for blk in self.single_transformer_blocks]
+                                            ).detach().float() if len(self.single_transformer_blocks) else None
+
+    def all_gate_rows(self, mods):
+        """float32 (gates, gates * biases) of every gated projection, two small elementwise ops per step:
+        dual [B, L, 2, 2, C] pairs and single [B, Ls, C] pairs (None where there are no such blocks)."""
+        if mods is None or not hasattr(self, "_res_bias_dual") or next(self.parameters()).dtype == torch.float32:
+            return None, None
+        C = self.inner_dim
+        dual = single = None
+        if self._res_bias_dual is not None:
+            B, L = mods[0].shape[:2]
+            g = mods[0].view(B, L, 2, 2, 3 * C)[..., 2 * C:].float()
+            dual = (g, g * self._res_bias_dual)
+        if self._res_bias_single is not None:
+            g = mods[1][..., 2 * C:].float()
+            single = (g, g * self._res_bias_single)
+        return dual, single
 
     def all_modulations(self, temb: torch.Tensor):
         """(dual [B, L, 2, 6C], single [B, Ls, 3C]) or None when not fused."""
@@ -380,16 +420,20 @@ class FluxTransformer2DModel(nn.Module):
 
     def run_blocks(self, img, txt, temb, rotary, joint_attention_kwargs=None):
         mods = self.all_modulations(temb)
+        dual_rows, single_rows = self.all_gate_rows(mods)
         for i, block in enumerate(self.transformer_blocks):
             mp = (mods[0][:, i, 0], mods[0][:, i, 1]) if mods is not None else None
+            gr = (dual_rows[0][:, i], dual_rows[1][:, i]) if dual_rows is not None else None
             txt, img = block(hidden_states=img, encoder_hidden_states=txt, temb=temb, image_rotary_emb=rotary,
-                             joint_attention_kwargs=joint_attention_kwargs, mod_params=mp)
+                             joint_attention_kwargs=joint_attention_kwargs, mod_params=mp, gate_rows=gr)
         if len(self.single_transformer_blocks) == 0:
             return img, txt
         n_txt = txt.shape[1]
         x = torch.cat([txt, img], dim=1)  # once for the whole single-stream stack
         for i, block in enumerate(self.single_transformer_blocks):
-            x = block.forward_joint(x, temb, rotary, mod=mods[1][:, i] if mods is not None else None, in_place=True)
+            gr = (single_rows[0][:, i], single_rows[1][:, i]) if single_rows is not None else None
+            x = block.forward_joint(x, temb, rotary, mod=mods[1][:, i] if mods is not None else None, in_place=True,
+                                    gate_rows=gr)
         return x[:, n_txt:], x[:, :n_txt]
 
     def finish(self, img, temb, return_dict: bool = True):

@@ -423,7 +423,7 @@ class QwenImageTransformer2DModel(nn.Module):
     def all_gate_rows(self, mods: torch.Tensor | None):
         """float32 (gates, gates * biases) [B, L, 2, 2, C] of the four gated projections of every block,
         from the stacked modulation parameters: two small elementwise ops per step."""
-        if mods is None or getattr(self, "_res_bias", None) is None:
+        if mods is None or getattr(self, "_res_bias", None) is None or mods.dtype == torch.float32:
             return None
         B, L, C = mods.shape[0], mods.shape[1], self.inner_dim
         gates = mods.view(B, L, 2, 2, 3 * C)[..., 2 * C:].float()

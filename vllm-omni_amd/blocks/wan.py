@@ -143,9 +143,9 @@ class WanSelfAttention(nn.Module):
                               softmax_scale=1.0 / (head_dim ** 0.5), causal=False)
 
     def forward(self, hidden_states: torch.Tensor, rotary_emb=None, residual: torch.Tensor | None = None,
-                gate: torch.Tensor | None = None) -> torch.Tensor:
+                gate: torch.Tensor | None = None, pre=None) -> torch.Tensor:
         """With ``residual``: residual + gate * attention output (a new tensor), formed in the output
-        projection's epilogue."""
+        projection's epilogue; ``pre`` = caller-made float32 (gate, gate * bias) rows."""
         rot = _rotary(rotary_emb)
         B, S, _ = hidden_states.shape
         H, D = self.num_heads, self.head_dim
@@ -157,7 +157,7 @@ class WanSelfAttention(nn.Module):
                             cos, sin, eps=self.norm_q.eps, norm_mode=ODIT_NORM_ROW)
         o = self.attn(q, k, qkv[:, :, 2]).flatten(2, 3)
         if residual is not None:
-            return project_residual(self.to_out, o, residual, gate)
+            return project_residual(self.to_out, o, residual, gate, pre=pre)
         return self.to_out(o)
 
 
@@ -231,9 +231,11 @@ class WanTransformerBlock(nn.Module):
         return self._ln2_f32[1], self._ln2_f32[2]
 
     def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, temb: torch.Tensor,
-                rotary_emb=None, mod: torch.Tensor | None = None) -> torch.Tensor:
+                rotary_emb=None, mod: torch.Tensor | None = None,
+                gate_bias: torch.Tensor | None = None) -> torch.Tensor:
         """``mod`` = float32 [B, 6, C] = scale_shift_table + temb when the caller formed it for all
-        blocks at once; otherwise it is formed here as in the reference."""
+        blocks at once; otherwise it is formed here as in the reference. ``gate_bias`` = float32 [B, 2, C]:
+        the two gates times the biases of the projections they scale (attn1.to_out, ffn.net_2)."""
         if temb is not None and temb.ndim == 4:
             raise NotImplementedError("per-token timesteps (temb [B,S,6,C]) are not built")
         if mod is None:
@@ -241,7 +243,9 @@ class WanTransformerBlock(nn.Module):
         shift_msa, scale_msa, gate_msa, c_shift, c_scale, c_gate = (mod[:, i] for i in range(6))
         x = hidden_states
         n = kernels.adaln_modulate(x, shift_msa, scale_msa, eps=self.eps)
-        x = self.attn1(n, rotary_emb, residual=x, gate=gate_msa)   # new tensor: the input is not written
+        pre1 = (gate_msa, gate_bias[:, 0]) if gate_bias is not None else None
+        pre2 = (c_gate, gate_bias[:, 1]) if gate_bias is not None else None
+        x = self.attn1(n, rotary_emb, residual=x, gate=gate_msa, pre=pre1)   # new tensor: the input is not written
         if isinstance(self.norm2, nn.Identity):
             n = x
         else:
@@ -249,7 +253,7 @@ class WanTransformerBlock(nn.Module):
             n = kernels.adaln_modulate(x, None, None, eps=self.eps, ln_weight=lw, ln_bias=lb, out=n)
         x = self.attn2(n, encoder_hidden_states, residual=x, out=x)
         n = kernels.adaln_modulate(x, c_shift, c_scale, eps=self.eps, out=n if n is not x else None)
-        return project_residual(self.ffn.net_2, self.ffn.net_0(n), x, c_gate, out=x)
+        return project_residual(self.ffn.net_2, self.ffn.net_0(n), x, c_gate, out=x, pre=pre2)
 
 
 class PixArtAlphaTextProjection(nn.Module):
@@ -360,8 +364,12 @@ class WanTransformer3DModel(nn.Module):
 
     def run_blocks(self, x, ctx, timestep_proj, rotary):
         mods = self.all_modulations(timestep_proj)
+        gb = None
+        if x.dtype != torch.float32:  # gates (rows 2 and 5) times the biases they scale, [L, B, 2, C]
+            biases = torch.stack([torch.stack([blk.attn1.to_out.bias, blk.ffn.net_2.bias]) for blk in self.blocks])
+            gb = mods[:, :, 2::3] * biases.float().unsqueeze(1)
         for i, block in enumerate(self.blocks):
-            x = block(x, ctx, None, rotary, mod=mods[i])
+            x = block(x, ctx, None, rotary, mod=mods[i], gate_bias=None if gb is None else gb[i])
         return x
 
     def finish(self, x: torch.Tensor, temb: torch.Tensor, grid: tuple[int, int, int], return_dict: bool = True):
