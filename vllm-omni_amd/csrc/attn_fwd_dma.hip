@@ -79,8 +79,15 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   // buffer descriptors end right after the last valid key row: later rows read as zeros
   const uint32_t k_bytes = static_cast<uint32_t>(((p.Sk - 1) * p.ks_s + D) * 2);
   const uint32_t v_bytes = static_cast<uint32_t>(((p.Sk - 1) * p.vs_s + D) * 2);
-  const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(kbase), 0, k_bytes, 0x00020000);
-  const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(vbase), 0, v_bytes, 0x00020000);
+  // raw buffer descriptors {base[31:0], base[47:32] (stride 0), bytes, dword3 = 0x00020000}
+  auto make_rsrc = [](const void* base, uint32_t bytes) {
+    const uint64_t a = reinterpret_cast<uint64_t>(base);
+    u32x4_v r;
+    r.x = static_cast<uint32_t>(a); r.y = static_cast<uint32_t>(a >> 32) & 0xffffu; r.z = bytes; r.w = 0x00020000u;
+    return r;
+  };
+  const u32x4_v krsrc = make_rsrc(kbase, k_bytes);
+  const u32x4_v vrsrc = make_rsrc(vbase, v_bytes);
 
   // per-lane global byte offsets of the chunks this lane moves, relative to the tile's first row
   uint32_t kvoff[IPW], vvoff[IPW];
@@ -94,12 +101,23 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   const uint32_t k_tile_step = static_cast<uint32_t>(BN * p.ks_s * 2);
   const uint32_t v_tile_step = static_cast<uint32_t>(BN * p.vs_s * 2);
 
-  auto dma_tile = [&](const __amdgpu_buffer_rsrc_t& rsrc, const uint32_t(&voff)[IPW], uint32_t soff, char* dst) {
-#if defined(__HIP_DEVICE_COMPILE__)  // the host pass cannot parse this builtin and would drop the kernel stub
+  // The tile loads are written as inline assembly on purpose. Issued through the compiler's builtin they
+  // are known to it as pending LDS writes, and it then puts `s_waitcnt vmcnt(0)` in front of the first V
+  // fragment read of every tile (it cannot prove that the XOR-swizzled read addresses miss the buffer
+  // being filled): the loads issued at the top of a tile, meant to land a whole tile later, were waited
+  // for half a tile after issue. Here the ordering is explicit instead: one `s_waitcnt vmcnt(0)` and one
+  // barrier at the end of each tile, before any wave reads the buffers those loads filled.
+  auto dma_tile = [&](const u32x4_v& rsrc, const uint32_t(&voff)[IPW], uint32_t soff, char* dst) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_p)(dst + wave * IPW * 1024)));
 #pragma unroll
-    for (int i = 0; i < IPW; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_p)(dst + (wave * IPW + i) * 1024), 16, voff[i],
-                                               soff, 0, 0);
+    for (int i = 0; i < IPW; ++i) {
+      const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds0 + i * 1024);
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                   :
+                   : "s"(m0v), "v"(voff[i]), "s"(rsrc), "s"(soff)
+                   : "memory", "m0");
+    }
 #endif
   };
 
