@@ -320,6 +320,34 @@ def kernel_rooflines(torch):
     return out
 
 
+def mfma_ceiling(torch):
+    """Sustained rate of the bf16 MFMA this path uses with nothing else in the loop, for constant and for
+    random operand data (the part is power-limited: the two differ by about 30 %)."""
+    import ctypes as C
+
+    from vllm_omni_amd import _lib
+
+    lib = _lib.load()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    sink = torch.empty(cus * 512, device="cuda", dtype=torch.float32)
+    st = torch.cuda.current_stream().cuda_stream
+    out = {}
+    for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
+        flop = C.c_double(0.0)
+        _lib.check(lib.odit_probe_mfma(rnd, 2000, cus, sink.data_ptr(), C.byref(flop), st), "odit_probe_mfma")
+        torch.cuda.synchronize()
+        best = 0.0
+        for _ in range(3):
+            a, b = _events(torch)
+            a.record()
+            _lib.check(lib.odit_probe_mfma(rnd, 20000, cus, sink.data_ptr(), C.byref(flop), st), "odit_probe_mfma")
+            b.record()
+            torch.cuda.synchronize()
+            best = max(best, flop.value / a.elapsed_time(b) / 1e9)
+        out[name] = {"TFLOP/s": best, "frac_of_nominal_peak": best / PEAK_MFMA_BF16_TFLOPS}
+    return out
+
+
 def cpu_baseline(torch):
     """The CPU oracle (plain-torch restatement of the reference path) on the host cores: ONE block of
     the 60 at the full B=2 shape in fp32, extrapolated to a step."""
@@ -468,6 +496,9 @@ def main():
     if not args.no_kernels:
         with torch.inference_mode():
             result["kernels"] = kernel_rooflines(torch)
+            result["mfma_ceiling"] = mfma_ceiling(torch)
+            result["roofline"]["frac_of_measured_mfma_ceiling_random_data"] = (
+                attn_tflops / result["mfma_ceiling"]["random_operands"]["TFLOP/s"])
     del model
     torch.cuda.empty_cache()
     if not args.no_cpu:

@@ -252,6 +252,15 @@ int odit_linear_tune(const void* x, const void* w, const void* bias, void* out, 
                      int epilogue, int gate_dtype, int dtype, void* workspace, size_t workspace_bytes,
                      void* stream, int iters, void* flush, size_t flush_bytes, float* best_us);
 
+/* ---------------------------------------------------------------------------------------------
+ * Roofline calibration (no counterpart in the reference): launches `workgroups` workgroups of 8
+ * wavefronts that issue nothing but v_mfma_f32_32x32x16_bf16 (iters x 8 per wavefront) on register
+ * operands holding constant (random_operands = 0) or pseudo-random data, writes one float per thread to
+ * `sink` (workgroups * 512 floats) and returns the flop count of the launch in *flop. Timed by the
+ * caller with events on `stream`: the sustained matrix rate of the device for that kind of data.
+ */
+int odit_probe_mfma(int random_operands, int iters, int workgroups, float* sink, double* flop, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

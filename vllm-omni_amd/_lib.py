@@ -75,6 +75,7 @@ _SIGNATURES = {
          C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p,
          C.c_int, C.c_void_p, C.c_size_t, C.POINTER(C.c_float)],
     ),
+    "odit_probe_mfma": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double), C.c_void_p]),
     "odit_gelu_tanh": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p]),
     "odit_silu": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p]),
 }

@@ -35,6 +35,7 @@ UNITS: list[tuple[str, list[str], str]] = [
     ("attn_fwd.hip", [], "attn_fwd"),
     ("attn_fwd_dma.hip", [], "attn_fwd_dma"),
     ("linear.hip", [], "linear"),
+    ("probe.hip", [], "probe"),
 ]
 
 # the dense projections call hipBLASLt (its MFMA GEMM kernels); everything else is self-contained
