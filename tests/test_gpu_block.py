@@ -159,6 +159,24 @@ def test_fused_modulation_is_bit_identical(gpu):
     assert (after.float() - before.float()).abs().max().item() <= 2e-2 and _cosine(after, before) >= 0.9999
 
 
+def test_weights_loaded_after_fusing_are_used(gpu):
+    """fuse_modulation() stacks weights and the model caches float32 copies of the gated projections' biases;
+    loading another state afterwards must be picked up by both."""
+    cfg, w, model = _build(gpu, seed=0)
+    lat, txt, t = _inputs(2, seed=12)
+    args = (lat.to(gpu), txt.to(gpu), None, t.to(gpu), [IMG_SHAPE], [S_TXT])
+    model.fuse_modulation()
+    with torch.inference_mode():
+        model(*args)                                   # populates the caches with the seed-0 biases
+    w2 = {k: v.bfloat16() for k, v in oq.init_params(cfg, seed=5, bias_std=0.05).items()}
+    model.load_flat_state(w2)
+    _, _, fresh = _build(gpu, seed=5, bias_std=0.05)
+    with torch.inference_mode():
+        got = model(*args).sample
+        want = fresh(*args).sample
+    assert (got.float() - want.float()).abs().max().item() <= 2e-2 and _cosine(got, want) >= 0.9999
+
+
 def test_cfg_batched_equals_sequential(gpu):
     cfg, w, model = _build(gpu)
     lat, _, _ = _inputs(1, seed=5)

@@ -346,6 +346,7 @@ class FluxTransformer2DModel(nn.Module):
         self.proj_out = nn.Linear(self.inner_dim, patch_size * patch_size * self.out_channels, bias=True)
         self.parallel_config = None
         self.do_true_cfg = False
+        self._res_bias = None
 
     # -- stages ---------------------------------------------------------------------------------
     def prepare(self, hidden_states, encoder_hidden_states, pooled_projections, timestep, img_ids, txt_ids,
@@ -384,28 +385,38 @@ class FluxTransformer2DModel(nn.Module):
                 l.weight.data, l.bias.data = w_all[r:r + n], b_all[r:r + n]
                 r += n
         self._mod_weight, self._mod_bias = w_all, b_all
-        # float32 biases of the gated output projections: dual [L, 2 (hidden, context), 2, C], single [Ls, C]
-        self._res_bias_dual = torch.stack([
-            torch.stack([torch.stack([blk.attn.to_out[0].bias, blk.ff.net[2].bias]),
-                         torch.stack([blk.attn.to_add_out.bias, blk.ff_context.net[2].bias])])
-            for blk in self.transformer_blocks]).detach().float() if len(self.transformer_blocks) else None
-        self._res_bias_single = torch.stack([blk.proj_out.bias for blk in self.single_transformer_blocks]
-                                            ).detach().float() if len(self.single_transformer_blocks) else None
+        self._res_bias = None
+
+    def _gated_biases(self):
+        """float32 biases of the gated output projections, dual [L, 2 (hidden, context), 2, C] and single
+        [Ls, C] (None where there are no such blocks); rebuilt when any of them has been written since."""
+        dual = [p for blk in self.transformer_blocks
+                for p in (blk.attn.to_out[0].bias, blk.ff.net[2].bias, blk.attn.to_add_out.bias, blk.ff_context.net[2].bias)]
+        single = [blk.proj_out.bias for blk in self.single_transformer_blocks]
+        ps = dual + single
+        tag = (sum(p._version for p in ps), ps[0].device, ps[0].dtype)
+        if self._res_bias is None or self._res_bias[0] != tag:
+            C = self.inner_dim
+            d = torch.stack(dual).detach().float().view(len(self.transformer_blocks), 2, 2, C) if dual else None
+            sgl = torch.stack(single).detach().float() if single else None
+            self._res_bias = (tag, d, sgl)
+        return self._res_bias[1], self._res_bias[2]
 
     def all_gate_rows(self, mods):
         """float32 (gates, gates * biases) of every gated projection, two small elementwise ops per step:
         dual [B, L, 2, 2, C] pairs and single [B, Ls, C] pairs (None where there are no such blocks)."""
-        if mods is None or not hasattr(self, "_res_bias_dual") or next(self.parameters()).dtype == torch.float32:
+        if mods is None or mods[0].dtype == torch.float32:
             return None, None
         C = self.inner_dim
+        bias_dual, bias_single = self._gated_biases()
         dual = single = None
-        if self._res_bias_dual is not None:
+        if bias_dual is not None:
             B, L = mods[0].shape[:2]
             g = mods[0].view(B, L, 2, 2, 3 * C)[..., 2 * C:].float()
-            dual = (g, g * self._res_bias_dual)
-        if self._res_bias_single is not None:
+            dual = (g, g * bias_dual)
+        if bias_single is not None:
             g = mods[1][..., 2 * C:].float()
-            single = (g, g * self._res_bias_single)
+            single = (g, g * bias_single)
         return dual, single
 
     def all_modulations(self, temb: torch.Tensor):

@@ -383,6 +383,7 @@ class QwenImageTransformer2DModel(nn.Module):
         self.norm_out = AdaLayerNormContinuous(self.inner_dim, self.inner_dim, eps=1e-6)
         self.proj_out = nn.Linear(self.inner_dim, patch_size * patch_size * self.out_channels, bias=True)
         self.zero_cond_t = False
+        self._res_bias = None
         self.parallel_config = None
         self.do_true_cfg = False
 
@@ -414,20 +415,27 @@ class QwenImageTransformer2DModel(nn.Module):
                     lin.weight.data = w_all[i, j]
                     lin.bias.data = b_all[i, j]
         self._mod_weight, self._mod_bias = w_all, b_all
-        # biases of the four gated output projections of every block, float32 [L, 2 (img, txt), 2, C]
-        self._res_bias = torch.stack([
-            torch.stack([torch.stack([blk.attn.to_out.bias, blk.img_mlp.net[2].bias]),
-                         torch.stack([blk.attn.to_add_out.bias, blk.txt_mlp.net[2].bias])])
-            for blk in self.transformer_blocks]).detach().float()
+        self._res_bias = None
+
+    def _gated_biases(self) -> torch.Tensor:
+        """float32 [L, 2 (img, txt), 2 (attention, MLP), C]: biases of the four gated output projections
+        of every block; rebuilt when any of them has been written since (in-place loads bump _version)."""
+        ps = [p for blk in self.transformer_blocks
+              for p in (blk.attn.to_out.bias, blk.img_mlp.net[2].bias, blk.attn.to_add_out.bias, blk.txt_mlp.net[2].bias)]
+        tag = (sum(p._version for p in ps), ps[0].device, ps[0].dtype)
+        if self._res_bias is None or self._res_bias[0] != tag:
+            L, C = len(self.transformer_blocks), self.inner_dim
+            self._res_bias = (tag, torch.stack(ps).detach().float().view(L, 2, 2, C))
+        return self._res_bias[1]
 
     def all_gate_rows(self, mods: torch.Tensor | None):
         """float32 (gates, gates * biases) [B, L, 2, 2, C] of the four gated projections of every block,
         from the stacked modulation parameters: two small elementwise ops per step."""
-        if mods is None or getattr(self, "_res_bias", None) is None or mods.dtype == torch.float32:
+        if mods is None or mods.dtype == torch.float32:
             return None
         B, L, C = mods.shape[0], mods.shape[1], self.inner_dim
         gates = mods.view(B, L, 2, 2, 3 * C)[..., 2 * C:].float()
-        return gates, gates * self._res_bias
+        return gates, gates * self._gated_biases()
 
     def all_modulations(self, temb: torch.Tensor) -> torch.Tensor | None:
         """[B, L, 2, 6C] modulation parameters of every block, or None when not fused."""
