@@ -310,6 +310,13 @@ def kernel_rooflines(torch):
     ms = _time_op(torch, lambda: kernels.attn_fwd(q, k, v, sc))
     fl = 4.0 * B * HEADS * S * S * HEAD_DIM
     out["attn_fwd"] = {"ms": ms, "TFLOP/s": fl / ms / 1e9, "frac_mfma": fl / ms / 1e9 / PEAK_MFMA_BF16_TFLOPS}
+    # the same launch on constant inputs: the matrix pipe is power-limited, and operand data that does
+    # not toggle lets it hold its clock - the difference to the line above is the chip, not the kernel
+    q1 = torch.ones_like(q)
+    ms1 = _time_op(torch, lambda: kernels.attn_fwd(q1, q1, q1, sc))
+    out["attn_fwd_constant_inputs"] = {"ms": ms1, "TFLOP/s": fl / ms1 / 1e9,
+                                       "frac_mfma": fl / ms1 / 1e9 / PEAK_MFMA_BF16_TFLOPS}
+    del q1
     xm = torch.randn(B * S_IMG, C, device=dev, dtype=bf)
     wm = torch.randn(MLP_RATIO * C, C, device=dev, dtype=bf)
     bm = torch.zeros(MLP_RATIO * C, device=dev, dtype=bf)

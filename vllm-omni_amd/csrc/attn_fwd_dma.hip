@@ -20,6 +20,15 @@
 // barrier per tile, XCD-aware workgroup order) is as in attn_fwd_pipe_kernel.
 #include "attn_common.h"
 
+// LDS fragment reads issued ahead of the MFMA that consumes them (K: 16-byte reads, V: pairs of
+// transpose reads); overridable for tuning builds.
+#ifndef ODIT_ATTN_KPF
+#define ODIT_ATTN_KPF 3
+#endif
+#ifndef ODIT_ATTN_VPF
+#define ODIT_ATTN_VPF 3
+#endif
+
 namespace odit {
 
 typedef short s16x4_d __attribute__((ext_vector_type(4)));
@@ -237,7 +246,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int e = 0; e < 16; ++e) s_next[kt][e] = 0.f;
-      constexpr int KPF = 3;  // K fragments in flight ahead of the MFMA that consumes them
+      constexpr int KPF = ODIT_ATTN_KPF;  // K fragments in flight ahead of the MFMA that consumes them
       u32x4_v kfr[KPF + 1];
       auto k_fetch = [&](int i) {
         const int ks = i >> 1, kt = i & 1;
@@ -284,7 +293,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
     // S(j+1) — vector work with nothing to wait for — is placed in the shadow of these MFMAs.
     const char* vt_base = Vb + buf * TILEB;
     constexpr int NSTEP = 4 * DT;
-    constexpr int PF = 3;
+    constexpr int PF = ODIT_ATTN_VPF;
     s16x4_d vlo[PF + 1], vhi[PF + 1];
     auto v_fetch = [&](int step) {
       const int dt = step % DT, kt = (step / DT) >> 1, g2 = (step / DT) & 1;
