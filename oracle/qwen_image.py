@@ -117,20 +117,42 @@ def qwen_rope_freqs(cfg: QwenConfig, frame: int, height: int, width: int, txt_le
     """(vid_freqs [F*H*W, D/2], txt_freqs [txt_len, D/2]) complex64 with scale_rope=True: rows/cols
     are centred ([-ceil(n/2) .. -1, 0 .. floor(n/2)-1]), frame index starts at 0, and text positions
     start at max(H//2, W//2) on all three axes. qit.py:298-396."""
+    return qwen_rope_freqs_images(cfg, [(frame, height, width)], txt_len)
+
+
+def qwen_rope_freqs_images(cfg: QwenConfig, shapes, txt_len: int):
+    """The same tables for a sample made of several images (editing: source, then targets): image
+    number ``idx`` takes frame positions idx .. idx+frame-1, its rows and columns are centred on its own
+    grid, the token rows of all images are concatenated, and text positions start after the largest
+    half-extent of any image. qit.py:340-396."""
     a0, a1, a2 = cfg.axes_dims_rope
     pos = torch.arange(4096)
     neg = torch.arange(4096).flip(0) * -1 - 1
     pos_f = [_axis_freqs(pos, a, cfg.theta) for a in (a0, a1, a2)]
     neg_f = [_axis_freqs(neg, a, cfg.theta) for a in (a0, a1, a2)]
-    f_frame = pos_f[0][:frame].view(frame, 1, 1, -1).expand(frame, height, width, -1)
-    f_h = torch.cat([neg_f[1][-(height - height // 2):], pos_f[1][: height // 2]], dim=0)
-    f_h = f_h.view(1, height, 1, -1).expand(frame, height, width, -1)
-    f_w = torch.cat([neg_f[2][-(width - width // 2):], pos_f[2][: width // 2]], dim=0)
-    f_w = f_w.view(1, 1, width, -1).expand(frame, height, width, -1)
-    vid = torch.cat([f_frame, f_h, f_w], dim=-1).reshape(frame * height * width, -1).contiguous()
-    start = max(height // 2, width // 2)
+    vids, start = [], 0
+    for idx, (frame, height, width) in enumerate(shapes):
+        f_frame = pos_f[0][idx:idx + frame].view(frame, 1, 1, -1).expand(frame, height, width, -1)
+        f_h = torch.cat([neg_f[1][-(height - height // 2):], pos_f[1][: height // 2]], dim=0)
+        f_h = f_h.view(1, height, 1, -1).expand(frame, height, width, -1)
+        f_w = torch.cat([neg_f[2][-(width - width // 2):], pos_f[2][: width // 2]], dim=0)
+        f_w = f_w.view(1, 1, width, -1).expand(frame, height, width, -1)
+        vids.append(torch.cat([f_frame, f_h, f_w], dim=-1).reshape(frame * height * width, -1))
+        start = max(start, height // 2, width // 2)
     txt = torch.cat(pos_f, dim=1)[start:start + txt_len].contiguous()
-    return vid, txt
+    return torch.cat(vids, dim=0).contiguous(), txt
+
+
+def modulate_index(img_shapes) -> torch.Tensor:
+    """[B, S_img] int32 for the editing variant (``zero_cond_t``): 0 for the tokens of each sample's first
+    image, 1 for those of every later image; ``img_shapes`` = per sample a list of (frame, height,
+    width). qit.py:141-154."""
+    rows = []
+    for sample in img_shapes:
+        first = sample[0][0] * sample[0][1] * sample[0][2]
+        rest = sum(f * h * w for f, h, w in sample[1:])
+        rows.append([0] * first + [1] * rest)
+    return torch.tensor(rows, dtype=torch.int32)
 
 
 # ------------------------------------------------------------------------------------- forward
@@ -168,10 +190,14 @@ def feed_forward(w, pre, x):
 
 
 def block_forward(w, i: int, cfg: QwenConfig, img, txt, temb, vid_freqs, txt_freqs, key_mask=None,
-                  modulate_index=None):
-    """QwenImageTransformerBlock.forward, qit.py:746-814. Returns (txt, img) like the reference."""
+                  modulate_index=None, zero_cond_t: bool = False):
+    """QwenImageTransformerBlock.forward, qit.py:746-814. Returns (txt, img) like the reference.
+    With ``zero_cond_t`` temb is [2B, C] (real timestep rows, then timestep-zero rows): the image stream
+    picks per token through ``modulate_index``, the text stream uses the first half (qit.py:758-767)."""
     pre = f"transformer_blocks.{i}."
     img_mod = _lin(w, pre + "img_mod.1", F.silu(temb))
+    if zero_cond_t:
+        temb = torch.chunk(temb, 2, dim=0)[0]
     txt_mod = _lin(w, pre + "txt_mod.1", F.silu(temb))
     img_mod1, img_mod2 = img_mod.chunk(2, dim=-1)
     txt_mod1, txt_mod2 = txt_mod.chunk(2, dim=-1)
@@ -218,15 +244,24 @@ def modulated_input(w, cfg: QwenConfig, img, temb):
 
 
 def transformer_forward(w, cfg: QwenConfig, latents, text, timestep, img_shape, key_mask=None,
-                        collect_blocks: bool = False):
+                        collect_blocks: bool = False, zero_cond_t: bool = False):
     """QwenImageTransformer2DModel.forward, qit.py:951-1071. latents [B,S_img,in], text [B,S_txt,J],
-    timestep [B] in [0,1]; img_shape = (frame, height, width) of the patch grid."""
+    timestep [B] in [0,1]; img_shape = (frame, height, width) of the patch grid, or a list of them when the
+    sample is several images (rotary tables and, with ``zero_cond_t``, the per-token conditioning index
+    follow the first sample's list, like the reference's). ``zero_cond_t``: the timestep is doubled to
+    [t, 0*t] (qit.py:141-145), the head uses the first half of temb (qit.py:1062-1063)."""
+    shapes = [tuple(img_shape)] if isinstance(img_shape[0], int) else [tuple(s) for s in img_shape]
+    index = None
+    if zero_cond_t:
+        timestep = torch.cat([timestep, timestep * 0], dim=0)
+        index = modulate_index([shapes] * latents.shape[0]).to(latents.device)
     img, txt, temb = stem(w, cfg, latents, text, timestep)
-    vid_freqs, txt_freqs = qwen_rope_freqs(cfg, *img_shape, txt_len=text.shape[1])
+    vid_freqs, txt_freqs = qwen_rope_freqs_images(cfg, shapes, txt_len=text.shape[1])
     per_block = []
     for i in range(cfg.num_layers):
-        txt, img = block_forward(w, i, cfg, img, txt, temb, vid_freqs, txt_freqs, key_mask)
+        txt, img = block_forward(w, i, cfg, img, txt, temb, vid_freqs, txt_freqs, key_mask,
+                                 modulate_index=index, zero_cond_t=zero_cond_t)
         if collect_blocks:
             per_block.append((img, txt))
-    out = head(w, cfg, img, temb)
+    out = head(w, cfg, img, temb.chunk(2, dim=0)[0] if zero_cond_t else temb)
     return (out, per_block) if collect_blocks else out

@@ -21,7 +21,7 @@ def _cosine(a, b):
     return float(torch.dot(a, b) / (a.norm() * b.norm()))
 
 
-def _build(gpu, dtype=torch.bfloat16, seed=0, bias_std=0.02, ref_rounding=False):
+def _build(gpu, dtype=torch.bfloat16, seed=0, bias_std=0.02, ref_rounding=False, **model_kwargs):
     from vllm_omni_amd.attention.selector import get_attn_backend
     from vllm_omni_amd.blocks.qwen_image import QwenImageTransformer2DModel
 
@@ -33,7 +33,7 @@ def _build(gpu, dtype=torch.bfloat16, seed=0, bias_std=0.02, ref_rounding=False)
         in_channels=cfg.in_channels, out_channels=cfg.out_channels, num_layers=cfg.num_layers,
         attention_head_dim=cfg.head_dim, num_attention_heads=cfg.num_heads,
         joint_attention_dim=cfg.joint_attention_dim, axes_dims_rope=cfg.axes_dims_rope,
-        ref_rounding=ref_rounding).to(gpu).to(dtype)
+        ref_rounding=ref_rounding, **model_kwargs).to(gpu).to(dtype)
     model.load_flat_state(w_lp)
     return cfg, w_lp, model
 
@@ -70,6 +70,43 @@ def test_tiny_model_per_block_parity(gpu):
     with torch.inference_mode():
         out2 = model(lat.to(gpu), txt.to(gpu), None, t.to(gpu), [IMG_SHAPE], [S_TXT]).sample
     assert torch.equal(out2, out)
+
+
+@pytest.mark.parametrize("fuse", [False, True])
+def test_editing_variant_per_token_conditioning(gpu, fuse):
+    """zero_cond_t: doubled timestep, per-token choice between the two conditioning rows in both norms
+    and both gates of the image stream, text stream and head on the real-timestep rows. Source image
+    8x16, two target images 4x16 each (256 tokens)."""
+    cfg, w, model = _build(gpu, zero_cond_t=True)
+    # N(0, 0.02) weights make the timestep almost irrelevant: strengthen the conditioning path so that a
+    # dropped or swapped index moves the output far beyond the bf16 tolerance
+    w = {k: (v * 8 if "img_mod.1.weight" in k or "timestep_embedder.linear_2.weight" in k else v) for k, v in w.items()}
+    model.load_flat_state(w)
+    if fuse:
+        model.fuse_modulation()
+    shapes = [(1, 8, 16), (1, 4, 16), (1, 4, 16)]
+    lat, txt, t = _inputs(2, seed=21)
+    w32 = {k: v.float() for k, v in w.items()}
+    want = oq.transformer_forward(w32, cfg, lat.float(), txt.float(), t.float(), shapes, zero_cond_t=True)
+    plain = oq.transformer_forward(w32, cfg, lat.float(), txt.float(), t.float(), shapes)
+    with torch.inference_mode():
+        index = model.modulate_index([shapes, shapes], gpu)
+        assert index.dtype == torch.int32 and index.cpu().tolist() == [[0] * 128 + [1] * 128] * 2
+        got = model(lat.to(gpu), txt.to(gpu), None, t.to(gpu), [shapes, shapes], [S_TXT]).sample
+    err = (got.float().cpu() - want).abs().max().item()
+    print(f"editing variant (fused modulation {fuse}): max-abs {err:.4f} cosine {_cosine(got, want):.6f}", flush=True)
+    assert err <= 2e-2 and _cosine(got, want) >= 0.9995
+    # the test would not notice a dropped index if the two models agreed anyway: they do not
+    assert (plain - want).abs().max().item() > 10 * err
+
+
+def test_teacache_refuses_the_editing_variant(gpu):
+    from vllm_omni_amd.cache.teacache.extractors import extract_qwen_context
+
+    cfg, w, model = _build(gpu, zero_cond_t=True)
+    lat, txt, t = _inputs(1)
+    with pytest.raises(NotImplementedError):
+        extract_qwen_context(model, lat.to(gpu), txt.to(gpu), None, t.to(gpu), [[IMG_SHAPE]], [S_TXT])
 
 
 def test_block_with_text_padding_mask(gpu):

@@ -366,7 +366,8 @@ class QwenImageTransformer2DModel(nn.Module):
     def __init__(self, patch_size: int = 2, in_channels: int = 64, out_channels: int | None = 16,
                  num_layers: int = 60, attention_head_dim: int = 128, num_attention_heads: int = 24,
                  joint_attention_dim: int = 3584, axes_dims_rope: tuple[int, int, int] = (16, 56, 56),
-                 mlp_ratio: int = 4, ref_rounding: bool = False, fuse_epilogues: bool = True):
+                 mlp_ratio: int = 4, ref_rounding: bool = False, fuse_epilogues: bool = True,
+                 zero_cond_t: bool = False):
         super().__init__()
         self.in_channels = in_channels
         self.out_channels = out_channels or in_channels
@@ -378,25 +379,40 @@ class QwenImageTransformer2DModel(nn.Module):
         self.txt_in = nn.Linear(joint_attention_dim, self.inner_dim)
         self.transformer_blocks = nn.ModuleList([
             QwenImageTransformerBlock(self.inner_dim, num_attention_heads, attention_head_dim,
-                                      mlp_ratio=mlp_ratio, ref_rounding=ref_rounding, fuse_epilogues=fuse_epilogues)
+                                      mlp_ratio=mlp_ratio, ref_rounding=ref_rounding, fuse_epilogues=fuse_epilogues,
+                                      zero_cond_t=zero_cond_t)
             for _ in range(num_layers)])
         self.norm_out = AdaLayerNormContinuous(self.inner_dim, self.inner_dim, eps=1e-6)
         self.proj_out = nn.Linear(self.inner_dim, patch_size * patch_size * self.out_channels, bias=True)
-        self.zero_cond_t = False
+        self.zero_cond_t = zero_cond_t
         self._res_bias = None
         self.parallel_config = None
         self.do_true_cfg = False
 
     # -- stages ---------------------------------------------------------------------------------
     def prepare(self, hidden_states, encoder_hidden_states, timestep, img_shapes, txt_seq_lens):
+        """Stem. With ``zero_cond_t`` (editing checkpoints) the timestep is doubled to [t, 0 * t], so temb
+        has 2B rows: real-timestep conditioning, then timestep-zero conditioning (qit.py:141-145)."""
         img = self.img_in(hidden_states)
         timestep = timestep.to(device=img.device, dtype=img.dtype)
+        if self.zero_cond_t:
+            timestep = torch.cat([timestep, timestep * 0], dim=0)
         txt = self.txt_in(self.txt_norm(encoder_hidden_states))
         temb = self.time_text_embed(timestep, img)
         if txt_seq_lens is None:
             txt_seq_lens = [encoder_hidden_states.shape[1]]
         vid_freqs, txt_freqs = self.pos_embed(img_shapes, txt_seq_lens, device=img.device)
         return img, txt, temb, RotaryTables(vid_freqs, txt_freqs)
+
+    def modulate_index(self, img_shapes, device) -> torch.Tensor | None:
+        """[B, S_img] int32 per-token conditioning choice of the editing variant: 0 (real timestep) for the
+        tokens of each sample's first image, 1 (timestep zero) for every later image; ``img_shapes`` is
+        per sample a list of (frame, height, width) (qit.py:146-154). None for the plain model."""
+        if not self.zero_cond_t:
+            return None
+        samples = [[s] if isinstance(s[0], int) else list(s) for s in img_shapes]  # bare (f, h, w) = one image
+        rows = [[0] * math.prod(s[0]) + [1] * sum(math.prod(x) for x in s[1:]) for s in samples]
+        return torch.tensor(rows, device=device, dtype=torch.int32)
 
     def fuse_modulation(self) -> None:
         """Stack every block's img_mod / txt_mod Linear into one [L, 2, 6C, C] weight so that the
@@ -431,36 +447,41 @@ class QwenImageTransformer2DModel(nn.Module):
     def all_gate_rows(self, mods: torch.Tensor | None):
         """float32 (gates, gates * biases) [B, L, 2, 2, C] of the four gated projections of every block,
         from the stacked modulation parameters: two small elementwise ops per step."""
-        if mods is None or mods.dtype == torch.float32:
-            return None
+        if mods is None or mods.dtype == torch.float32 or self.zero_cond_t:
+            return None  # per-token gates of the editing variant do not fit one row per batch entry
         B, L, C = mods.shape[0], mods.shape[1], self.inner_dim
         gates = mods.view(B, L, 2, 2, 3 * C)[..., 2 * C:].float()
         return gates, gates * self._gated_biases()
 
     def all_modulations(self, temb: torch.Tensor) -> torch.Tensor | None:
-        """[B, L, 2, 6C] modulation parameters of every block, or None when not fused."""
+        """[B, L, 2, 6C] modulation parameters of every block, or None when not fused. For the editing
+        variant temb has 2B rows and so has the result: the image stream reads all of them through the
+        per-token index, the text stream the first B (qit.py:758-767)."""
         w = getattr(self, "_mod_weight", None)
-        if w is None or self.zero_cond_t:
+        if w is None:
             return None
         L, C = w.shape[0], self.inner_dim
         out = F.linear(kernels.silu(temb), w.view(L * 2 * 6 * C, C), self._mod_bias.view(-1))
         return out.view(temb.shape[0], L, 2, 6 * C)
 
-    def run_blocks(self, img, txt, temb, rotary, encoder_hidden_states_mask=None, attention_kwargs=None):
+    def run_blocks(self, img, txt, temb, rotary, encoder_hidden_states_mask=None, attention_kwargs=None,
+                   modulate_index=None):
         mask = encoder_hidden_states_mask
         if mask is not None and bool(mask.all()):
             mask = None  # all-true masks are dropped (qit.py:1044-1048)
         mods = self.all_modulations(temb)
         rows = self.all_gate_rows(mods)
         for i, block in enumerate(self.transformer_blocks):
-            mp = (mods[:, i, 0], mods[:, i, 1]) if mods is not None else None
+            mp = (mods[:, i, 0], mods[:txt.shape[0], i, 1]) if mods is not None else None
             gr = (rows[0][:, i], rows[1][:, i]) if rows is not None else None
             txt, img = block(hidden_states=img, encoder_hidden_states=txt, encoder_hidden_states_mask=mask,
                              temb=temb, image_rotary_emb=rotary, joint_attention_kwargs=attention_kwargs,
-                             mod_params=mp, gate_rows=gr)
+                             modulate_index=modulate_index, mod_params=mp, gate_rows=gr)
         return img, txt
 
     def finish(self, img, temb, return_dict: bool = True):
+        if self.zero_cond_t:
+            temb = temb.chunk(2, dim=0)[0]  # the head is conditioned on the real timestep (qit.py:1062-1063)
         out = self.proj_out(self.norm_out(img, temb))
         return Transformer2DModelOutput(sample=out) if return_dict else (out,)
 
@@ -469,7 +490,9 @@ class QwenImageTransformer2DModel(nn.Module):
                 img_shapes=None, txt_seq_lens=None, guidance: torch.Tensor = None,
                 attention_kwargs: dict[str, Any] | None = None, additional_t_cond=None, return_dict: bool = True):
         img, txt, temb, rotary = self.prepare(hidden_states, encoder_hidden_states, timestep, img_shapes, txt_seq_lens)
-        img, txt = self.run_blocks(img, txt, temb, rotary, encoder_hidden_states_mask, attention_kwargs)
+        index = self.modulate_index(img_shapes, img.device)
+        img, txt = self.run_blocks(img, txt, temb, rotary, encoder_hidden_states_mask, attention_kwargs,
+                                   modulate_index=index)
         return self.finish(img, temb, return_dict=return_dict)
 
     # -- weights --------------------------------------------------------------------------------
