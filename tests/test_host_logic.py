@@ -262,3 +262,106 @@ def test_load_weights_stacks_qkv_and_renames_like_the_reference():
         m.load_weights([("transformer_blocks.0.attn.to_q.weight", torch.zeros(3, cfg.dim))])
     with pytest.raises(KeyError):
         m.load_weights([("transformer_blocks.0.nothing.weight", torch.zeros(1))])
+
+
+# ------------------------------------------------------------------------------ vLLM-Omni plugin
+def _stub_vllm_omni(monkeypatch):
+    """A stand-in for the four reference modules the plugin touches, with the interfaces they have there:
+    a closed enum + override registry (attention/backends/registry.py:38-152), ``register_extractor``
+    (cache/teacache/extractors.py:585-615) and the two CustomOp classes."""
+    import enum
+    import sys
+    import types
+
+    import torch.nn as nn
+
+    class DiffusionAttentionBackendEnum(enum.Enum):
+        FLASH_ATTN = "vllm_omni.diffusion.attention.backends.flash_attn.FlashAttentionBackend"
+        TORCH_SDPA = "vllm_omni.diffusion.attention.backends.sdpa.SDPABackend"
+        SAGE_ATTN = "vllm_omni.diffusion.attention.backends.sage_attn.SageAttentionBackend"
+
+    overrides, extractors = {}, {}
+
+    def register_diffusion_backend(backend, class_path=None):
+        assert isinstance(backend, DiffusionAttentionBackendEnum) and class_path
+        overrides[backend] = class_path
+        return lambda x: x
+
+    class AdaLayerNorm(nn.Module):
+        def forward_hip(self, x, mod_params, index=None):
+            raise AssertionError("reference path")
+
+    class RotaryEmbedding(nn.Module):
+        def forward_hip(self, x, cos, sin):
+            raise AssertionError("reference path")
+
+    tree = {
+        "vllm_omni": {}, "vllm_omni.diffusion": {}, "vllm_omni.diffusion.attention": {},
+        "vllm_omni.diffusion.attention.backends": {},
+        "vllm_omni.diffusion.attention.backends.registry": {
+            "DiffusionAttentionBackendEnum": DiffusionAttentionBackendEnum,
+            "register_diffusion_backend": register_diffusion_backend},
+        "vllm_omni.diffusion.cache": {}, "vllm_omni.diffusion.cache.teacache": {},
+        "vllm_omni.diffusion.cache.teacache.extractors": {
+            "register_extractor": lambda name, fn: extractors.__setitem__(name, fn)},
+        "vllm_omni.diffusion.layers": {},
+        "vllm_omni.diffusion.layers.adalayernorm": {"AdaLayerNorm": AdaLayerNorm},
+        "vllm_omni.diffusion.layers.rope": {"RotaryEmbedding": RotaryEmbedding},
+    }
+    for name, attrs in tree.items():
+        mod = types.ModuleType(name)
+        mod.__path__ = []
+        for k, v in attrs.items():
+            setattr(mod, k, v)
+        monkeypatch.setitem(sys.modules, name, mod)
+    return DiffusionAttentionBackendEnum, overrides, extractors, AdaLayerNorm, RotaryEmbedding
+
+
+def test_plugin_needs_vllm_omni():
+    import sys
+
+    from vllm_omni_amd import plugin
+
+    assert "vllm_omni" not in sys.modules
+    with pytest.raises(ImportError, match="vllm-omni"):
+        plugin.register()
+
+
+def test_plugin_registers_backend_layers_and_extractor(monkeypatch):
+    import importlib
+
+    from vllm_omni_amd import plugin, torch_ops
+    from vllm_omni_amd.cache.teacache.extractors import extract_flux_context
+
+    E, overrides, extractors, AdaLN, Rope = _stub_vllm_omni(monkeypatch)
+    plugin.register()
+    plugin.register()  # loaded once per process at least; twice must be harmless
+    assert overrides == {E.FLASH_ATTN: plugin.BACKEND_PATH, E.TORCH_SDPA: plugin.BACKEND_PATH}
+    mod, cls = plugin.BACKEND_PATH.rsplit(".", 1)
+    backend = getattr(importlib.import_module(mod), cls)   # how the reference's selector resolves it
+    assert backend.get_name() == "HIP_FLASH_ATTN" and backend.supports_attention_mask()
+    assert backend.supports_head_size(128) and not backend.supports_head_size(96)
+    impl = backend.get_impl_cls()(num_heads=4, head_size=64, softmax_scale=0.125, causal=False, num_kv_heads=4)
+    assert type(impl).forward_hip is torch_ops.attention_forward_hip
+    assert AdaLN.forward_hip is torch_ops.adaln_forward_hip and Rope.forward_hip is torch_ops.rope_forward_hip
+    assert extractors == {"FluxTransformer2DModel": extract_flux_context}
+    with pytest.raises(TypeError, match="FluxTransformer2DModel"):
+        extract_flux_context(type("Other", (), {"transformer_blocks": [0]})(), None)
+
+
+def test_custom_ops_trace_with_fake_tensors():
+    """Shape propagation of the three ops without any device: what torch.compile's tracer sees."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from vllm_omni_amd import torch_ops  # noqa: F401  (defines torch.ops.omni_dit)
+
+    with FakeTensorMode():
+        q = torch.empty(2, 70, 4, 64, dtype=torch.bfloat16, device="cuda")
+        k = torch.empty(2, 90, 4, 64, dtype=torch.bfloat16, device="cuda")
+        o = torch.ops.omni_dit.attention(q, k, k, 0.125, torch.ones(2, 90, dtype=torch.bool, device="cuda"))
+        assert o.shape == q.shape and o.dtype == q.dtype and o.device.type == "cuda"
+        x = torch.empty(2, 70, 256, dtype=torch.bfloat16, device="cuda")
+        m = torch.empty(2, 256, dtype=torch.bfloat16, device="cuda")
+        assert torch.ops.omni_dit.adaln_modulate(x, m, m, 1e-6).shape == x.shape
+        t = torch.empty(70, 32, device="cuda")
+        assert torch.ops.omni_dit.rotary(q, t, t, False).shape == q.shape

@@ -100,6 +100,9 @@ def extract_flux_context(module: nn.Module, hidden_states: torch.Tensor,
     coefficients it already ships (config.py:11-17). ``module`` is this package's FluxTransformer2DModel."""
     if not hasattr(module, "transformer_blocks") or len(module.transformer_blocks) == 0:
         raise ValueError("Module must have transformer_blocks")
+    if not hasattr(module, "prepare"):
+        raise TypeError("extract_flux_context drives this package's FluxTransformer2DModel (prepare / run_blocks / "
+                        f"finish stages); got {type(module).__module__}.{type(module).__name__}")
     img, txt, temb, rotary = module.prepare(hidden_states, encoder_hidden_states, pooled_projections, timestep,
                                             img_ids, txt_ids, guidance)
     modulated = module.transformer_blocks[0].norm1(img, emb=temb)[0]
