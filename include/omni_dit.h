@@ -143,17 +143,23 @@ int odit_qknorm_rope(const void* q_in, const void* k_in, const void* v_in, void*
  *  wan2_2_transformer.py:659, 668-670).
  *
  * x, out: [B,S,C], x_strides/out_strides = (batch, seq) strides; C contiguous.
- * shift, scale: element (b, c) at ptr[b*mod_stride_b + c]; NULL = 0. Type per mod_dtype (`dtype` or
- *   ODIT_F32). `gate` is not touched here: the caller returns it as a view.
+ * shift, scale: element (b, s, c) at ptr[b*mod_stride_b + s*mod_stride_s + c]; NULL = 0. Type per
+ *   mod_dtype (`dtype` or ODIT_F32). mod_stride_s = 0 is one row per batch entry; non-zero is one row
+ *   per token (Wan per-token timesteps, temb [B,S,6,C], wan2_2_transformer.py:641-652).
+ *   `gate` is not touched here: the caller returns it as a view.
+ * shift_bias, scale_bias: NULL or float32 [C] added to the shift / scale row in fp32 (Wan's
+ *   scale_shift_table + temb.float(), wan2_2_transformer.py:643-645, 654-656, without forming the sum
+ *   in memory).
  * index: NULL, or int32 [B,S] (row stride S): token (b,s) uses modulation row b when index == 0 and
- *   row b + B otherwise (adalayernorm.py:31-54).
+ *   row b + B otherwise (adalayernorm.py:31-54); needs mod_stride_s == 0.
  * ln_weight, ln_bias: NULL or float32 [C] (elementwise-affine LayerNorm, applied before modulation).
  */
 int odit_adaln_modulate(const void* x, void* out, const void* shift, const void* scale,
-                        const int32_t* index, const float* ln_weight, const float* ln_bias, int B,
-                        int S, int C, const int64_t x_strides[2], const int64_t out_strides[2],
-                        int64_t mod_stride_b, float eps, int mod_dtype, int dtype, unsigned flags,
-                        void* stream);
+                        const int32_t* index, const float* ln_weight, const float* ln_bias,
+                        const float* shift_bias, const float* scale_bias, int B, int S, int C,
+                        const int64_t x_strides[2], const int64_t out_strides[2],
+                        int64_t mod_stride_b, int64_t mod_stride_s, float eps, int mod_dtype,
+                        int dtype, unsigned flags, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * K4  gated residual:  out = h + gate * y     (gate broadcast over the sequence, or per token)
@@ -164,9 +170,12 @@ int odit_adaln_modulate(const void* x, void* out, const void* shift, const void*
  *
  * h, y, out: [B,S,C] with (batch, seq) strides; out may alias h.
  * gate element (b,s,c) at gate[b*gate_strides[0] + s*gate_strides[1] + c]; type per gate_dtype.
+ * gate_bias: NULL or float32 [C] added to the gate in fp32 (Wan's scale_shift_table row + per-token
+ *   temb row, wan2_2_transformer.py:643-652); with gate == NULL the table alone is the gate.
  */
-int odit_gated_residual(const void* h, const void* y, const void* gate, void* out, int B, int S,
-                        int C, const int64_t h_strides[2], const int64_t y_strides[2],
+int odit_gated_residual(const void* h, const void* y, const void* gate, const float* gate_bias,
+                        void* out, int B, int S, int C, const int64_t h_strides[2],
+                        const int64_t y_strides[2],
                         const int64_t out_strides[2], const int64_t gate_strides[2], int gate_dtype,
                         int dtype, unsigned flags, void* stream);
 

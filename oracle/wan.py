@@ -1,14 +1,18 @@
-"""Oracle restatement of the Wan video DiT forward, text-to-video form (test infrastructure only).
+"""Oracle restatement of the Wan video DiT forward (test infrastructure only).
 
 Functional: weights are a flat ``dict[str, Tensor]`` keyed with the reference's parameter names.
 Reference file: ``vllm_omni/diffusion/models/wan2_2/wan2_2_transformer.py`` (``wan.py`` below).
-Covered: the T2V path (``temb`` [B, 6, C]); the per-token-timestep TI2V form (``temb.ndim == 4``,
-wan.py:641-652) and the I2V image branch of the cross-attention (wan.py:541-575) are not restated.
+Covered: the T2V path (``temb`` [B, 6, C]), the per-token-timestep TI2V form (``timestep`` [B, S],
+``temb`` [B, S, 6, C], wan.py:641-652, 864-876) and the I2V image branch (image embedder wan.py:224-248,
+second cross-attention over the image context wan.py:541-575).
 
 Third-party arithmetic on this path (diffusers>=0.36.0, absent from the reference tree — **parity
 unpinned** at that boundary, upstream conventions adopted): ``FP32LayerNorm`` (layer_norm evaluated
-in fp32, cast back to the input dtype), ``Timesteps`` / ``TimestepEmbedding``,
-``PixArtAlphaTextProjection(act_fn="gelu_tanh")`` (Linear, GELU-tanh, Linear).
+in fp32, cast back to the input dtype; an ``nn.LayerNorm`` subclass, so eps 1e-5 and an affine pair
+where the reference passes no arguments), ``Timesteps`` / ``TimestepEmbedding``,
+``PixArtAlphaTextProjection(act_fn="gelu_tanh")`` (Linear, GELU-tanh, Linear),
+``FeedForward(mult=1, activation_fn="gelu")`` of the image embedder (Linear, exact GELU, Linear; parameter
+names ``net.0.proj`` / ``net.2``).
 """
 
 from __future__ import annotations
@@ -39,6 +43,10 @@ class WanConfig:
     eps: float = 1e-6
     rope_max_seq_len: int = 1024
     theta: float = 10000.0
+    image_dim: int | None = None            # I2V: width of the image-encoder features
+    added_kv_proj_dim: int | None = None    # I2V: width of the embedded image context (= dim in the checkpoints)
+    pos_embed_seq_len: int | None = None    # first+last-frame variant: learned positions over 2 x 257 tokens
+    text_context_len: int = 512             # the reference hardcodes 512 text tokens (wan.py:540-543)
 
     @property
     def dim(self) -> int:
@@ -69,12 +77,27 @@ def block_param_shapes(cfg: WanConfig) -> dict[str, tuple[int, ...]]:
     }
     if cfg.cross_attn_norm:
         out.update({"norm2.weight": (C,), "norm2.bias": (C,)})
+    if cfg.added_kv_proj_dim is not None:
+        A = cfg.added_kv_proj_dim
+        out.update({"attn2.add_k_proj.weight": (C, A), "attn2.add_k_proj.bias": (C,),
+                    "attn2.add_v_proj.weight": (C, A), "attn2.add_v_proj.bias": (C,),
+                    "attn2.norm_added_k.weight": (C,)})
     return out
 
 
 def stem_param_shapes(cfg: WanConfig) -> dict[str, tuple[int, ...]]:
     C = cfg.dim
+    img = {}
+    if cfg.image_dim is not None:
+        I, p = cfg.image_dim, "condition_embedder.image_embedder."
+        img = {p + "norm1.weight": (I,), p + "norm1.bias": (I,),
+               p + "ff.net.0.proj.weight": (I, I), p + "ff.net.0.proj.bias": (I,),
+               p + "ff.net.2.weight": (C, I), p + "ff.net.2.bias": (C,),
+               p + "norm2.weight": (C,), p + "norm2.bias": (C,)}
+        if cfg.pos_embed_seq_len is not None:
+            img[p + "pos_embed"] = (1, cfg.pos_embed_seq_len, I)
     return {
+        **img,
         "patch_embedding.weight": (C, cfg.in_channels, *cfg.patch_size), "patch_embedding.bias": (C,),
         "condition_embedder.time_embedder.linear_1.weight": (C, cfg.freq_dim),
         "condition_embedder.time_embedder.linear_1.bias": (C,),
@@ -101,7 +124,7 @@ def init_params(cfg: WanConfig, seed: int = 0, dtype: torch.dtype = torch.float3
     def make(name: str, shape: tuple[int, ...]):
         if name.endswith("scale_shift_table"):
             t = torch.randn(shape, generator=g) / shape[-1] ** 0.5
-        elif name.endswith(("norm_q.weight", "norm_k.weight", "norm2.weight")):
+        elif name.endswith(("norm_q.weight", "norm_k.weight", "norm_added_k.weight", "norm1.weight", "norm2.weight")):
             t = torch.ones(shape) + (torch.randn(shape, generator=g) * norm_jitter if norm_jitter > 0 else 0)
         elif name.endswith(".bias"):
             t = torch.randn(shape, generator=g) * bias_std if bias_std > 0 else torch.zeros(shape)
@@ -167,21 +190,36 @@ def self_attention(w, pre, cfg: WanConfig, x, cos, sin):
 
 
 def cross_attention(w, pre, cfg: WanConfig, x, ctx):
-    """WanCrossAttention.forward without the image branch, wan.py:532-586: q from the video tokens,
-    k/v from the text tokens, whole-row RMSNorm on q and k, no rotary."""
+    """WanCrossAttention.forward, wan.py:532-586: q from the video tokens, k/v from the text tokens,
+    whole-row RMSNorm on q and k, no rotary. With the image branch (``added_kv_proj_dim``) the context is
+    [image tokens; 512 text tokens]: a second, separate softmax attention of the same q over the image
+    tokens (own k/v projections, own k norm) is added to the text attention before the output projection."""
     H, D = cfg.num_heads, cfg.head_dim
+    ctx_img = None
+    if cfg.added_kv_proj_dim is not None:
+        n_img = ctx.shape[1] - cfg.text_context_len
+        ctx_img, ctx = ctx[:, :n_img], ctx[:, n_img:]
     q = ops.rms_norm_row_fp32(_lin(w, pre + "to_q", x), w[pre + "norm_q.weight"], cfg.eps).unflatten(2, (H, D))
     k = ops.rms_norm_row_fp32(_lin(w, pre + "to_k", ctx), w[pre + "norm_k.weight"], cfg.eps).unflatten(2, (H, D))
     v = _lin(w, pre + "to_v", ctx).unflatten(2, (H, D))
     o = ops.sdpa(q, k, v, 1.0 / (D ** 0.5)).flatten(2, 3).type_as(q)
+    if ctx_img is not None:
+        ki = ops.rms_norm_row_fp32(_lin(w, pre + "add_k_proj", ctx_img), w[pre + "norm_added_k.weight"], cfg.eps)
+        vi = _lin(w, pre + "add_v_proj", ctx_img)
+        oi = ops.sdpa(q, ki.unflatten(2, (H, D)), vi.unflatten(2, (H, D)), 1.0 / (D ** 0.5))
+        o = o + oi.flatten(2, 3).type_as(q)
     return _lin(w, pre + "to_out", o)
 
 
 def block_forward(w, i: int, cfg: WanConfig, x, ctx, temb6, cos, sin):
-    """WanTransformerBlock.forward (T2V form), wan.py:634-675. temb6 [B, 6, C]; modulation and the
-    gated residuals are evaluated in fp32 and cast back."""
+    """WanTransformerBlock.forward, wan.py:634-675. temb6 [B, 6, C], or [B, S, 6, C] with per-token
+    timesteps; modulation and the gated residuals are evaluated in fp32 and cast back."""
     pre = f"blocks.{i}."
-    sh, sc, g, csh, csc, cg = (w[pre + "scale_shift_table"] + temb6.float()).chunk(6, dim=1)
+    if temb6.ndim == 4:
+        mods = (w[pre + "scale_shift_table"].unsqueeze(0) + temb6.float()).chunk(6, dim=2)
+        sh, sc, g, csh, csc, cg = (m.squeeze(2) for m in mods)
+    else:
+        sh, sc, g, csh, csc, cg = (w[pre + "scale_shift_table"] + temb6.float()).chunk(6, dim=1)
     n = (fp32_layer_norm(x.float(), None, None, cfg.eps) * (1 + sc) + sh).type_as(x)
     a = self_attention(w, pre + "attn1.", cfg, n, cos, sin)
     x = (x.float() + a * g).type_as(x)
@@ -195,10 +233,27 @@ def block_forward(w, i: int, cfg: WanConfig, x, ctx, temb6, cos, sin):
     return (x.float() + ff.float() * cg).type_as(x)
 
 
-def condition_embedder(w, cfg: WanConfig, timestep, text):
-    """WanTimeTextImageEmbedding.forward, wan.py:275-296 -> (temb [B,C], timestep_proj [B,6C], text)."""
+def image_embedder(w, cfg: WanConfig, image_feats):
+    """WanImageEmbedding.forward, wan.py:239-248: (optional learned positions over the first+last frame
+    pair, rows of two consecutive batch entries joined) -> FP32LayerNorm -> Linear, GELU, Linear ->
+    FP32LayerNorm. The two norms are built without arguments: eps 1e-5, affine."""
+    pre = "condition_embedder.image_embedder."
+    x = image_feats
+    if pre + "pos_embed" in w:
+        _, n, e = x.shape
+        x = x.view(-1, 2 * n, e) + w[pre + "pos_embed"]
+    x = fp32_layer_norm(x, w[pre + "norm1.weight"], w[pre + "norm1.bias"], 1e-5)
+    x = _lin(w, pre + "ff.net.2", F.gelu(_lin(w, pre + "ff.net.0.proj", x)))
+    return fp32_layer_norm(x, w[pre + "norm2.weight"], w[pre + "norm2.bias"], 1e-5)
+
+
+def condition_embedder(w, cfg: WanConfig, timestep, text, timestep_seq_len: int | None = None):
+    """WanTimeTextImageEmbedding.forward, wan.py:275-296 -> (temb [B,C], timestep_proj [B,6C], text);
+    with ``timestep_seq_len`` the flattened [B*S] timesteps give temb [B,S,C] and timestep_proj [B,S,6C]."""
     pre = "condition_embedder."
     t = ops.timestep_embedding(timestep, dim=cfg.freq_dim, scale=1.0)
+    if timestep_seq_len is not None:
+        t = t.unflatten(0, (-1, timestep_seq_len))
     t = t.to(w[pre + "time_embedder.linear_1.weight"].dtype)
     temb = _lin(w, pre + "time_embedder.linear_2", F.silu(_lin(w, pre + "time_embedder.linear_1", t))).type_as(text)
     tproj = _lin(w, pre + "time_proj", F.silu(temb))
@@ -206,33 +261,49 @@ def condition_embedder(w, cfg: WanConfig, timestep, text):
     return temb, tproj, ctx
 
 
-def stem(w, cfg: WanConfig, video, timestep, text):
+def stem(w, cfg: WanConfig, video, timestep, text, image_feats=None):
     """Patch embedding (Conv3d with kernel = stride = patch), flatten to tokens, condition embeddings.
-    wan.py:852-881. video [B, C_in, F, H, W]."""
+    wan.py:852-881. video [B, C_in, F, H, W]; timestep [B] or, per token, [B, S]; with ``image_feats``
+    the embedded image tokens are put in front of the text tokens (wan.py:878-879)."""
     x = F.conv3d(video, w["patch_embedding.weight"], w["patch_embedding.bias"], stride=cfg.patch_size)
     x = x.flatten(2).transpose(1, 2)
-    temb, tproj, ctx = condition_embedder(w, cfg, timestep, text)
-    return x, temb, tproj.unflatten(1, (6, -1)), ctx
+    ts_len = None
+    if timestep.ndim == 2:
+        ts_len, timestep = timestep.shape[1], timestep.flatten()
+    temb, tproj, ctx = condition_embedder(w, cfg, timestep, text, ts_len)
+    if image_feats is not None:
+        ctx = torch.cat([image_embedder(w, cfg, image_feats), ctx], dim=1)
+    return x, temb, tproj.unflatten(tproj.ndim - 1, (6, -1)), ctx
 
 
 def head(w, cfg: WanConfig, x, temb, grid, batch):
     """Output modulation (shift, scale = table + temb), fp32 LayerNorm, projection, unpatchify.
-    wan.py:887-905."""
-    shift, scale = (w["output_scale_shift_prepare.scale_shift_table"] + temb.unsqueeze(1)).chunk(2, dim=1)
+    wan.py:887-905; per-token temb [B,S,C] gives per-token shift and scale (wan.py:324-331)."""
+    table = w["output_scale_shift_prepare.scale_shift_table"]
+    if temb.ndim == 3:
+        shift, scale = ((table.unsqueeze(0) + temb.unsqueeze(2)).chunk(2, dim=2))
+        shift, scale = shift.squeeze(2), scale.squeeze(2)
+        x = (fp32_layer_norm(x.float(), None, None, cfg.eps) * (1 + scale) + shift).type_as(x)
+        return _unpatchify(cfg, _lin(w, "proj_out", x), grid, batch)
+    shift, scale = (table + temb.unsqueeze(1)).chunk(2, dim=1)
     x = (fp32_layer_norm(x.float(), None, None, cfg.eps) * (1 + scale) + shift).type_as(x)
-    x = _lin(w, "proj_out", x)
+    return _unpatchify(cfg, _lin(w, "proj_out", x), grid, batch)
+
+
+def _unpatchify(cfg: WanConfig, x, grid, batch):
     p_t, p_h, p_w = cfg.patch_size
     x = x.reshape(batch, *grid, p_t, p_h, p_w, -1).permute(0, 7, 1, 4, 2, 5, 3, 6)
     return x.flatten(6, 7).flatten(4, 5).flatten(2, 3)
 
 
-def transformer_forward(w, cfg: WanConfig, video, timestep, text, collect_blocks: bool = False):
+def transformer_forward(w, cfg: WanConfig, video, timestep, text, collect_blocks: bool = False,
+                        image_feats=None):
     """WanTransformer3DModel.forward, wan.py:838-910."""
     B, _, nf, hh, ww = video.shape
     p_t, p_h, p_w = cfg.patch_size
     grid = (nf // p_t, hh // p_h, ww // p_w)
     cos, sin = wan_rope_tables(cfg, *grid)
-    x, temb, temb6, ctx = stem(w, cfg, video, timestep, text)
+    x, temb, temb6, ctx = stem(w, cfg, video, timestep, text, image_feats)
     per_block = []
     for i in range(cfg.num_layers):
         x = block_forward(w, i, cfg, x, ctx, temb6, cos, sin)

@@ -53,9 +53,13 @@ def test_argument_errors_are_caught_before_launch():
     rc = lib.odit_attn_fwd(p16, p16, p16, p16, None, None, 1, 4, 4, 3, 2, 64, s3, s3, s3, s3, 0.1, 0, None)
     assert rc == -1
     # null pointers
-    rc = lib.odit_adaln_modulate(None, p16, None, None, None, None, None, 1, 1, 8, _strides(8, 8), _strides(8, 8),
-                                 8, 1e-6, 0, 0, 0, None)
+    rc = lib.odit_adaln_modulate(None, p16, None, None, None, None, None, None, None, 1, 1, 8, _strides(8, 8),
+                                 _strides(8, 8), 8, 0, 1e-6, 0, 0, 0, None)
     assert rc == -1
+    # a row index and per-token modulation rows exclude each other
+    rc = lib.odit_adaln_modulate(p16, p16, p16, p16, p16, None, None, None, None, 1, 1, 8, _strides(8, 8),
+                                 _strides(8, 8), 8, 8, 1e-6, 0, 0, 0, None)
+    assert rc == -1 and b"exclude" in lib.odit_last_error()
     # joint rows out of range
     rc = lib.odit_qknorm_rope(p16, None, None, p16, None, None, None, None, None, None, 1, 4, 1, 64, 0,
                               _strides(256, 64), 2, 4, 1e-6, 1, 0, 0, 0, None)
@@ -66,7 +70,7 @@ def test_argument_errors_are_caught_before_launch():
     assert rc == -4
     # empty problems succeed without touching the device
     assert lib.odit_gelu_tanh(None, None, 0, 0, None) == 0
-    assert lib.odit_gated_residual(p16, p16, None, p16, 0, 4, 8, _strides(32, 8), _strides(32, 8), _strides(32, 8),
+    assert lib.odit_gated_residual(p16, p16, None, None, p16, 0, 4, 8, _strides(32, 8), _strides(32, 8), _strides(32, 8),
                                    None, 0, 0, 0, None) == 0
 
 

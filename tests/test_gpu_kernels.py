@@ -89,6 +89,35 @@ def test_adaln_index_fp32_params_affine_and_strides(gpu):
     _close(got3, torch.nn.functional.layer_norm(wide[:, :, C:].float(), (C,), eps=1e-6), atol=2e-2, what="plain LN")
 
 
+@pytest.mark.parametrize("C", [256, 3072, 5120, 100])
+def test_adaln_and_gate_with_per_token_rows_and_tables(gpu, C):
+    """Per-token modulation rows (views of a [B,S,6,C] tensor, token stride 6C) plus float32 [C] tables
+    added in-kernel, against the expression the reference evaluates: (table + temb.float()) chunks, fp32
+    LayerNorm, modulate; (h.float() + y * gate). C = 100 takes the kernels' unvectorised paths."""
+    from vllm_omni_amd import kernels
+
+    B, S = 2, 11
+    x, y = _rand(B, S, C, seed=1), _rand(B, S, C, seed=2)
+    temb = _rand(B, S, 6, C, seed=3, scale=0.3)
+    table = _rand(6, C, seed=4, dtype=torch.float32, scale=0.3)
+    mods = (table[None, None] + temb.float()).unbind(2)
+    ln = torch.nn.functional.layer_norm(x.float(), (C,), eps=1e-6)
+    tg, tabg = temb.to(gpu), table.to(gpu)
+    got = kernels.adaln_modulate(x.to(gpu), tg[:, :, 0], tg[:, :, 1], shift_bias=tabg[0], scale_bias=tabg[1])
+    _close(got, ln * (1 + mods[1]) + mods[0], atol=2e-2, rtol=1e-2, what="per-token adaln + tables")
+    # rows only / tables only (the table alone is then the modulation of every token)
+    got = kernels.adaln_modulate(x.to(gpu), tg[:, :, 3], tg[:, :, 4])
+    _close(got, ln * (1 + temb[:, :, 4].float()) + temb[:, :, 3].float(), atol=2e-2, rtol=1e-2, what="per-token adaln")
+    got = kernels.adaln_modulate(x.to(gpu), None, None, shift_bias=tabg[0], scale_bias=tabg[1])
+    _close(got, ln * (1 + table[1]) + table[0], atol=2e-2, rtol=1e-2, what="tables only")
+    got = kernels.gated_residual(x.to(gpu), y.to(gpu), tg[:, :, 2], gate_bias=tabg[2])
+    _close(got, x.float() + y.float() * mods[2], atol=1e-6, rtol=2 ** -8, what="per-token gate + table")
+    got = kernels.gated_residual(x.to(gpu), y.to(gpu), None, gate_bias=tabg[5])
+    _close(got, x.float() + y.float() * table[5], atol=1e-6, rtol=2 ** -8, what="table as the gate")
+    with pytest.raises(ValueError, match="exclude"):
+        kernels.adaln_modulate(x.to(gpu), tg[:, :, 0], tg[:, :, 1], index=torch.zeros(B, S, dtype=torch.int32, device=gpu))
+
+
 # ========================================================================================= K4
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_gated_residual(gpu, dtype):

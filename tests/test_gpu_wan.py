@@ -26,7 +26,8 @@ def _model(gpu, cfg, w_lp, dtype=torch.bfloat16):
         patch_size=cfg.patch_size, num_attention_heads=cfg.num_heads, attention_head_dim=cfg.head_dim,
         in_channels=cfg.in_channels, out_channels=cfg.out_channels, text_dim=cfg.text_dim, freq_dim=cfg.freq_dim,
         ffn_dim=cfg.ffn_dim, num_layers=cfg.num_layers, cross_attn_norm=cfg.cross_attn_norm, eps=cfg.eps,
-        rope_max_seq_len=cfg.rope_max_seq_len).to(gpu).to(dtype)
+        rope_max_seq_len=cfg.rope_max_seq_len, image_dim=cfg.image_dim, added_kv_proj_dim=cfg.added_kv_proj_dim,
+        pos_embed_seq_len=cfg.pos_embed_seq_len, text_context_len=cfg.text_context_len).to(gpu).to(dtype)
     model.load_flat_state(w_lp)
     return model
 
@@ -60,13 +61,77 @@ def test_tiny_wan_per_block_parity(gpu, fhw, n_txt, B):
     assert torch.equal(out2, out)
 
 
-def test_unbuilt_variants_raise(gpu):
-    from vllm_omni_amd.blocks.wan import WanTransformer3DModel, WanTransformerBlock
+def test_per_token_timesteps(gpu):
+    """timestep [B,S] (the TI2V form): two timestep values spread over the tokens, different per sample.
+    The kernels read the per-token rows of timestep_proj and add the float32 table rows in registers;
+    compared per block with the oracle, which forms the sums like the reference."""
+    cfg = ow.tiny_config()
+    w32 = ow.init_params(cfg, seed=2, bias_std=0.02, norm_jitter=0.1)
+    # N(0, 0.02) weights make the timestep nearly irrelevant: strengthen time_proj so that a wrong row shows
+    w32["condition_embedder.time_proj.weight"] = w32["condition_embedder.time_proj.weight"] * 20
+    w = {k: v.bfloat16() for k, v in w32.items()}
+    model = _model(gpu, cfg, w)
+    fhw, n_txt, B = (3, 10, 14), 13, 2
+    S = 3 * 5 * 7
+    g = torch.Generator().manual_seed(3)
+    video = torch.randn(B, cfg.in_channels, *fhw, generator=g).bfloat16()
+    text = torch.randn(B, n_txt, cfg.text_dim, generator=g).bfloat16()
+    pick = torch.rand(B, S, generator=g) < 0.4
+    ts = torch.where(pick, torch.tensor(0.0), torch.tensor([[731.0], [204.0]]).expand(B, S)).contiguous()
+    wf = {k: v.float() for k, v in w.items()}
+    want, per_block = ow.transformer_forward(wf, cfg, video.float(), ts, text.float(), collect_blocks=True)
+    scalar = ow.transformer_forward(wf, cfg, video.float(), torch.tensor([731.0, 204.0]), text.float())
+    with torch.inference_mode():
+        x, ctx, temb, tproj, rot = model.prepare(video.to(gpu), ts.to(gpu), text.to(gpu))
+        assert tproj.shape == (B, S, 6, cfg.dim) and temb.shape == (B, S, cfg.dim)
+        for i, block in enumerate(model.blocks):
+            x = block(x, ctx, tproj, rot)
+            err = (x.float().cpu() - per_block[i]).abs().max().item()
+            print(f"wan per-token block {i}: max-abs {err:.4f} cosine {_cosine(x, per_block[i]):.6f}", flush=True)
+            assert err <= 2e-2 and _cosine(x, per_block[i]) >= 0.9995
+        out = model(video.to(gpu), ts.to(gpu), text.to(gpu)).sample
+    err = (out.float().cpu() - want).abs().max().item()
+    assert err <= 2e-2 and _cosine(out, want) >= 0.9995
+    assert (scalar - want).abs().max().item() > 10 * err   # the per-token values do matter in this set-up
 
-    with pytest.raises(NotImplementedError):
-        WanTransformerBlock(256, 640, 4, added_kv_proj_dim=128)
-    with pytest.raises(NotImplementedError):
-        WanTransformer3DModel(num_attention_heads=4, attention_head_dim=64, ffn_dim=640, num_layers=1, image_dim=64)
+
+@pytest.mark.parametrize("pos", [False, True])
+def test_image_conditioned_cross_attention(gpu, pos):
+    """I2V: image-encoder tokens through the image embedder, put in front of the text tokens; every
+    block's cross-attention adds a second softmax over them. ``pos``: the first+last-frame variant with
+    learned positions over the joined token rows of two images per sample."""
+    import dataclasses
+
+    n_img, n_txt, B = 9, 13, 2
+    cfg = dataclasses.replace(ow.tiny_config(), image_dim=48, added_kv_proj_dim=256, text_context_len=n_txt,
+                              pos_embed_seq_len=2 * n_img if pos else None)
+    w32 = ow.init_params(cfg, seed=4, bias_std=0.02, norm_jitter=0.1)
+    w = {k: v.bfloat16() for k, v in w32.items()}
+    model = _model(gpu, cfg, w)
+    g = torch.Generator().manual_seed(5)
+    video = torch.randn(B, cfg.in_channels, 2, 8, 10, generator=g).bfloat16()
+    text = torch.randn(B, n_txt, cfg.text_dim, generator=g).bfloat16()
+    feats = torch.randn(2 * B if pos else B, n_img, cfg.image_dim, generator=g).bfloat16()
+    t = torch.tensor([731.0, 204.0])
+    wf = {k: v.float() for k, v in w.items()}
+    want, per_block = ow.transformer_forward(wf, cfg, video.float(), t, text.float(), collect_blocks=True,
+                                             image_feats=feats.float())
+    no_image = ow.transformer_forward(wf, dataclasses.replace(cfg, image_dim=None, added_kv_proj_dim=None),
+                                      video.float(), t, text.float())
+    with torch.inference_mode():
+        x, ctx, temb, tproj, rot = model.prepare(video.to(gpu), t.to(gpu), text.to(gpu), feats.to(gpu))
+        assert ctx.shape == (B, (2 * n_img if pos else n_img) + n_txt, cfg.dim)
+        for i, block in enumerate(model.blocks):
+            x = block(x, ctx, tproj, rot)
+            err = (x.float().cpu() - per_block[i]).abs().max().item()
+            print(f"wan i2v block {i}: max-abs {err:.4f} cosine {_cosine(x, per_block[i]):.6f}", flush=True)
+            assert err <= 2e-2 and _cosine(x, per_block[i]) >= 0.9995
+        out = model(video.to(gpu), t.to(gpu), text.to(gpu), encoder_hidden_states_image=feats.to(gpu)).sample
+    err = (out.float().cpu() - want).abs().max().item()
+    assert err <= 2e-2 and _cosine(out, want) >= 0.9995
+    assert (no_image - want).abs().max().item() > 10 * err   # the image branch does contribute
+    with pytest.raises(ValueError, match="image tokens"):
+        model.blocks[0].attn2(x, ctx[:, :n_txt])
 
 
 def _wide_block(gpu, seed=0):

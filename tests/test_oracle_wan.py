@@ -125,3 +125,102 @@ def test_fp32_agrees_with_fp64():
     got = ow.transformer_forward(w32, cfg, video.float(), t.float(), text.float())
     assert got.shape == video.shape
     torch.testing.assert_close(got.double(), want, atol=5e-4, rtol=1e-3)
+
+
+# ---------------------------------------------------------------------- per-token timesteps (TI2V)
+def test_per_token_timesteps_all_equal_reduce_to_the_scalar_form():
+    cfg, w, video, text, t = _setup(B=2)
+    S = 2 * 2 * 3
+    want = ow.transformer_forward(w, cfg, video, t, text)
+    got = ow.transformer_forward(w, cfg, video, t[:, None].expand(2, S).contiguous(), text)
+    torch.testing.assert_close(got, want, atol=1e-12, rtol=0)
+
+
+def test_per_token_timesteps_are_token_local_when_attention_is_cut():
+    """Self- and cross-attention output projections zeroed: every token is processed on its own, so with
+    two timestep values spread over the tokens each token must come out as in the scalar-timestep run
+    with its own value - through both modulations, both gates and the head."""
+    cfg, w, video, text, _ = _setup(B=1)
+    w = dict(w)
+    for i in range(cfg.num_layers):
+        for a in ("attn1", "attn2"):
+            for kind in ("weight", "bias"):
+                w[f"blocks.{i}.{a}.to_out.{kind}"] = torch.zeros_like(w[f"blocks.{i}.{a}.to_out.{kind}"])
+    S = 12
+    ta, tb = 130.0, 860.0
+    pick = torch.tensor([0, 1, 1, 0, 0, 0, 1, 0, 1, 1, 0, 1], dtype=torch.bool)
+    ts = torch.where(pick, torch.tensor(tb), torch.tensor(ta)).to(video.dtype)[None]
+    mixed = ow.transformer_forward(w, cfg, video, ts, text)
+    out_a = ow.transformer_forward(w, cfg, video, torch.tensor([ta], dtype=video.dtype), text)
+    out_b = ow.transformer_forward(w, cfg, video, torch.tensor([tb], dtype=video.dtype), text)
+    # token (f, h, w) of the 2x2x3 patch grid owns output pixels [:, :, f, 2h:2h+2, 2w:2w+2]
+    for tok in range(S):
+        f, h, x = tok // 6, (tok % 6) // 3, tok % 3
+        sl = (slice(None), slice(None), slice(f, f + 1), slice(2 * h, 2 * h + 2), slice(2 * x, 2 * x + 2))
+        torch.testing.assert_close(mixed[sl], (out_b if pick[tok] else out_a)[sl], atol=1e-12, rtol=0)
+    assert (out_a - out_b).abs().max().item() > 1e-3
+
+
+# ---------------------------------------------------------------------- image conditioning (I2V)
+def _i2v_setup(seed=0, B=1, n_img=7, n_txt=5, pos=False):
+    import dataclasses
+
+    cfg = dataclasses.replace(ow.tiny_config(), image_dim=48, added_kv_proj_dim=256, text_context_len=n_txt,
+                              pos_embed_seq_len=2 * n_img if pos else None)
+    w = {k: v.double() for k, v in ow.init_params(cfg, seed=seed, std=0.05, bias_std=0.05, norm_jitter=0.1).items()}
+    g = torch.Generator().manual_seed(seed + 1)
+    video = torch.randn(B, cfg.in_channels, 2, 4, 6, generator=g, dtype=torch.float64)
+    text = torch.randn(B, n_txt, cfg.text_dim, generator=g, dtype=torch.float64)
+    feats = torch.randn(2 * B if pos else B, n_img, cfg.image_dim, generator=g, dtype=torch.float64)
+    t = torch.tensor([417.0, 902.0][:B], dtype=torch.float64)
+    return cfg, w, video, text, feats, t
+
+
+def test_image_embedder_against_library_modules():
+    cfg, w, _, _, feats, _ = _i2v_setup()
+    p = "condition_embedder.image_embedder."
+    n1, n2 = torch.nn.LayerNorm(48).double(), torch.nn.LayerNorm(256).double()
+    l1, l2 = torch.nn.Linear(48, 48).double(), torch.nn.Linear(48, 256).double()
+    with torch.no_grad():
+        for m, name in ((n1, "norm1"), (n2, "norm2"), (l1, "ff.net.0.proj"), (l2, "ff.net.2")):
+            m.weight.copy_(w[p + name + ".weight"])
+            m.bias.copy_(w[p + name + ".bias"])
+        want = n2(l2(torch.nn.GELU()(l1(n1(feats)))))
+    torch.testing.assert_close(ow.image_embedder(w, cfg, feats), want, atol=1e-6, rtol=0)  # norms run in fp32
+    # learned positions: rows of two consecutive entries are joined before the positions are added
+    cfg2, w2, _, _, feats2, _ = _i2v_setup(pos=True)
+    joined = ow.image_embedder(w2, cfg2, feats2)
+    assert joined.shape == (1, 14, 256)
+    w3 = dict(w2)
+    pe = w3.pop(p + "pos_embed")
+    shifted = torch.cat([feats2[0], feats2[1]], dim=0)[None] + pe
+    torch.testing.assert_close(joined, ow.image_embedder(w3, cfg2, shifted), atol=1e-12, rtol=0)
+
+
+def test_image_branch_is_a_second_softmax_added_to_the_text_attention():
+    """A dead image value projection must give the text-only model (pins the split point of the context
+    and that the two attentions are added, not merged into one softmax); permuting the image tokens must
+    change nothing; and doubling the image branch's contribution by duplicating every image token must
+    change nothing either (a separate softmax is invariant to key duplication, a plain sum is not)."""
+    cfg, w, video, text, feats, t = _i2v_setup()
+    import dataclasses
+
+    base = ow.transformer_forward(w, cfg, video, t, text, image_feats=feats)
+    dead = dict(w)
+    for i in range(cfg.num_layers):
+        for kind in ("weight", "bias"):
+            dead[f"blocks.{i}.attn2.add_v_proj.{kind}"] = torch.zeros_like(w[f"blocks.{i}.attn2.add_v_proj.{kind}"])
+    text_only_cfg = dataclasses.replace(cfg, image_dim=None, added_kv_proj_dim=None)
+    torch.testing.assert_close(ow.transformer_forward(dead, cfg, video, t, text, image_feats=feats),
+                               ow.transformer_forward(w, text_only_cfg, video, t, text), atol=1e-12, rtol=0)
+    assert (base - ow.transformer_forward(w, text_only_cfg, video, t, text)).abs().max().item() > 1e-4
+    perm = torch.randperm(feats.shape[1], generator=torch.Generator().manual_seed(3))
+    torch.testing.assert_close(ow.transformer_forward(w, cfg, video, t, text, image_feats=feats[:, perm]), base,
+                               atol=2e-6, rtol=0)  # softmax and RMS statistics are fp32 inside the oracle
+    twice = torch.cat([feats, feats], dim=1)
+    torch.testing.assert_close(ow.transformer_forward(w, cfg, video, t, text, image_feats=twice), base,
+                               atol=2e-6, rtol=0)
+    # a text token moved into the image slice would break the count: the context is [image; text]
+    x, temb, temb6, ctx = ow.stem(w, cfg, video, t, text, feats)
+    assert ctx.shape[1] == feats.shape[1] + text.shape[1]
+    torch.testing.assert_close(ctx[:, :feats.shape[1]], ow.image_embedder(w, cfg, feats), atol=0, rtol=0)

@@ -49,12 +49,12 @@ _SIGNATURES = {
     "odit_adaln_modulate": (
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
-         C.c_int, C.c_int, C.c_int, _i64p, _i64p, C.c_int64, C.c_float, C.c_int, C.c_int,
-         C.c_uint, C.c_void_p],
+         C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, _i64p, _i64p, C.c_int64, C.c_int64,
+         C.c_float, C.c_int, C.c_int, C.c_uint, C.c_void_p],
     ),
     "odit_gated_residual": (
         C.c_int,
-        [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
+        [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
          _i64p, _i64p, _i64p, _i64p, C.c_int, C.c_int, C.c_uint, C.c_void_p],
     ),
     "odit_rel_l1_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int64]),

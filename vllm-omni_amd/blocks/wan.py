@@ -16,8 +16,11 @@ interfaces:
     timestep only and are formed for all blocks in one small op per step;
   * self-attention (S x S) and cross-attention (S x 512, no rotary) both run on the flash kernel.
 
-Not built: per-token timesteps (``temb.ndim == 4``, wan.py:641-652) and the image branch of the
-cross-attention (``added_kv_proj_dim``, wan.py:541-575); both raise NotImplementedError.
+Per-token timesteps (``timestep`` [B,S], ``temb`` [B,S,6,C], wan.py:641-652): the table + temb sums are
+never formed in memory; the modulation and gating kernels read the per-token 16-bit rows and add the
+float32 table rows in registers. Image conditioning (``image_dim`` / ``added_kv_proj_dim``,
+wan.py:224-248, 541-575): a second attention of the same queries over the embedded image tokens, added
+to the text attention before the output projection.
 """
 
 from __future__ import annotations
@@ -162,13 +165,20 @@ class WanSelfAttention(nn.Module):
 
 
 class WanCrossAttention(nn.Module):
-    """wan.py:433-586 without the image branch."""
+    """wan.py:433-586. With ``added_kv_proj_dim`` the context is [image tokens; ``text_context_len`` text
+    tokens] (the reference hardcodes 512, wan.py:540-543) and the image tokens get their own k/v
+    projections, k norm and softmax."""
 
     def __init__(self, dim: int, num_heads: int, head_dim: int, eps: float = 1e-5,
-                 added_kv_proj_dim: int | None = None):
+                 added_kv_proj_dim: int | None = None, text_context_len: int = 512):
         super().__init__()
+        self.added_kv_proj_dim, self.text_context_len = added_kv_proj_dim, text_context_len
         if added_kv_proj_dim is not None:
-            raise NotImplementedError("image-conditioned cross-attention (added_kv_proj_dim) is not built")
+            self.add_k_proj = nn.Linear(added_kv_proj_dim, num_heads * head_dim, bias=True)
+            self.add_v_proj = nn.Linear(added_kv_proj_dim, num_heads * head_dim, bias=True)
+            self.norm_added_k = DistributedRMSNorm(num_heads * head_dim, eps=eps)
+        else:
+            self.add_k_proj = self.add_v_proj = self.norm_added_k = None
         self.dim, self.num_heads, self.head_dim = dim, num_heads, head_dim
         self.inner_dim = num_heads * head_dim
         self.to_q = nn.Linear(dim, self.inner_dim, bias=True)
@@ -184,17 +194,31 @@ class WanCrossAttention(nn.Module):
                 residual: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
         """With ``residual``: residual + attention output (written to ``out`` when given)."""
         B, S, _ = hidden_states.shape
-        T = encoder_hidden_states.shape[1]
         H, D = self.num_heads, self.head_dim
-        q_in = self.to_q(hidden_states).view(B, S, H, D)
-        k_in = self.to_k(encoder_hidden_states).view(B, T, H, D)
-        q, k = torch.empty_like(q_in), torch.empty_like(k_in)
-        kernels.qknorm_rope(q_in, None, None, q, None, None, self.norm_q.weight, None, None, None,
-                            eps=self.norm_q.eps, norm_mode=ODIT_NORM_ROW)
-        kernels.qknorm_rope(k_in, None, None, k, None, None, self.norm_k.weight, None, None, None,
-                            eps=self.norm_k.eps, norm_mode=ODIT_NORM_ROW)
+        ctx_img = None
+        if self.add_k_proj is not None:
+            n_img = encoder_hidden_states.shape[1] - self.text_context_len
+            if n_img <= 0:
+                raise ValueError(f"image-conditioned cross-attention expects image tokens in front of "
+                                 f"{self.text_context_len} text tokens, got {encoder_hidden_states.shape[1]} in all")
+            ctx_img, encoder_hidden_states = encoder_hidden_states[:, :n_img], encoder_hidden_states[:, n_img:]
+        T = encoder_hidden_states.shape[1]
+
+        def normed(x_in: torch.Tensor, norm: DistributedRMSNorm) -> torch.Tensor:
+            out_ = torch.empty_like(x_in)
+            kernels.qknorm_rope(x_in, None, None, out_, None, None, norm.weight, None, None, None,
+                                eps=norm.eps, norm_mode=ODIT_NORM_ROW)
+            return out_
+
+        q = normed(self.to_q(hidden_states).view(B, S, H, D), self.norm_q)
+        k = normed(self.to_k(encoder_hidden_states).view(B, T, H, D), self.norm_k)
         v = self.to_v(encoder_hidden_states).view(B, T, H, D)
         o = self.attn(q, k, v).flatten(2, 3)
+        if ctx_img is not None:
+            k_img = normed(self.add_k_proj(ctx_img).view(B, n_img, H, D), self.norm_added_k)
+            v_img = self.add_v_proj(ctx_img).view(B, n_img, H, D)
+            o_img = self.attn(q, k_img, v_img).flatten(2, 3)
+            o = kernels.gated_residual(o, o_img, None, out=o)  # two separate softmaxes, summed (wan.py:577-579)
         if residual is not None:
             return project_residual(self.to_out, o, residual, None, out=out)
         return self.to_out(o)
@@ -205,22 +229,32 @@ class FP32LayerNorm(nn.LayerNorm):
 
 
 class WanTransformerBlock(nn.Module):
-    """wan.py:589-675 (T2V form): self-attention, cross-attention, feed-forward."""
+    """wan.py:589-675: self-attention, cross-attention, feed-forward."""
 
     def __init__(self, dim: int, ffn_dim: int, num_heads: int, eps: float = 1e-6,
-                 added_kv_proj_dim: int | None = None, cross_attn_norm: bool = False):
+                 added_kv_proj_dim: int | None = None, cross_attn_norm: bool = False,
+                 text_context_len: int = 512):
         super().__init__()
         head_dim = dim // num_heads
         self.eps = eps
         self.norm1 = FP32LayerNorm(dim, eps, elementwise_affine=False)
         self.attn1 = WanSelfAttention(dim=dim, num_heads=num_heads, head_dim=head_dim, eps=eps)
         self.attn2 = WanCrossAttention(dim=dim, num_heads=num_heads, head_dim=head_dim, eps=eps,
-                                       added_kv_proj_dim=added_kv_proj_dim)
+                                       added_kv_proj_dim=added_kv_proj_dim, text_context_len=text_context_len)
         self.norm2 = FP32LayerNorm(dim, eps, elementwise_affine=True) if cross_attn_norm else nn.Identity()
         self.ffn = WanFeedForward(dim=dim, inner_dim=ffn_dim, dim_out=dim)
         self.norm3 = FP32LayerNorm(dim, eps, elementwise_affine=False)
         self.scale_shift_table = nn.Parameter(torch.randn(1, 6, dim) / dim ** 0.5)
         self._ln2_f32: tuple[int, torch.Tensor, torch.Tensor] | None = None
+        self._table_f32: tuple[tuple, torch.Tensor] | None = None
+
+    def _table(self) -> torch.Tensor:
+        """float32 [6, C] copy of scale_shift_table, refreshed when the parameter changes."""
+        p = self.scale_shift_table
+        tag = (p._version, p.data_ptr(), p.device)
+        if self._table_f32 is None or self._table_f32[0] != tag:
+            self._table_f32 = (tag, p.detach().float().reshape(6, -1).contiguous())
+        return self._table_f32[1]
 
     def _norm2_affine(self):
         """float32 copies of norm2's weight/bias, refreshed when the parameters change."""
@@ -236,8 +270,8 @@ class WanTransformerBlock(nn.Module):
         """``mod`` = float32 [B, 6, C] = scale_shift_table + temb when the caller formed it for all
         blocks at once; otherwise it is formed here as in the reference. ``gate_bias`` = float32 [B, 2, C]:
         the two gates times the biases of the projections they scale (attn1.to_out, ffn.net_2)."""
-        if temb is not None and temb.ndim == 4:
-            raise NotImplementedError("per-token timesteps (temb [B,S,6,C]) are not built")
+        if mod is None and temb.ndim == 4:
+            return self._forward_per_token(hidden_states, encoder_hidden_states, temb, rotary_emb)
         if mod is None:
             mod = self.scale_shift_table + temb.float()
         shift_msa, scale_msa, gate_msa, c_shift, c_scale, c_gate = (mod[:, i] for i in range(6))
@@ -256,6 +290,28 @@ class WanTransformerBlock(nn.Module):
         return project_residual(self.ffn.net_2, self.ffn.net_0(n), x, c_gate, out=x, pre=pre2)
 
 
+    def _forward_per_token(self, x: torch.Tensor, ctx: torch.Tensor, temb: torch.Tensor, rotary_emb) -> torch.Tensor:
+        """temb [B, S, 6, C] (wan.py:641-652): every token has its own six modulation rows. The reference
+        forms table + temb.float() as six float32 [B,S,C] tensors per block; here the kernels read the
+        rows of ``temb`` as they are and add the float32 table row in registers — the same fp32 sum."""
+        if temb.shape[:2] != x.shape[:2] or temb.shape[2] != 6 or temb.stride(-1) != 1:
+            raise ValueError(f"per-token temb must be [B,S,6,C] matching x, got {tuple(temb.shape)}")
+        tab = self._table()
+        row = lambda i: temb[:, :, i]  # noqa: E731  ([B,S,C] view, token stride 6C)
+        n = kernels.adaln_modulate(x, row(0), row(1), eps=self.eps, shift_bias=tab[0], scale_bias=tab[1])
+        a = self.attn1(n, rotary_emb)
+        x = kernels.gated_residual(x, a, row(2), gate_bias=tab[2])          # new tensor: the input is not written
+        if isinstance(self.norm2, nn.Identity):
+            n = x
+        else:
+            lw, lb = self._norm2_affine()
+            n = kernels.adaln_modulate(x, None, None, eps=self.eps, ln_weight=lw, ln_bias=lb, out=n)
+        x = self.attn2(n, ctx, residual=x, out=x)
+        n = kernels.adaln_modulate(x, row(3), row(4), eps=self.eps, shift_bias=tab[3], scale_bias=tab[4],
+                                   out=n if n is not x else None)
+        return kernels.gated_residual(x, self.ffn(n), row(5), out=x, gate_bias=tab[5])
+
+
 class PixArtAlphaTextProjection(nn.Module):
     """Linear -> GELU(tanh) -> Linear (the ``act_fn="gelu_tanh"`` form, wan.py:269)."""
 
@@ -269,29 +325,75 @@ class PixArtAlphaTextProjection(nn.Module):
         return self.linear_2(kernels.gelu_tanh(y, out=y))
 
 
+class _ImageFeedForward(nn.Module):
+    """diffusers ``FeedForward(mult=1, activation_fn="gelu")`` of the image embedder: parameter names
+    ``net.0.proj`` / ``net.2``, exact (erf) GELU between them."""
+
+    def __init__(self, dim: int, dim_out: int):
+        super().__init__()
+        act = nn.Module()
+        act.proj = nn.Linear(dim, dim)
+        self.net = nn.ModuleList([act, nn.Identity(), nn.Linear(dim, dim_out)])
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.net[2](F.gelu(self.net[0].proj(x)))
+
+
+class WanImageEmbedding(nn.Module):
+    """wan.py:224-248: (learned positions over the joined first/last-frame tokens) -> LayerNorm -> MLP ->
+    LayerNorm on the image-encoder tokens; a few hundred rows once per step. The two norms are the
+    reference's default-constructed FP32LayerNorm: eps 1e-5 with an affine pair."""
+
+    def __init__(self, in_features: int, out_features: int, pos_embed_seq_len: int | None = None):
+        super().__init__()
+        self.norm1 = FP32LayerNorm(in_features)
+        self.ff = _ImageFeedForward(in_features, out_features)
+        self.norm2 = FP32LayerNorm(out_features)
+        self.pos_embed = (nn.Parameter(torch.zeros(1, pos_embed_seq_len, in_features))
+                          if pos_embed_seq_len is not None else None)
+
+    @staticmethod
+    def _norm(ln: nn.LayerNorm, x: torch.Tensor) -> torch.Tensor:
+        return kernels.adaln_modulate(x, None, None, eps=ln.eps, ln_weight=ln.weight.detach().float().contiguous(),
+                                      ln_bias=ln.bias.detach().float().contiguous())
+
+    def forward(self, encoder_hidden_states_image: torch.Tensor) -> torch.Tensor:
+        x = encoder_hidden_states_image
+        if self.pos_embed is not None:
+            _, n, e = x.shape
+            x = x.reshape(-1, 2 * n, e) + self.pos_embed
+        return self._norm(self.norm2, self.ff(self._norm(self.norm1, x.contiguous())))
+
+
 class WanTimeTextImageEmbedding(nn.Module):
-    """wan.py:251-296 without the image embedder."""
+    """wan.py:251-296."""
 
     def __init__(self, dim: int, time_freq_dim: int, time_proj_dim: int, text_embed_dim: int,
                  image_embed_dim: int | None = None, pos_embed_seq_len: int | None = None):
         super().__init__()
-        if image_embed_dim is not None:
-            raise NotImplementedError("the image embedder of the I2V variants is not built")
         self.time_freq_dim = time_freq_dim
         self.time_embedder = TimestepEmbedding(time_freq_dim, dim)
         self.time_proj = nn.Linear(dim, time_proj_dim)
         self.text_embedder = PixArtAlphaTextProjection(text_embed_dim, dim)
-        self.image_embedder = None
+        self.image_embedder = (WanImageEmbedding(image_embed_dim, dim, pos_embed_seq_len=pos_embed_seq_len)
+                               if image_embed_dim is not None else None)
 
     def forward(self, timestep: torch.Tensor, encoder_hidden_states: torch.Tensor,
                 encoder_hidden_states_image: torch.Tensor | None = None, timestep_seq_len: int | None = None):
-        if timestep_seq_len is not None or encoder_hidden_states_image is not None:
-            raise NotImplementedError("per-token timesteps / image conditioning are not built")
+        """timestep [B] -> temb [B,C], timestep_proj [B,6C]; flattened per-token timesteps [B*S] with
+        ``timestep_seq_len`` = S -> temb [B,S,C], timestep_proj [B,S,6C] (wan.py:282-296)."""
         t = QwenTimestepProjEmbeddings.time_proj(timestep, dim=self.time_freq_dim, scale=1.0)
+        if timestep_seq_len is not None:
+            t = t.unflatten(0, (-1, timestep_seq_len))
         t = t.to(self.time_embedder.linear_1.weight.dtype)
         temb = self.time_embedder(t).type_as(encoder_hidden_states)
         timestep_proj = self.time_proj(kernels.silu(temb))
-        return temb, timestep_proj, self.text_embedder(encoder_hidden_states), None
+        image = None
+        if encoder_hidden_states_image is not None:
+            if self.image_embedder is None:
+                raise ValueError("image features given to a model built without image_dim")
+            image = self.image_embedder(encoder_hidden_states_image)
+        return temb, timestep_proj, self.text_embedder(encoder_hidden_states), image
 
 
 class OutputScaleShiftPrepare(nn.Module):
@@ -300,8 +402,10 @@ class OutputScaleShiftPrepare(nn.Module):
         self.scale_shift_table = nn.Parameter(torch.randn(1, 2, inner_dim) / inner_dim ** 0.5)
 
     def forward(self, temb: torch.Tensor):
+        """temb [B,C] -> shift, scale [B,C]; per-token temb [B,S,C] -> [B,S,C] each (wan.py:324-337)."""
         if temb.ndim == 3:
-            raise NotImplementedError("per-token timesteps are not built")
+            shift, scale = (self.scale_shift_table.unsqueeze(0) + temb.unsqueeze(2)).chunk(2, dim=2)
+            return shift.squeeze(2), scale.squeeze(2)
         shift, scale = (self.scale_shift_table + temb.unsqueeze(1)).chunk(2, dim=1)
         return shift.squeeze(1), scale.squeeze(1)
 
@@ -317,7 +421,8 @@ class WanTransformer3DModel(nn.Module):
                  attention_head_dim: int = 128, in_channels: int = 16, out_channels: int = 16, text_dim: int = 4096,
                  freq_dim: int = 256, ffn_dim: int = 13824, num_layers: int = 40, cross_attn_norm: bool = True,
                  eps: float = 1e-6, image_dim: int | None = None, added_kv_proj_dim: int | None = None,
-                 rope_max_seq_len: int = 1024, pos_embed_seq_len: int | None = None):
+                 rope_max_seq_len: int = 1024, pos_embed_seq_len: int | None = None,
+                 text_context_len: int = 512):
         super().__init__()
         inner_dim = num_attention_heads * attention_head_dim
         self.patch_size, self.inner_dim, self.eps = tuple(patch_size), inner_dim, eps
@@ -329,7 +434,8 @@ class WanTransformer3DModel(nn.Module):
                                                             image_embed_dim=image_dim,
                                                             pos_embed_seq_len=pos_embed_seq_len)
         self.blocks = nn.ModuleList([
-            WanTransformerBlock(inner_dim, ffn_dim, num_attention_heads, eps, added_kv_proj_dim, cross_attn_norm)
+            WanTransformerBlock(inner_dim, ffn_dim, num_attention_heads, eps, added_kv_proj_dim, cross_attn_norm,
+                                text_context_len=text_context_len)
             for _ in range(num_layers)])
         self.norm_out = FP32LayerNorm(inner_dim, eps, elementwise_affine=False)
         self.proj_out = nn.Linear(inner_dim, self.out_channels * math.prod(patch_size))
@@ -349,13 +455,22 @@ class WanTransformer3DModel(nn.Module):
         x = x.permute(0, 2, 4, 6, 1, 3, 5, 7).reshape(B, -1, Cin * p_t * p_h * p_w)
         return F.linear(x, self.patch_embedding.weight.view(self.inner_dim, -1), self.patch_embedding.bias)
 
-    def prepare(self, hidden_states: torch.Tensor, timestep: torch.Tensor, encoder_hidden_states: torch.Tensor):
-        if timestep.ndim == 2:
-            raise NotImplementedError("per-token timesteps are not built")
+    def prepare(self, hidden_states: torch.Tensor, timestep: torch.Tensor, encoder_hidden_states: torch.Tensor,
+                encoder_hidden_states_image: torch.Tensor | None = None):
+        """-> tokens, context, temb, timestep_proj ([B,6,C], or [B,S,6,C] for per-token timesteps [B,S]),
+        rotary. Image tokens, when given, are embedded and put in front of the text tokens (wan.py:878-879)."""
         rotary = self.rope(hidden_states)
         x = self.patchify(hidden_states)
-        temb, tproj, ctx, _ = self.condition_embedder(timestep, encoder_hidden_states)
-        return x, ctx, temb, tproj.unflatten(1, (6, -1)), rotary
+        ts_len = None
+        if timestep.ndim == 2:
+            if timestep.shape[1] != x.shape[1]:
+                raise ValueError(f"per-token timesteps need one value per token: {timestep.shape[1]} vs {x.shape[1]}")
+            ts_len, timestep = timestep.shape[1], timestep.flatten()
+        temb, tproj, ctx, image = self.condition_embedder(timestep, encoder_hidden_states,
+                                                          encoder_hidden_states_image, timestep_seq_len=ts_len)
+        if image is not None:
+            ctx = torch.cat([image, ctx], dim=1)
+        return x, ctx, temb, tproj.unflatten(tproj.ndim - 1, (6, -1)), rotary
 
     def all_modulations(self, timestep_proj: torch.Tensor) -> torch.Tensor:
         """float32 [L, B, 6, C]: every block's scale_shift_table + temb in one op."""
@@ -363,6 +478,10 @@ class WanTransformer3DModel(nn.Module):
         return tables.unsqueeze(1) + timestep_proj.float().unsqueeze(0)
 
     def run_blocks(self, x, ctx, timestep_proj, rotary):
+        if timestep_proj.ndim == 4:  # per-token timesteps: the blocks read the rows of timestep_proj directly
+            for block in self.blocks:
+                x = block(x, ctx, timestep_proj, rotary)
+            return x
         mods = self.all_modulations(timestep_proj)
         gb = None
         if x.dtype != torch.float32:  # gates (rows 2 and 5) times the biases they scale, [L, B, 2, C]
@@ -374,7 +493,9 @@ class WanTransformer3DModel(nn.Module):
 
     def finish(self, x: torch.Tensor, temb: torch.Tensor, grid: tuple[int, int, int], return_dict: bool = True):
         shift, scale = self.output_scale_shift_prepare(temb)
-        x = kernels.adaln_modulate(x, shift.contiguous(), scale.contiguous(), eps=self.eps)
+        if shift.ndim == 2:
+            shift, scale = shift.contiguous(), scale.contiguous()
+        x = kernels.adaln_modulate(x, shift, scale, eps=self.eps)
         x = self.proj_out(x)
         p_t, p_h, p_w = self.patch_size
         x = x.reshape(x.shape[0], *grid, p_t, p_h, p_w, -1).permute(0, 7, 1, 4, 2, 5, 3, 6)
@@ -384,11 +505,10 @@ class WanTransformer3DModel(nn.Module):
     def forward(self, hidden_states: torch.Tensor, timestep: torch.Tensor, encoder_hidden_states: torch.Tensor,
                 encoder_hidden_states_image: torch.Tensor | None = None, return_dict: bool = True,
                 attention_kwargs: dict[str, Any] | None = None):
-        if encoder_hidden_states_image is not None:
-            raise NotImplementedError("image conditioning is not built")
         _, _, nf, hh, ww = hidden_states.shape
         p_t, p_h, p_w = self.patch_size
-        x, ctx, temb, tproj, rotary = self.prepare(hidden_states, timestep, encoder_hidden_states)
+        x, ctx, temb, tproj, rotary = self.prepare(hidden_states, timestep, encoder_hidden_states,
+                                                   encoder_hidden_states_image)
         x = self.run_blocks(x, ctx, tproj, rotary)
         return self.finish(x, temb, (nf // p_t, hh // p_h, ww // p_w), return_dict=return_dict)
 

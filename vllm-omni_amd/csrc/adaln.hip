@@ -45,8 +45,10 @@ template <typename T, typename TM, int W, int NVL, bool REF_ROUND, bool PLAIN>
 __global__ __launch_bounds__(W * 64) void adaln_rows_kernel(
     const T* __restrict__ x, T* __restrict__ out, const TM* __restrict__ shift,
     const TM* __restrict__ scale, const int32_t* __restrict__ index,
-    const float* __restrict__ ln_w, const float* __restrict__ ln_b, int B, int S, int C,
-    int64_t xs_b, int64_t xs_s, int64_t os_b, int64_t os_s, int64_t mod_stride_b, float eps) {
+    const float* __restrict__ ln_w, const float* __restrict__ ln_b,
+    const float* __restrict__ shift_bias, const float* __restrict__ scale_bias, int B, int S, int C,
+    int64_t xs_b, int64_t xs_s, int64_t os_b, int64_t os_s, int64_t mod_stride_b,
+    int64_t mod_stride_s, float eps) {
   constexpr int EPV = Vec16<T>::N;
   const int tid = threadIdx.x;
   const unsigned row = blockIdx.x;  // the launcher keeps B*S below 2^31
@@ -93,8 +95,11 @@ __global__ __launch_bounds__(W * 64) void adaln_rows_kernel(
 
   int mrow = b;
   if (!PLAIN && index != nullptr && index[static_cast<int64_t>(b) * S + s] != 0) mrow = b + B;
-  const TM* sh = (PLAIN || shift) ? shift + mrow * mod_stride_b : nullptr;
-  const TM* sc = (PLAIN || scale) ? scale + mrow * mod_stride_b : nullptr;
+  // per-token modulation rows (mod_stride_s != 0) and the float32 [C] tables added to them are
+  // optional operands like the index: the PLAIN specialisation has neither
+  const int64_t moff = mrow * mod_stride_b + (PLAIN ? 0 : s * mod_stride_s);
+  const TM* sh = (PLAIN || shift) ? shift + moff : nullptr;
+  const TM* sc = (PLAIN || scale) ? scale + moff : nullptr;
 
 #pragma unroll
   for (int i = 0; i < NVL; ++i) {
@@ -106,6 +111,13 @@ __global__ __launch_bounds__(W * 64) void adaln_rows_kernel(
       if (!PLAIN) {
         load_params<float, EPV>(ln_w ? ln_w + c0 : nullptr, 1.f, lw_v);
         load_params<float, EPV>(ln_b ? ln_b + c0 : nullptr, 0.f, lb_v);
+        if (scale_bias || shift_bias) {
+          float scb[EPV], shb[EPV];
+          load_params<float, EPV>(scale_bias ? scale_bias + c0 : nullptr, 0.f, scb);
+          load_params<float, EPV>(shift_bias ? shift_bias + c0 : nullptr, 0.f, shb);
+#pragma unroll
+          for (int j = 0; j < EPV; ++j) { scl_v[j] += scb[j]; shf_v[j] += shb[j]; }
+        }
       }
       float r[EPV];
 #pragma unroll
@@ -133,8 +145,10 @@ template <typename T, typename TM, bool REF_ROUND>
 __global__ __launch_bounds__(256) void adaln_rows_generic_kernel(
     const T* __restrict__ x, T* __restrict__ out, const TM* __restrict__ shift,
     const TM* __restrict__ scale, const int32_t* __restrict__ index,
-    const float* __restrict__ ln_w, const float* __restrict__ ln_b, int B, int S, int C,
-    int64_t xs_b, int64_t xs_s, int64_t os_b, int64_t os_s, int64_t mod_stride_b, float eps) {
+    const float* __restrict__ ln_w, const float* __restrict__ ln_b,
+    const float* __restrict__ shift_bias, const float* __restrict__ scale_bias, int B, int S, int C,
+    int64_t xs_b, int64_t xs_s, int64_t os_b, int64_t os_s, int64_t mod_stride_b,
+    int64_t mod_stride_s, float eps) {
   const int lane = threadIdx.x & 63;
   const int64_t row = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (row >= static_cast<int64_t>(B) * S) return;
@@ -151,14 +165,15 @@ __global__ __launch_bounds__(256) void adaln_rows_generic_kernel(
   const float rstd = rsqrtf(wave_sum(sq) * inv_c + eps);
   int mrow = b;
   if (index != nullptr && index[static_cast<int64_t>(b) * S + s] != 0) mrow = b + B;
-  const TM* sh = shift ? shift + mrow * mod_stride_b : nullptr;
-  const TM* sc = scale ? scale + mrow * mod_stride_b : nullptr;
+  const int64_t moff = mrow * mod_stride_b + s * mod_stride_s;
+  const TM* sh = shift ? shift + moff : nullptr;
+  const TM* sc = scale ? scale + moff : nullptr;
   for (int c = lane; c < C; c += 64) {
     float y = (to_float(xr[c]) - mean) * rstd;
     if (ln_w) y *= ln_w[c];
     if (ln_b) y += ln_b[c];
-    const float scl = ModLoader<TM>::at(sc, c);
-    const float shf = ModLoader<TM>::at(sh, c);
+    const float scl = ModLoader<TM>::at(sc, c) + (scale_bias ? scale_bias[c] : 0.f);
+    const float shf = ModLoader<TM>::at(sh, c) + (shift_bias ? shift_bias[c] : 0.f);
     float r;
     if (REF_ROUND) {
       r = round_to<T>(round_to<T>(y) * round_to<T>(1.f + scl)) + shf;
@@ -171,9 +186,10 @@ __global__ __launch_bounds__(256) void adaln_rows_generic_kernel(
 
 template <typename T, typename TM, bool REF_ROUND>
 static int launch_adaln(const void* x, void* out, const void* shift, const void* scale,
-                        const int32_t* index, const float* ln_w, const float* ln_b, int B, int S,
-                        int C, const int64_t* xs, const int64_t* os, int64_t mod_stride_b, float eps,
-                        hipStream_t stream) {
+                        const int32_t* index, const float* ln_w, const float* ln_b,
+                        const float* shift_bias, const float* scale_bias, int B, int S, int C,
+                        const int64_t* xs, const int64_t* os, int64_t mod_stride_b,
+                        int64_t mod_stride_s, float eps, hipStream_t stream) {
   constexpr int EPV = Vec16<T>::N;
   constexpr int EPM = Vec16<TM>::N;
   const int64_t rows = static_cast<int64_t>(B) * S;
@@ -181,15 +197,17 @@ static int launch_adaln(const void* x, void* out, const void* shift, const void*
   const bool vec_ok = (C % EPV == 0) && aligned16(x) && aligned16(out) && xs[0] % EPV == 0 &&
                       xs[1] % EPV == 0 && os[0] % EPV == 0 && os[1] % EPV == 0 &&
                       aligned16(shift) && aligned16(scale) && mod_stride_b % EPM == 0 &&
-                      aligned16(ln_w) && aligned16(ln_b);
+                      mod_stride_s % EPM == 0 && aligned16(ln_w) && aligned16(ln_b) &&
+                      aligned16(shift_bias) && aligned16(scale_bias);
   const int nvec = (C + EPV - 1) / EPV;  // 16-byte vectors per row
-  const bool plain = shift && scale && !index && !ln_w && !ln_b;
+  const bool plain = shift && scale && !index && !ln_w && !ln_b && !shift_bias && !scale_bias &&
+                     mod_stride_s == 0;
 #define ODIT_ADALN_LAUNCH(WW, NVLL, PL)                                                            \
   hipLaunchKernelGGL((adaln_rows_kernel<T, TM, WW, NVLL, REF_ROUND, PL>),                          \
                      dim3(static_cast<unsigned>(rows)), dim3(WW * 64), 0, stream,                  \
                      static_cast<const T*>(x), static_cast<T*>(out), static_cast<const TM*>(shift), \
-                     static_cast<const TM*>(scale), index, ln_w, ln_b, B, S, C, xs[0], xs[1],      \
-                     os[0], os[1], mod_stride_b, eps)
+                     static_cast<const TM*>(scale), index, ln_w, ln_b, shift_bias, scale_bias, B,  \
+                     S, C, xs[0], xs[1], os[0], os[1], mod_stride_b, mod_stride_s, eps)
 #define ODIT_ADALN_CASE(WW, NVLL)                                                                  \
   do { if (plain) ODIT_ADALN_LAUNCH(WW, NVLL, true); else ODIT_ADALN_LAUNCH(WW, NVLL, false); } while (0)
   if (vec_ok && nvec <= 8 * 64 * 2 && rows <= 0x7fffffffll) {
@@ -205,7 +223,8 @@ static int launch_adaln(const void* x, void* out, const void* shift, const void*
     hipLaunchKernelGGL((adaln_rows_generic_kernel<T, TM, REF_ROUND>), grid, dim3(256), 0, stream,
                        static_cast<const T*>(x), static_cast<T*>(out),
                        static_cast<const TM*>(shift), static_cast<const TM*>(scale), index, ln_w,
-                       ln_b, B, S, C, xs[0], xs[1], os[0], os[1], mod_stride_b, eps);
+                       ln_b, shift_bias, scale_bias, B, S, C, xs[0], xs[1], os[0], os[1],
+                       mod_stride_b, mod_stride_s, eps);
   }
 #undef ODIT_ADALN_CASE
 #undef ODIT_ADALN_LAUNCH
@@ -216,10 +235,11 @@ static int launch_adaln(const void* x, void* out, const void* shift, const void*
 
 extern "C" int odit_adaln_modulate(const void* x, void* out, const void* shift, const void* scale,
                                    const int32_t* index, const float* ln_weight,
-                                   const float* ln_bias, int B, int S, int C,
+                                   const float* ln_bias, const float* shift_bias,
+                                   const float* scale_bias, int B, int S, int C,
                                    const int64_t x_strides[2], const int64_t out_strides[2],
-                                   int64_t mod_stride_b, float eps, int mod_dtype, int dtype,
-                                   unsigned flags, void* stream) {
+                                   int64_t mod_stride_b, int64_t mod_stride_s, float eps,
+                                   int mod_dtype, int dtype, unsigned flags, void* stream) {
   using namespace odit;
   ODIT_CHECK_ARG(x && out, "odit_adaln_modulate: x/out must not be null");
   ODIT_CHECK_ARG(x_strides && out_strides, "odit_adaln_modulate: strides must not be null");
@@ -228,14 +248,19 @@ extern "C" int odit_adaln_modulate(const void* x, void* out, const void* shift, 
                  "odit_adaln_modulate: mod_dtype must equal dtype or be ODIT_F32 (got %d vs %d)",
                  mod_dtype, dtype);
   ODIT_CHECK_ARG(static_cast<int64_t>(B) * S < (1ll << 33), "odit_adaln_modulate: too many rows");
+  ODIT_CHECK_ARG(mod_stride_b >= 0 && mod_stride_s >= 0, "odit_adaln_modulate: negative modulation stride");
+  ODIT_CHECK_ARG(!(index && mod_stride_s != 0),
+                 "odit_adaln_modulate: per-token modulation rows and a row index exclude each other");
   if (B == 0 || S == 0) return ODIT_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool rr = (flags & ODIT_FLAG_REF_ROUNDING) && mod_dtype == dtype && dtype != ODIT_F32;
 #define ODIT_ADALN_GO(T, TM)                                                                     \
-  return rr ? launch_adaln<T, TM, true>(x, out, shift, scale, index, ln_weight, ln_bias, B, S, C, \
-                                        x_strides, out_strides, mod_stride_b, eps, st)           \
-            : launch_adaln<T, TM, false>(x, out, shift, scale, index, ln_weight, ln_bias, B, S, C, \
-                                         x_strides, out_strides, mod_stride_b, eps, st)
+  return rr ? launch_adaln<T, TM, true>(x, out, shift, scale, index, ln_weight, ln_bias,           \
+                                        shift_bias, scale_bias, B, S, C, x_strides, out_strides,  \
+                                        mod_stride_b, mod_stride_s, eps, st)                      \
+            : launch_adaln<T, TM, false>(x, out, shift, scale, index, ln_weight, ln_bias,          \
+                                         shift_bias, scale_bias, B, S, C, x_strides, out_strides, \
+                                         mod_stride_b, mod_stride_s, eps, st)
   if (mod_dtype == dtype) {
     ODIT_DISPATCH_DTYPE(dtype, T, ODIT_ADALN_GO(T, T));
   } else {

@@ -7,11 +7,14 @@ namespace odit {
 
 constexpr int kStreamUnroll = 1;  // 16-byte vectors per thread; measured: more per thread streams slower here
 
-template <typename T, typename TG, bool REF_ROUND>
+// GBIAS: a float32 [C] table is added to the gate (the gate is then table + per-token row, formed in
+// registers); a template parameter so the plain pass carries no trace of it.
+template <typename T, typename TG, bool REF_ROUND, bool GBIAS>
 __global__ __launch_bounds__(256) void gated_residual_kernel(
     const T* __restrict__ h, const T* __restrict__ y, const TG* __restrict__ gate,
-    T* __restrict__ out, int S, int vec_per_row, int64_t total_vecs, int64_t hs_b, int64_t hs_s,
-    int64_t ys_b, int64_t ys_s, int64_t os_b, int64_t os_s, int64_t gs_b, int64_t gs_s) {
+    const float* __restrict__ gate_bias, T* __restrict__ out, int S, int vec_per_row,
+    int64_t total_vecs, int64_t hs_b, int64_t hs_s, int64_t ys_b, int64_t ys_s, int64_t os_b,
+    int64_t os_s, int64_t gs_b, int64_t gs_s) {
   constexpr int EPV = Vec16<T>::N;
   constexpr int EPG = Vec16<TG>::N;
   constexpr int U = kStreamUnroll;
@@ -44,7 +47,15 @@ __global__ __launch_bounds__(256) void gated_residual_kernel(
         }
       } else {
 #pragma unroll
-        for (int j = 0; j < EPV; ++j) g[u][j] = 1.f;
+        for (int j = 0; j < EPV; ++j) g[u][j] = GBIAS ? 0.f : 1.f;
+      }
+      if (GBIAS) {
+#pragma unroll
+        for (int q = 0; q < EPV / 4; ++q) {
+          const Vec16<float> bv = load16(gate_bias + c0 + q * 4);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) g[u][q * 4 + j] += bv.e[j];
+        }
       }
     }
   }
@@ -68,8 +79,9 @@ __global__ __launch_bounds__(256) void gated_residual_kernel(
 template <typename T, typename TG, bool REF_ROUND>
 __global__ __launch_bounds__(256) void gated_residual_scalar_kernel(
     const T* __restrict__ h, const T* __restrict__ y, const TG* __restrict__ gate,
-    T* __restrict__ out, int S, int C, int64_t total, int64_t hs_b, int64_t hs_s, int64_t ys_b,
-    int64_t ys_s, int64_t os_b, int64_t os_s, int64_t gs_b, int64_t gs_s) {
+    const float* __restrict__ gate_bias, T* __restrict__ out, int S, int C, int64_t total,
+    int64_t hs_b, int64_t hs_s, int64_t ys_b, int64_t ys_s, int64_t os_b, int64_t os_s,
+    int64_t gs_b, int64_t gs_s) {
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total;
        i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
     const int64_t row = i / C;
@@ -78,7 +90,8 @@ __global__ __launch_bounds__(256) void gated_residual_scalar_kernel(
     const int s = static_cast<int>(row - static_cast<int64_t>(b) * S);
     const float hf = to_float(h[b * hs_b + s * hs_s + c]);
     const float yf = to_float(y[b * ys_b + s * ys_s + c]);
-    const float g = gate ? to_float(gate[b * gs_b + s * gs_s + c]) : 1.f;
+    const float g = (gate ? to_float(gate[b * gs_b + s * gs_s + c]) : (gate_bias ? 0.f : 1.f)) +
+                    (gate_bias ? gate_bias[c] : 0.f);
     const float r = REF_ROUND ? hf + round_to<T>(g * yf) : fmaf(g, yf, hf);
     out[b * os_b + s * os_s + c] = from_float<T>(r);
   }
@@ -91,30 +104,34 @@ static inline unsigned stream_grid(int64_t work_items) {
 }
 
 template <typename T, typename TG, bool REF_ROUND>
-static int launch_gated(const void* h, const void* y, const void* gate, void* out, int B, int S,
-                        int C, const int64_t* hs, const int64_t* ys, const int64_t* os,
-                        const int64_t* gs, hipStream_t stream) {
+static int launch_gated(const void* h, const void* y, const void* gate, const float* gate_bias,
+                        void* out, int B, int S, int C, const int64_t* hs, const int64_t* ys,
+                        const int64_t* os, const int64_t* gs, hipStream_t stream) {
   constexpr int EPV = Vec16<T>::N;
   constexpr int EPG = Vec16<TG>::N;
   const int64_t gs0 = gs ? gs[0] : 0, gs1 = gs ? gs[1] : 0;
   const bool vec_ok = C % EPV == 0 && aligned16(h) && aligned16(y) && aligned16(out) &&
-                      aligned16(gate) && hs[0] % EPV == 0 && hs[1] % EPV == 0 && ys[0] % EPV == 0 &&
+                      aligned16(gate) && aligned16(gate_bias) && hs[0] % EPV == 0 && hs[1] % EPV == 0 && ys[0] % EPV == 0 &&
                       ys[1] % EPV == 0 && os[0] % EPV == 0 && os[1] % EPV == 0 && gs0 % EPG == 0 &&
                       gs1 % EPG == 0;
   if (vec_ok) {
     const int vpr = C / EPV;
     const int64_t total = static_cast<int64_t>(B) * S * vpr;
     const int64_t nblk = (total + 256 * kStreamUnroll - 1) / (256 * kStreamUnroll);
-    hipLaunchKernelGGL((gated_residual_kernel<T, TG, REF_ROUND>), dim3(static_cast<unsigned>(nblk)),
-                       dim3(256), 0, stream, static_cast<const T*>(h), static_cast<const T*>(y),
-                       static_cast<const TG*>(gate), static_cast<T*>(out), S, vpr, total, hs[0],
-                       hs[1], ys[0], ys[1], os[0], os[1], gs0, gs1);
+#define ODIT_GATED_LAUNCH(GB)                                                                      \
+  hipLaunchKernelGGL((gated_residual_kernel<T, TG, REF_ROUND, GB>),                                \
+                     dim3(static_cast<unsigned>(nblk)), dim3(256), 0, stream,                      \
+                     static_cast<const T*>(h), static_cast<const T*>(y),                           \
+                     static_cast<const TG*>(gate), gate_bias, static_cast<T*>(out), S, vpr, total, \
+                     hs[0], hs[1], ys[0], ys[1], os[0], os[1], gs0, gs1)
+    if (gate_bias) ODIT_GATED_LAUNCH(true); else ODIT_GATED_LAUNCH(false);
+#undef ODIT_GATED_LAUNCH
   } else {
     const int64_t total = static_cast<int64_t>(B) * S * C;
     hipLaunchKernelGGL((gated_residual_scalar_kernel<T, TG, REF_ROUND>), dim3(stream_grid(total)),
                        dim3(256), 0, stream, static_cast<const T*>(h), static_cast<const T*>(y),
-                       static_cast<const TG*>(gate), static_cast<T*>(out), S, C, total, hs[0], hs[1],
-                       ys[0], ys[1], os[0], os[1], gs0, gs1);
+                       static_cast<const TG*>(gate), gate_bias, static_cast<T*>(out), S, C, total,
+                       hs[0], hs[1], ys[0], ys[1], os[0], os[1], gs0, gs1);
   }
   return check_launch("odit_gated_residual");
 }
@@ -171,8 +188,9 @@ static int launch_unary(const void* x, void* out, int64_t n, hipStream_t stream,
 
 }  // namespace odit
 
-extern "C" int odit_gated_residual(const void* h, const void* y, const void* gate, void* out, int B,
-                                   int S, int C, const int64_t h_strides[2],
+extern "C" int odit_gated_residual(const void* h, const void* y, const void* gate,
+                                   const float* gate_bias, void* out, int B, int S, int C,
+                                   const int64_t h_strides[2],
                                    const int64_t y_strides[2], const int64_t out_strides[2],
                                    const int64_t gate_strides[2], int gate_dtype, int dtype,
                                    unsigned flags, void* stream) {
@@ -188,10 +206,10 @@ extern "C" int odit_gated_residual(const void* h, const void* y, const void* gat
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool rr = (flags & ODIT_FLAG_REF_ROUNDING) && gate_dtype == dtype && dtype != ODIT_F32;
 #define ODIT_GR_GO(T, TG)                                                                       \
-  return rr ? launch_gated<T, TG, true>(h, y, gate, out, B, S, C, h_strides, y_strides,         \
-                                        out_strides, gate_strides, st)                          \
-            : launch_gated<T, TG, false>(h, y, gate, out, B, S, C, h_strides, y_strides,        \
-                                         out_strides, gate_strides, st)
+  return rr ? launch_gated<T, TG, true>(h, y, gate, gate_bias, out, B, S, C, h_strides,         \
+                                        y_strides, out_strides, gate_strides, st)               \
+            : launch_gated<T, TG, false>(h, y, gate, gate_bias, out, B, S, C, h_strides,        \
+                                         y_strides, out_strides, gate_strides, st)
   if (gate_dtype == dtype) {
     ODIT_DISPATCH_DTYPE(dtype, T, ODIT_GR_GO(T, T));
   } else {

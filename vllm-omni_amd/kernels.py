@@ -240,39 +240,56 @@ def adaln_modulate(
     index: torch.Tensor | None = None,
     ln_weight: torch.Tensor | None = None,
     ln_bias: torch.Tensor | None = None,
+    shift_bias: torch.Tensor | None = None,
+    scale_bias: torch.Tensor | None = None,
     ref_rounding: bool = False,
     out: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """LayerNorm(x) * (1 + scale) + shift for x [B,S,C]; shift/scale [Bm,C] views of one modulation
-    tensor (Bm = B, or 2B with a per-token `index` [B,S] choosing row b or b+B)."""
-    _dev(x, shift, scale, index, ln_weight, ln_bias, out)
+    tensor (Bm = B, or 2B with a per-token `index` [B,S] choosing row b or b+B), or [B,S,C] views with
+    one row per token. ``shift_bias`` / ``scale_bias``: float32 [C] tables added to the rows in fp32."""
+    _dev(x, shift, scale, index, ln_weight, ln_bias, shift_bias, scale_bias, out)
     if x.dim() != 3:
         raise ValueError("adaln_modulate expects x [B,S,C]")
     B, S, Cdim = x.shape
     _last_contig(x, "x")
     mod_dtype = _code(x)
-    mod_stride = 0
+    mod_stride, mod_stride_s = 0, 0
     rows_needed = 2 * B if index is not None else B
+    first = shift if shift is not None else scale
+    per_token = first is not None and first.dim() == 3
+    if per_token and index is not None:
+        raise ValueError("per-token shift/scale rows and an index exclude each other")
     for name, t in (("shift", shift), ("scale", scale)):
         if t is None:
             continue
-        if t.dim() != 2 or t.shape[1] != Cdim or t.shape[0] < rows_needed:
+        if per_token:
+            if tuple(t.shape) != (B, S, Cdim):
+                raise ValueError(f"{name}: expected [{B},{S},{Cdim}], got {tuple(t.shape)}")
+        elif t.dim() != 2 or t.shape[1] != Cdim or t.shape[0] < rows_needed:
             raise ValueError(f"{name}: expected [{rows_needed},{Cdim}], got {tuple(t.shape)}")
         _last_contig(t, name)
         mod_dtype = _code(t)
     if shift is not None and scale is not None:
-        if shift.dtype != scale.dtype or shift.stride(0) != scale.stride(0):
-            raise ValueError("shift and scale must share dtype and batch stride")
-    first = shift if shift is not None else scale
+        if shift.dtype != scale.dtype or shift.stride()[:-1] != scale.stride()[:-1]:
+            raise ValueError("shift and scale must share dtype and strides")
     if first is not None:
-        mod_stride = first.stride(0) if first.shape[0] > 1 else first.shape[1]
+        mod_stride = first.stride(0) if first.shape[0] > 1 else 0
+        if per_token:
+            mod_stride_s = first.stride(1) if S > 1 else Cdim
+            if mod_stride_s == 0:  # an expanded row: the same as one row per batch entry
+                per_token = False
+        elif first.shape[0] == 1:
+            mod_stride = first.shape[1]
     if index is not None:
         if tuple(index.shape) != (B, S):
             raise ValueError(f"index must be [B,S]={B, S}")
         index = index.to(torch.int32).contiguous()
-    for name, t in (("ln_weight", ln_weight), ("ln_bias", ln_bias)):
-        if t is not None and (t.dtype != torch.float32 or t.numel() != Cdim or not t.is_contiguous()):
-            raise ValueError(f"{name}: expected contiguous float32 [{Cdim}]")
+    for name, t in (("ln_weight", ln_weight), ("ln_bias", ln_bias), ("shift_bias", shift_bias),
+                    ("scale_bias", scale_bias)):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != Cdim or t.dim() == 0 or t.stride(-1) != 1
+                              or t.numel() != t.shape[-1]):
+            raise ValueError(f"{name}: expected float32 [{Cdim}] with unit stride")
     if out is None:
         out = torch.empty((B, S, Cdim), dtype=x.dtype, device=x.device)
     elif tuple(out.shape) != (B, S, Cdim) or out.dtype != x.dtype or out.stride(-1) != 1:
@@ -280,8 +297,8 @@ def adaln_modulate(
     lib = _lib.load()
     rc = lib.odit_adaln_modulate(
         x.data_ptr(), out.data_ptr(), _ptr(shift), _ptr(scale), _ptr(index), _ptr(ln_weight),
-        _ptr(ln_bias), B, S, Cdim, _lib.i64_array(x.stride()[:2]), _lib.i64_array(out.stride()[:2]),
-        int(mod_stride), float(eps), mod_dtype, _code(x),
+        _ptr(ln_bias), _ptr(shift_bias), _ptr(scale_bias), B, S, Cdim, _lib.i64_array(x.stride()[:2]),
+        _lib.i64_array(out.stride()[:2]), int(mod_stride), int(mod_stride_s), float(eps), mod_dtype, _code(x),
         ODIT_FLAG_REF_ROUNDING if ref_rounding else 0, _stream(),
     )
     _lib.check(rc, "odit_adaln_modulate")
@@ -296,9 +313,14 @@ def gated_residual(
     *,
     out: torch.Tensor | None = None,
     ref_rounding: bool = False,
+    gate_bias: torch.Tensor | None = None,
 ) -> torch.Tensor:
-    """h + gate * y for h,y [B,S,C]; gate [B,C], [B,1,C] (broadcast over S) or [B,S,C]; None = ones."""
-    _dev(h, y, gate, out)
+    """h + gate * y for h,y [B,S,C]; gate [B,C], [B,1,C] (broadcast over S) or [B,S,C]; None = ones.
+    ``gate_bias``: float32 [C] table added to the gate in fp32 (alone it is the gate)."""
+    _dev(h, y, gate, out, gate_bias)
+    if gate_bias is not None and (gate_bias.dtype != torch.float32 or gate_bias.numel() != h.shape[-1]
+                                  or gate_bias.stride(-1) != 1 or gate_bias.numel() != gate_bias.shape[-1]):
+        raise ValueError(f"gate_bias: expected float32 [{h.shape[-1]}] with unit stride")
     if h.dim() != 3 or tuple(y.shape) != tuple(h.shape) or y.dtype != h.dtype:
         raise ValueError("gated_residual expects h and y of identical [B,S,C] shape and dtype")
     B, S, Cdim = h.shape
@@ -321,7 +343,7 @@ def gated_residual(
         raise ValueError("out must match h in shape and dtype with a contiguous last axis")
     lib = _lib.load()
     rc = lib.odit_gated_residual(
-        h.data_ptr(), y.data_ptr(), _ptr(gate), out.data_ptr(), B, S, Cdim,
+        h.data_ptr(), y.data_ptr(), _ptr(gate), _ptr(gate_bias), out.data_ptr(), B, S, Cdim,
         _lib.i64_array(h.stride()[:2]), _lib.i64_array(y.stride()[:2]),
         _lib.i64_array(out.stride()[:2]), _lib.i64_array(gs), gate_dtype, _code(h),
         ODIT_FLAG_REF_ROUNDING if ref_rounding else 0, _stream(),
