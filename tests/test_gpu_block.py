@@ -46,7 +46,13 @@ def _inputs(B, seed=1, dtype=torch.bfloat16):
     return lat, txt, t
 
 
-def test_tiny_model_per_block_parity(gpu):
+@pytest.mark.parametrize("fuse_min_rows", [0, 1024])
+def test_tiny_model_per_block_parity(gpu, monkeypatch, fuse_min_rows):
+    """``fuse_min_rows`` = 0: every gated projection is one GEMM per batch entry with the gate and the
+    residual in its epilogue; 1024: at this size all of them run as one GEMM plus the gated-residual kernel."""
+    from vllm_omni_amd.blocks import qwen_image
+
+    monkeypatch.setattr(qwen_image, "FUSE_MIN_ROWS", fuse_min_rows)
     cfg, w, model = _build(gpu)
     lat, txt, t = _inputs(2)
     w32 = {k: v.float() for k, v in w.items()}

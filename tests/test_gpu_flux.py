@@ -49,8 +49,12 @@ def _inputs(cfg, B, grid=(8, 8), n_txt=16, seed=1, dtype=torch.bfloat16):
     return lat, txt, pooled, t, guidance, ofx.latent_image_ids(*grid), torch.zeros(n_txt, 3)
 
 
+@pytest.mark.parametrize("fuse_min_rows", [0, 1024])
 @pytest.mark.parametrize("grid,n_txt,B", [((8, 8), 16, 2), ((8, 11), 13, 1)])
-def test_tiny_flux_per_block_parity(gpu, grid, n_txt, B):
+def test_tiny_flux_per_block_parity(gpu, monkeypatch, grid, n_txt, B, fuse_min_rows):
+    from vllm_omni_amd.blocks import qwen_image
+
+    monkeypatch.setattr(qwen_image, "FUSE_MIN_ROWS", fuse_min_rows)  # 0: gated epilogues also at this size
     cfg, w, model = _build(gpu)
     lat, txt, pooled, t, gd, img_ids, txt_ids = _inputs(cfg, B, grid, n_txt)
     w32 = {k: v.float() for k, v in w.items()}

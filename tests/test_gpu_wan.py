@@ -32,8 +32,12 @@ def _model(gpu, cfg, w_lp, dtype=torch.bfloat16):
     return model
 
 
+@pytest.mark.parametrize("fuse_min_rows", [0, 1024])
 @pytest.mark.parametrize("fhw,n_txt,B", [((3, 10, 14), 13, 2), ((1, 16, 16), 32, 1)])
-def test_tiny_wan_per_block_parity(gpu, fhw, n_txt, B):
+def test_tiny_wan_per_block_parity(gpu, monkeypatch, fhw, n_txt, B, fuse_min_rows):
+    from vllm_omni_amd.blocks import qwen_image
+
+    monkeypatch.setattr(qwen_image, "FUSE_MIN_ROWS", fuse_min_rows)  # 0: gated epilogues also at this size
     cfg = ow.tiny_config()
     w32 = ow.init_params(cfg, seed=0, bias_std=0.02, norm_jitter=0.1)
     w = {k: v.bfloat16() for k, v in w32.items()}
