@@ -78,6 +78,24 @@ def test_tiny_model_per_block_parity(gpu, monkeypatch, fuse_min_rows):
     assert torch.equal(out2, out)
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float16, 4e-3), (torch.float32, 2e-4)])
+def test_tiny_model_fp16_and_fp32(gpu, dtype, tol):
+    """fp16 runs the same kernels as bf16 (with the +-65504 clip of qit.py:809-812 live); fp32 activations
+    bypass the flash backend for torch SDPA like the reference's Attention layer does
+    (attention/layer.py:127-132) and use the fp32 instantiations of the other kernels."""
+    cfg, w, model = _build(gpu, dtype=dtype)
+    model.fuse_modulation()
+    lat, txt, t = _inputs(2, seed=31, dtype=dtype)
+    w32 = {k: v.float() for k, v in w.items()}
+    want = oq.transformer_forward(w32, cfg, lat.float(), txt.float(), t.float(), IMG_SHAPE)
+    with torch.inference_mode():
+        got = model(lat.to(gpu), txt.to(gpu), None, t.to(gpu), [IMG_SHAPE], [S_TXT]).sample
+    assert got.dtype == dtype
+    err = (got.float().cpu() - want).abs().max().item()
+    print(f"{dtype}: max-abs {err:.2e} cosine {_cosine(got, want):.7f}", flush=True)
+    assert err <= tol and _cosine(got, want) >= 0.99999
+
+
 @pytest.mark.parametrize("fuse", [False, True])
 def test_editing_variant_per_token_conditioning(gpu, fuse):
     """zero_cond_t: doubled timestep, per-token choice between the two conditioning rows in both norms
