@@ -94,6 +94,24 @@ class AttnTimer:
         return sum(ms) / len(ms), top, len(ms)
 
 
+def max_engine_clock_mhz():
+    """Highest 'Max Clock Freq. (MHz)' that rocminfo lists for a GPU agent, or None when it cannot be read."""
+    import re
+    import subprocess
+
+    try:
+        text = subprocess.run(["rocminfo"], capture_output=True, text=True, timeout=30).stdout
+    except (OSError, subprocess.SubprocessError):
+        return None
+    best = None
+    for agent in text.split("*******")[1:]:
+        if "Device Type:             GPU" in agent or re.search(r"Device Type:\s+GPU", agent):
+            m = re.search(r"Max Clock Freq\. \(MHz\):\s+(\d+)", agent)
+            if m:
+                best = max(best or 0, int(m.group(1)))
+    return float(best) if best else None
+
+
 def build_model(torch, layers, fuse_epilogues=True):
     from vllm_omni_amd.blocks.qwen_image import QwenImageTransformer2DModel
 
@@ -506,6 +524,15 @@ def main():
             result["mfma_ceiling"] = mfma_ceiling(torch)
             result["roofline"]["frac_of_measured_mfma_ceiling_random_data"] = (
                 attn_tflops / result["mfma_ceiling"]["random_operands"]["TFLOP/s"])
+    props = torch.cuda.get_device_properties(0)
+    mhz = max_engine_clock_mhz()
+    result["device"] = {
+        "name": props.name, "gcn_arch": getattr(props, "gcnArchName", None), "compute_units": props.multi_processor_count,
+        "max_engine_clock_MHz": mhz, "hbm_GiB": props.total_memory / 2 ** 30,
+        # 4 SIMDs x one 32x32x16 bf16 MFMA (32768 FLOP) per 32 cycles = 4096 FLOP per clock per CU
+        "bf16_mfma_peak_from_clock_TFLOP/s": (props.multi_processor_count * mhz * 1e6 * 4096 / 1e12) if mhz else None,
+        "peaks_used": {"bf16_mfma_TFLOP/s": PEAK_MFMA_BF16_TFLOPS, "hbm_GB/s": PEAK_HBM_GBS},
+    }
     del model
     torch.cuda.empty_cache()
     if not args.no_cpu:
