@@ -24,10 +24,11 @@ if ROOT not in sys.path:
 
 PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, vendor figure
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E, vendor figure
-# HBM bytes of one attention launch at the headline shape, from rocprofv3 FETCH_SIZE / WRITE_SIZE passes
+# HBM bytes of one attention call at the headline shape, from rocprofv3 FETCH_SIZE / WRITE_SIZE passes
 # over `bench.py --traffic-probe`, each scaled by what the same counter reads for a 512 MiB copy
-# (FETCH_SIZE x2.0, WRITE_SIZE x1.0): 228.0 MB fetched + 53.5 MB written.
-ATTN_TRAFFIC_BYTES = 281.5e6
+# (FETCH_SIZE x2.0, WRITE_SIZE x1.0). One call = three launches: the full units (203.7 MB fetched + 51.9 MB
+# written), the key ranges of the last round (74.0 + 36.4 MB) and their merge (33.5 + 3.1 MB).
+ATTN_TRAFFIC_BYTES = 402.6e6
 
 # Qwen-Image shape at 1024x1024 (BASELINE.json configs[2])
 LAYERS, HEADS, HEAD_DIM, MLP_RATIO = 60, 24, 128, 4
@@ -508,7 +509,8 @@ def main():
                    "valid": args.blocks == LAYERS, "gemm": "hipBLASLt via torch" + (" (tuned solution table)" if tuned else "") +
                            ("; GELU and gated residuals as separate kernels" if args.unfused_epilogues else
                             "; GELU and gated residuals in the GEMM epilogues (odit_linear)")},
-        "roofline": {"kernel": "attn_fwd_kernel (joint attention, B=2, 24x128, S=4352)", "bound": "mfma",
+        "roofline": {"kernel": "attn_fwd_dma_kernel (joint attention, B=2, 24x128, S=4352; one call = the full units + "
+                               "the key-split last round + its merge, timed together)", "bound": "mfma",
                      "achieved": attn_tflops, "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": attn_tflops / PEAK_MFMA_BF16_TFLOPS,
                      "traffic": ATTN_TRAFFIC_BYTES if args.blocks == LAYERS else None,

@@ -436,13 +436,14 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const AttnParams p, int
 }
 
 // How the last round of workgroups is cut along the keys. `slots` workgroups run at once; after
-// `units / slots` full rounds, `rem` units are left: when they would occupy at most an eighth of the
+// `units / slots` full rounds, `rem` units are left: when they would occupy at most a quarter of the
 // slots, each is cut into as many key ranges as fit the slots (ranges of an even number of tiles, at
 // least kMinTilesPerChunk), so the tail takes 1/key_chunks of a round instead of most of one. Measured
-// at rem = 96 of 512 slots (the 4352-token, 48-head shape): the unsplit tail costs 0.7 of a round, the
-// split one 0.2 of a round plus two more launches and 130 MB of partial results - no gain, hence the
-// threshold. (Running the key ranges on a side stream, concurrently with the full units, was measured
-// too: no gain either.)
+// side by side in one process at rem = 96 of 512 slots (the 4352-token, 48-head shape): the unsplit tail
+// costs 0.5 of a round (its workgroups have their CUs to themselves), the split one 0.2 of a round plus
+// two more launches and the partial results: 471 -> 454 us. At rem = 256 (half the slots, two ranges)
+// the split loses, 227 -> 242 us; twice as many, shorter ranges lose as well. Running the key ranges on
+// a side stream, concurrently with the full units, gave nothing over the same-stream order.
 struct TailPlan { int rem, key_chunks, tiles_per_chunk; };
 constexpr int kMinTilesPerChunk = 8;
 constexpr int kMaxKeyChunks = 16;
@@ -459,10 +460,14 @@ static int device_slots(int nw) {
   return cus[dev] * (8 / nw);
 }
 
+#ifndef ODIT_ATTN_TAIL_DIV
+#define ODIT_ATTN_TAIL_DIV 4   // split the last round's units by keys when they fill at most 1/4 of the GPU
+#endif
+
 static TailPlan plan_tail(int64_t units, int n_tiles, int slots) {
   TailPlan t{0, 1, n_tiles};
   const int rem = static_cast<int>(units % slots);
-  if (rem == 0 || 8 * rem > slots) return t;
+  if (rem == 0 || ODIT_ATTN_TAIL_DIV * rem > slots) return t;
   int kc = slots / rem;
   if (kc > kMaxKeyChunks) kc = kMaxKeyChunks;
   if (kc > n_tiles / kMinTilesPerChunk) kc = n_tiles / kMinTilesPerChunk;
