@@ -120,6 +120,40 @@ def test_headline_shape_block_against_oracle(gpu):
         assert (want - (img if name == "img" else txt).float()).abs().max().item() > 20 * err  # the block did something
 
 
+def test_forward_under_hip_graph_capture(gpu):
+    """The whole forward can be recorded in a HIP graph (no host synchronisation, no allocation outside
+    torch's capture pool, no memset nodes on the path): several replays on new inputs, with eager work
+    and synchronisations in between, each give the eager result bit for bit."""
+    cfg, w, model = _build(gpu)
+    model.fuse_modulation()
+    lat, txt, t = _inputs(2, seed=41)
+    lat_g, txt_g, t_g = lat.to(gpu), txt.to(gpu), t.to(gpu)
+
+    def fwd():
+        return model(lat_g, txt_g, None, t_g, [IMG_SHAPE], [S_TXT]).sample
+
+    with torch.inference_mode():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):     # warm-up on the side stream: workspaces and plans exist before capture
+            for _ in range(2):
+                fwd()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = fwd()
+        for seed in (42, 43, 44):
+            new_lat, _, new_t = _inputs(2, seed=seed)
+            lat_g.copy_(new_lat.to(gpu))
+            t_g.copy_(new_t.to(gpu))
+            graph.replay()
+            torch.cuda.synchronize()
+            got = out.clone()
+            want = fwd()
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), f"replay with seed {seed} differs from eager"
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float16, 4e-3), (torch.float32, 2e-4)])
 def test_tiny_model_fp16_and_fp32(gpu, dtype, tol):
     """fp16 runs the same kernels as bf16 (with the +-65504 clip of qit.py:809-812 live); fp32 activations
