@@ -168,3 +168,56 @@ def test_flux_teacache_decisions_match_oracle(gpu):
     err = (got_lat.float().cpu() - want_lat.float()).abs().max().item()
     print(f"final latents max-abs diff vs bf16 oracle: {err:.4f}", flush=True)
     assert err < 0.25
+
+
+def test_flux_width_blocks_against_oracle(gpu):
+    """One dual and one single block at the Flux width and sequence (hidden 3072 = 24 heads x 128, 512 text +
+    4096 image tokens, batch 1) against the fp32 oracle: the launches of the Flux-shape benchmark (fused
+    epilogues, the two accumulating GEMMs of the single block's proj_out, attention on 4608 keys)."""
+    from vllm_omni_amd.attention.selector import get_attn_backend
+    from vllm_omni_amd.blocks.flux import FluxSingleTransformerBlock, FluxTransformerBlock
+
+    get_attn_backend.cache_clear()
+    cfg = ofx.FluxConfig(num_layers=1, num_single_layers=1)
+    g = torch.Generator().manual_seed(23)
+
+    def params(shapes, prefix):
+        out = {}
+        for n, shape in shapes.items():
+            if n.endswith(("norm_q.weight", "norm_k.weight", "norm_added_q.weight", "norm_added_k.weight")):
+                t = 1 + 0.1 * torch.randn(shape, generator=g)
+            else:
+                t = 0.02 * torch.randn(shape, generator=g)
+            out[prefix + n] = t.bfloat16()
+        return out
+
+    w = {**params(ofx.dual_block_param_shapes(cfg), "transformer_blocks.0."),
+         **params(ofx.single_block_param_shapes(cfg), "single_transformer_blocks.0.")}
+    dual = FluxTransformerBlock(cfg.dim, cfg.num_heads, cfg.head_dim).to(gpu).bfloat16()
+    single = FluxSingleTransformerBlock(cfg.dim, cfg.num_heads, cfg.head_dim).to(gpu).bfloat16()
+    with torch.no_grad():
+        for blk, prefix in ((dual, "transformer_blocks.0."), (single, "single_transformer_blocks.0.")):
+            for k, p in blk.named_parameters():
+                p.copy_(w[prefix + k].to(gpu))
+    S_img, S_txt = 4096, 512
+    img = torch.randn(1, S_img, cfg.dim, generator=g).bfloat16()
+    txt = torch.randn(1, S_txt, cfg.dim, generator=g).bfloat16()
+    temb = (0.5 * torch.randn(1, cfg.dim, generator=g)).bfloat16()
+    cos, sin = ofx.flux_pos_embed(cfg, torch.cat([torch.zeros(S_txt, 3), ofx.latent_image_ids(64, 64)], dim=0))
+    wf = {k: v.float() for k, v in w.items()}
+    t1, i1 = ofx.dual_block_forward(wf, 0, cfg, img.float(), txt.float(), temb.float(), cos, sin)
+    t2, i2 = ofx.single_block_forward(wf, 0, cfg, i1, t1, temb.float(), cos, sin)
+    rot = (cos.to(gpu), sin.to(gpu))
+    with torch.inference_mode():
+        gt1, gi1 = dual(hidden_states=img.to(gpu), encoder_hidden_states=txt.to(gpu), temb=temb.to(gpu),
+                        image_rotary_emb=rot)
+        # the single block is checked on the oracle's (rounded) input so that the two errors do not add
+        gt2, gi2 = single(hidden_states=i1.bfloat16().to(gpu), encoder_hidden_states=t1.bfloat16().to(gpu),
+                          temb=temb.to(gpu), image_rotary_emb=rot)
+    t2r, i2r = ofx.single_block_forward(wf, 0, cfg, i1.bfloat16().float(), t1.bfloat16().float(), temb.float(), cos, sin)
+    for name, got, want in (("dual img", gi1, i1), ("dual txt", gt1, t1), ("single img", gi2, i2r), ("single txt", gt2, t2r)):
+        a, b = got.flatten().cpu().double(), want.flatten().double()
+        err, mag = (a - b).abs().max().item(), b.abs().max().item()
+        cos_ab = float(torch.dot(a, b) / (a.norm() * b.norm()))
+        print(f"flux-width {name}: max-abs {err:.4f} cosine {cos_ab:.6f} (|x| max {mag:.2f})", flush=True)
+        assert err <= 2e-2 * max(1.0, mag / 2) and cos_ab >= 0.9995
