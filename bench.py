@@ -314,7 +314,13 @@ def kernel_rooflines(torch):
     w = torch.ones(HEAD_DIM, device=dev, dtype=bf)
     cos = torch.rand(S_IMG, HEAD_DIM // 2, device=dev)
     sin = torch.rand(S_IMG, HEAD_DIM // 2, device=dev)
+    # as in the step: q and k are normalised, rotated and written to the joint buffers; v stays where the
+    # projection left it (the attention kernel reads it there), so it is no traffic of this kernel
     bw("qknorm_rope",
+       [lambda i=i: kernels.qknorm_rope(qkvs[i][:, :, 0], qkvs[i][:, :, 1], None, jqs[i][0], jqs[i][1],
+                                        None, w, w, cos, sin, out_seq_offset=S_TXT, norm_mode=ODIT_NORM_HEAD)
+        for i in range(NSET)], 2 * (2 * qkvs[0].numel() // 3) * 2)
+    bw("qknorm_rope_with_v_copy",
        [lambda i=i: kernels.qknorm_rope(qkvs[i][:, :, 0], qkvs[i][:, :, 1], qkvs[i][:, :, 2], jqs[i][0], jqs[i][1],
                                         jqs[i][2], w, w, cos, sin, out_seq_offset=S_TXT, norm_mode=ODIT_NORM_HEAD)
         for i in range(NSET)], 2 * qkvs[0].numel() * 2)

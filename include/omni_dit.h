@@ -73,7 +73,14 @@ int odit_attn_fwd(const void* q, const void* k, const void* v, void* o, const ui
                   const int64_t v_strides[3], const int64_t o_strides[3], float scale, int dtype,
                   void* stream);
 
-/* Extended form of odit_attn_fwd with two optional additions.
+/* Extended form of odit_attn_fwd with three optional additions.
+ *
+ * Values in two tensors: with v_tail != NULL, key rows [0, k_split) take their values from `v` and rows
+ * [k_split, Sk) from `v_tail` (row r -> v_tail row r - k_split); k_split is a multiple of 64, both share
+ * the row stride (v_tail_strides[1] == v_strides[1]), batch and head strides are their own. Lets the
+ * joint attention read V straight out of the two fused-QKV projection outputs: the value halves of
+ * torch.cat([txt_value, img_value]) (qwen_image_transformer.py:603-606, flux_transformer.py:200-208)
+ * are never copied. Keys still come as one tensor (they are rewritten by norm + rotary anyway).
  *
  * Two outputs: with o_tail != NULL, query rows [0, q_split) are written to `o` (row r -> o row r) and
  * rows [q_split, Sq) to `o_tail` (row r -> o_tail row r - q_split), each with its own (batch, seq,
@@ -84,18 +91,19 @@ int odit_attn_fwd(const void* q, const void* k, const void* v, void* o, const ui
  * Scratch: `workspace` (device memory, 16-byte aligned, workspace_bytes >=
  * odit_attn_fwd_workspace_bytes for the same shape, contents irrelevant before and after) lets the
  * kernel cut the last, partly filled round of workgroups into key ranges that run side by side and
- * are merged by a second launch; it is used when that last round would fill at most an eighth of the
- * GPU (few heads x query blocks, many keys), where the unsplit launch leaves most of the GPU idle. NULL = never split. Results with and
+ * are merged by a second launch; it is used when that last round would fill at most a quarter of the
+ * GPU, where the unsplit launch leaves most of the GPU idle. NULL = never split. Results with and
  * without scratch agree to rounding (the merge re-associates the key sum); for given shapes and device
  * the partition is fixed, so repeated calls are bit-identical. No counterpart in the reference.
  *
- * o_tail == NULL and workspace == NULL behaves exactly like odit_attn_fwd.
+ * v_tail == NULL, o_tail == NULL and workspace == NULL behaves exactly like odit_attn_fwd.
  */
-int odit_attn_fwd_ex(const void* q, const void* k, const void* v, void* o, void* o_tail, int q_split,
-                     const uint8_t* key_mask, float* lse, int B, int Sq, int Sk, int H, int Hkv, int D,
-                     const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
-                     const int64_t o_strides[3], const int64_t o_tail_strides[3], float scale, int dtype,
-                     void* workspace, size_t workspace_bytes, void* stream);
+int odit_attn_fwd_ex(const void* q, const void* k, const void* v, const void* v_tail, int k_split, void* o,
+                     void* o_tail, int q_split, const uint8_t* key_mask, float* lse, int B, int Sq, int Sk,
+                     int H, int Hkv, int D, const int64_t q_strides[3], const int64_t k_strides[3],
+                     const int64_t v_strides[3], const int64_t v_tail_strides[3], const int64_t o_strides[3],
+                     const int64_t o_tail_strides[3], float scale, int dtype, void* workspace,
+                     size_t workspace_bytes, void* stream);
 
 /* Scratch bytes odit_attn_fwd_ex can use for this shape on the current device (0 = none needed). */
 size_t odit_attn_fwd_workspace_bytes(int B, int Sq, int Sk, int H, int D);

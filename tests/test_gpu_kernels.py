@@ -467,6 +467,40 @@ def test_attention_key_split_tail(gpu, monkeypatch, variant, shape):
         assert torch.equal(head, two[:, :cut]) and torch.equal(tail, two[:, cut:])
 
 
+@pytest.mark.parametrize("variant", ["34", "38", "28"])
+@pytest.mark.parametrize("shape,cut", [((2, 300, 300, 4, 4, 128), 64), ((1, 1100, 1100, 3, 3, 64), 256),
+                                       ((2, 130, 2048, 4, 2, 128), 1024), ((1, 300, 1100, 3, 3, 128), 192),
+                                       ((2, 200, 200, 2, 2, 128), 70)])
+def test_attention_values_in_two_tensors(gpu, monkeypatch, variant, shape, cut):
+    """Value rows of keys [0, cut) and [cut, Sk) taken from two tensors (strided views of two wider
+    buffers, like the value thirds of two fused-QKV outputs) give the result of the concatenated tensor bit
+    for bit: plain, masked, with two outputs, and on launches that split their last round by keys. A cut
+    that is not a multiple of 64 (last case) or a kernel variant without the feature ("28") goes through
+    a concatenation inside the wrapper."""
+    from vllm_omni_amd import kernels
+
+    monkeypatch.setenv("ODIT_ATTN_VARIANT", variant)
+    B, Sq, Sk, H, Hkv, D = shape
+    q, k, v = _attn_inputs(B, Sq, Sk, H, Hkv, D, seed=11)
+    scale = 1.0 / math.sqrt(D)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    wide_a = torch.zeros(B, cut, 3, Hkv, D, dtype=v.dtype, device=gpu)
+    wide_b = torch.zeros(B, Sk - cut, 3, Hkv, D, dtype=v.dtype, device=gpu)
+    wide_a[:, :, 2], wide_b[:, :, 2] = vg[:, :cut], vg[:, cut:]
+    pair = (wide_a[:, :, 2], wide_b[:, :, 2])
+    want = kernels.attn_fwd(qg, kg, vg, scale)
+    assert torch.equal(kernels.attn_fwd(qg, kg, pair, scale), want)
+    m = torch.rand(B, Sk, generator=torch.Generator().manual_seed(12)) > 0.3
+    m[:, -1] = True
+    assert torch.equal(kernels.attn_fwd(qg, kg, pair, scale, key_mask=m.to(gpu)),
+                       kernels.attn_fwd(qg, kg, vg, scale, key_mask=m.to(gpu)))
+    head, tail = kernels.attn_fwd(qg, kg, pair, scale, split=Sq // 3)
+    assert torch.equal(head, want[:, :Sq // 3]) and torch.equal(tail, want[:, Sq // 3:])
+    _close(want, ops.sdpa(q.float(), k.float(), v.float(), scale), atol=2e-2, rtol=2e-2, what="attention vs oracle")
+    with pytest.raises(ValueError, match="does not cover"):
+        kernels.attn_fwd(qg, kg, (pair[0], pair[1][:, :-1]), scale)
+
+
 def test_attention_workspace_too_small_is_an_error(gpu):
     from vllm_omni_amd import _lib
 
@@ -478,14 +512,22 @@ def test_attention_workspace_too_small_is_an_error(gpu):
     o = torch.empty_like(q)
     ws = torch.empty(need, device=gpu, dtype=torch.uint8)
     st = _lib.i64_array(q.stride()[:3])
-    rc = lib.odit_attn_fwd_ex(q.data_ptr(), q.data_ptr(), q.data_ptr(), o.data_ptr(), None, 0, None, None,
-                              B, Sq, Sk if False else Sq, H, H, D, st, st, st, st, None, 0.1, 0, ws.data_ptr(), 16, None)
+    rc = lib.odit_attn_fwd_ex(q.data_ptr(), q.data_ptr(), q.data_ptr(), None, 0, o.data_ptr(), None, 0, None, None,
+                              B, Sq, Sq, H, H, D, st, st, st, None, st, None, 0.1, 0, ws.data_ptr(), 16, None)
     assert rc == 0  # Sk = 128: nothing to split, any workspace size is fine
     k = torch.zeros(B, Sk, H, D, device=gpu, dtype=torch.bfloat16)
     sk = _lib.i64_array(k.stride()[:3])
-    rc = lib.odit_attn_fwd_ex(q.data_ptr(), k.data_ptr(), k.data_ptr(), o.data_ptr(), None, 0, None, None,
-                              B, Sq, Sk, H, H, D, st, sk, sk, st, None, 0.1, 0, ws.data_ptr(), need - 1, None)
+    rc = lib.odit_attn_fwd_ex(q.data_ptr(), k.data_ptr(), k.data_ptr(), None, 0, o.data_ptr(), None, 0, None, None,
+                              B, Sq, Sk, H, H, D, st, sk, sk, None, st, None, 0.1, 0, ws.data_ptr(), need - 1, None)
     assert rc == -4 and b"workspace" in lib.odit_last_error()
+    # values in two tensors: the cut must be a whole number of 64-key tiles, the row strides equal
+    rc = lib.odit_attn_fwd_ex(q.data_ptr(), k.data_ptr(), k.data_ptr(), k.data_ptr(), 100, o.data_ptr(), None, 0, None,
+                              None, B, Sq, Sk, H, H, D, st, sk, sk, sk, st, None, 0.1, 0, None, 0, None)
+    assert rc == -1 and b"multiple of 64" in lib.odit_last_error()
+    bad = _lib.i64_array((k.stride(0), 2 * k.stride(1), k.stride(2)))
+    rc = lib.odit_attn_fwd_ex(q.data_ptr(), k.data_ptr(), k.data_ptr(), k.data_ptr(), 64, o.data_ptr(), None, 0, None,
+                              None, B, Sq, Sk, H, H, D, st, sk, sk, bad, st, None, 0.1, 0, None, 0, None)
+    assert rc == -1 and b"row stride" in lib.odit_last_error()
     torch.cuda.synchronize()
 
 

@@ -34,9 +34,9 @@ _SIGNATURES = {
     ),
     "odit_attn_fwd_ex": (
         C.c_int,
-        [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p,
-         C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
-         _i64p, _i64p, _i64p, _i64p, _i64p, C.c_float, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p],
+        [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int,
+         C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
+         _i64p, _i64p, _i64p, _i64p, _i64p, _i64p, C.c_float, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p],
     ),
     "odit_attn_fwd_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
     "odit_qknorm_rope": (

@@ -52,7 +52,10 @@ class AttentionMetadata:
     """Per-call extras (abstract.py:54-66). ``attn_mask`` is a [B,Sk] key-padding mask; the joint_*
     fields carry a replicated text segment for sequence-parallel strategies and are unused on one GPU.
     ``output_split`` (not in the reference) asks the backend for two dense outputs, rows [0, s) and
-    [s, Sq) of the joint sequence, instead of one tensor the caller would slice and copy."""
+    [s, Sq) of the joint sequence, instead of one tensor the caller would slice and copy.
+    ``value_tail`` (not in the reference): the ``value`` argument then holds only the rows of the first
+    keys and this tensor the rest, so a caller with the values of two streams in two buffers does not
+    have to concatenate them."""
 
     attn_mask: torch.Tensor | None = None
     joint_attn_mask: torch.Tensor | None = None
@@ -61,6 +64,7 @@ class AttentionMetadata:
     joint_value: torch.Tensor | None = None
     joint_strategy: str = "front"
     output_split: int | None = None
+    value_tail: torch.Tensor | None = None
 
 
 T = TypeVar("T", bound=AttentionMetadata)

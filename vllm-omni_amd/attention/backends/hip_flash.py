@@ -47,7 +47,8 @@ class HipFlashAttentionImpl(AttentionImpl):
                     attn_metadata: AttentionMetadata | None = None) -> torch.Tensor:
         """q [B,Sq,H,D], k/v [B,Sk,Hkv,D] -> [B,Sq,H,D]. A [B,Sk] ``attn_mask`` excludes keys; an
         all-true mask is dropped like the reference does (flash_attn.py:80-84). With
-        ``attn_metadata.output_split`` = s the result is the pair (out[:, :s], out[:, s:]), both dense."""
+        ``attn_metadata.output_split`` = s the result is the pair (out[:, :s], out[:, s:]), both dense;
+        with ``attn_metadata.value_tail`` the values are [value; value_tail] along the keys, read in place."""
         mask = attn_metadata.attn_mask if attn_metadata is not None else None
         if mask is not None:
             if mask.dim() != 2:
@@ -55,6 +56,9 @@ class HipFlashAttentionImpl(AttentionImpl):
             if bool(torch.all(mask != 0)):
                 mask = None
         split = attn_metadata.output_split if attn_metadata is not None else None
+        v_tail = attn_metadata.value_tail if attn_metadata is not None else None
+        if v_tail is not None:
+            value = (value, v_tail)
         return kernels.attn_fwd(query, key, value, self.softmax_scale, key_mask=mask, split=split)
 
     # the platform never routes here; kept so a direct call cannot silently pick another kernel

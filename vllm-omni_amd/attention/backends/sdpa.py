@@ -36,6 +36,8 @@ class SDPAImpl(AttentionImpl):
         self.softmax_scale = softmax_scale
 
     def forward_hip(self, query, key, value, attn_metadata: AttentionMetadata | None = None):
+        if attn_metadata is not None and attn_metadata.value_tail is not None:
+            value = torch.cat([value, attn_metadata.value_tail], dim=1)
         q, k, v = (t.transpose(1, 2) for t in (query, key, value))
         mask = attn_metadata.attn_mask if attn_metadata else None
         if mask is not None and mask.dim() == 2:  # [B,Sk] key padding -> broadcastable boolean

@@ -139,17 +139,23 @@ class FluxAttention(nn.Module):
         cqkv = self.add_kv_proj(encoder_hidden_states).view(B, S_c, 3, H, D)
         S = S_c + S_x
         jq = torch.empty((B, S, H, D), dtype=qkv.dtype, device=qkv.device)
-        jk, jv = torch.empty_like(jq), torch.empty_like(jq)
+        jk = torch.empty_like(jq)
+        # v is only moved, never changed: read in place from the two projections when the kernel can
+        v_in_place = S_c % 64 == 0 and qkv.dtype != torch.float32 and kernels.attn_reads_value_pairs() and not rr
+        jv = None if v_in_place else torch.empty_like(jq)
         tc = ts = ic = isn = None
         if rot is not None:
             tc, ts, ic, isn = rot.cos32[:S_c], rot.sin32[:S_c], rot.cos32[S_c:], rot.sin32[S_c:]
-        kernels.qknorm_rope(cqkv[:, :, 0], cqkv[:, :, 1], cqkv[:, :, 2], jq, jk, jv, self.norm_added_q.weight,
-                            self.norm_added_k.weight, tc, ts, eps=self.eps, out_seq_offset=0,
+        kernels.qknorm_rope(cqkv[:, :, 0], cqkv[:, :, 1], None if v_in_place else cqkv[:, :, 2], jq, jk, jv,
+                            self.norm_added_q.weight, self.norm_added_k.weight, tc, ts, eps=self.eps,
+                            out_seq_offset=0, norm_mode=ODIT_NORM_HEAD, ref_rounding=rr)
+        kernels.qknorm_rope(qkv[:, :, 0], qkv[:, :, 1], None if v_in_place else qkv[:, :, 2], jq, jk, jv,
+                            self.norm_q.weight, self.norm_k.weight, ic, isn, eps=self.eps, out_seq_offset=S_c,
                             norm_mode=ODIT_NORM_HEAD, ref_rounding=rr)
-        kernels.qknorm_rope(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], jq, jk, jv, self.norm_q.weight,
-                            self.norm_k.weight, ic, isn, eps=self.eps, out_seq_offset=S_c,
-                            norm_mode=ODIT_NORM_HEAD, ref_rounding=rr)
-        ctx_attn, x_attn = self.attn(jq, jk, jv, AttentionMetadata(output_split=S_c))
+        meta = AttentionMetadata(output_split=S_c)
+        if v_in_place:
+            jv, meta.value_tail = cqkv[:, :, 2], qkv[:, :, 2]
+        ctx_attn, x_attn = self.attn(jq, jk, jv, meta)
         if residuals is not None:
             res, gate, c_res, c_gate = residuals[:4]
             pre, c_pre = residuals[4:] if len(residuals) == 6 else (None, None)

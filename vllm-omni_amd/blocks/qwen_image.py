@@ -221,16 +221,22 @@ class QwenImageCrossAttention(nn.Module):
         S = S_txt + S_img
         jq = torch.empty((B, S, H, D), dtype=img_qkv.dtype, device=img_qkv.device)
         jk = torch.empty_like(jq)
-        jv = torch.empty_like(jq)
+        # q and k are rewritten by norm + rotary into the joint buffers; v is only moved, so when the
+        # attention kernel can read the two value halves where the projections left them it is not copied
+        v_in_place = (S_txt % 64 == 0 and img_qkv.dtype != torch.float32 and kernels.attn_reads_value_pairs()
+                      and not self.ref_rounding)
+        jv = None if v_in_place else torch.empty_like(jq)
         rr = self.ref_rounding
-        kernels.qknorm_rope(txt_qkv[:, :, 0], txt_qkv[:, :, 1], txt_qkv[:, :, 2], jq, jk, jv,
+        kernels.qknorm_rope(txt_qkv[:, :, 0], txt_qkv[:, :, 1], None if v_in_place else txt_qkv[:, :, 2], jq, jk, jv,
                             self.norm_added_q.weight, self.norm_added_k.weight, tables.txt_cos, tables.txt_sin,
                             eps=self.eps, out_seq_offset=0, norm_mode=ODIT_NORM_HEAD, ref_rounding=rr)
-        kernels.qknorm_rope(img_qkv[:, :, 0], img_qkv[:, :, 1], img_qkv[:, :, 2], jq, jk, jv,
+        kernels.qknorm_rope(img_qkv[:, :, 0], img_qkv[:, :, 1], None if v_in_place else img_qkv[:, :, 2], jq, jk, jv,
                             self.norm_q.weight, self.norm_k.weight, tables.img_cos, tables.img_sin,
                             eps=self.eps, out_seq_offset=S_txt, norm_mode=ODIT_NORM_HEAD, ref_rounding=rr)
         # the backend writes the text and image rows of the output to two dense tensors
         meta = AttentionMetadata(output_split=S_txt)
+        if v_in_place:
+            jv, meta.value_tail = txt_qkv[:, :, 2], img_qkv[:, :, 2]
         if hidden_states_mask is not None or encoder_hidden_states_mask is not None:
             ones = lambda n: torch.ones((B, n), dtype=torch.bool, device=jq.device)  # noqa: E731
             txt_m = encoder_hidden_states_mask if encoder_hidden_states_mask is not None else ones(S_txt)

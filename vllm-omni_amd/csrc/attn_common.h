@@ -47,6 +47,10 @@ struct AttnParams {
   // optional second output: query rows >= q_split are written to o_tail[row - q_split]
   void* o_tail; int q_split;
   int64_t ts_b, ts_s, ts_h;
+  // optional second value tensor: key rows >= k_split take their values from v_tail[row - k_split]
+  // (same row stride as v; only the software-pipelined kernel of attn_fwd_dma.hip reads it)
+  const void* v_tail; int k_split;
+  int64_t vt_b, vt_h;
   // key-split tail (attn_fwd_dma.hip): workgroup ids < n_full own a whole (q-block, head, batch) unit;
   // the remaining units are cut into key_chunks ranges of tiles_per_chunk key tiles each, one
   // workgroup per range, which leave unnormalised partial results in `ws` for the merge kernel

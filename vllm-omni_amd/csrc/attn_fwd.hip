@@ -620,20 +620,21 @@ static int attn_variant() {
   return variant;
 }
 
-extern "C" int odit_attn_fwd_ex(const void* q, const void* k, const void* v, void* o, void* o_tail,
-                                int q_split, const uint8_t* key_mask, float* lse, int B, int Sq, int Sk,
-                                int H, int Hkv, int D, const int64_t q_strides[3],
+extern "C" int odit_attn_fwd_ex(const void* q, const void* k, const void* v, const void* v_tail, int k_split,
+                                void* o, void* o_tail, int q_split, const uint8_t* key_mask, float* lse,
+                                int B, int Sq, int Sk, int H, int Hkv, int D, const int64_t q_strides[3],
                                 const int64_t k_strides[3], const int64_t v_strides[3],
-                                const int64_t o_strides[3], const int64_t o_tail_strides[3], float scale,
-                                int dtype, void* workspace, size_t workspace_bytes, void* stream);
+                                const int64_t v_tail_strides[3], const int64_t o_strides[3],
+                                const int64_t o_tail_strides[3], float scale, int dtype, void* workspace,
+                                size_t workspace_bytes, void* stream);
 
 extern "C" int odit_attn_fwd(const void* q, const void* k, const void* v, void* o,
                              const uint8_t* key_mask, float* lse, int B, int Sq, int Sk, int H,
                              int Hkv, int D, const int64_t q_strides[3], const int64_t k_strides[3],
                              const int64_t v_strides[3], const int64_t o_strides[3], float scale,
                              int dtype, void* stream) {
-  return odit_attn_fwd_ex(q, k, v, o, nullptr, 0, key_mask, lse, B, Sq, Sk, H, Hkv, D, q_strides, k_strides,
-                          v_strides, o_strides, nullptr, scale, dtype, nullptr, 0, stream);
+  return odit_attn_fwd_ex(q, k, v, nullptr, 0, o, nullptr, 0, key_mask, lse, B, Sq, Sk, H, Hkv, D, q_strides,
+                          k_strides, v_strides, nullptr, o_strides, nullptr, scale, dtype, nullptr, 0, stream);
 }
 
 extern "C" size_t odit_attn_fwd_workspace_bytes(int B, int Sq, int Sk, int H, int D) {
@@ -643,12 +644,13 @@ extern "C" size_t odit_attn_fwd_workspace_bytes(int B, int Sq, int Sk, int H, in
   return odit::attn_dma_workspace_bytes(B, Sq, Sk, H, D, variant == 38 ? 8 : 4);
 }
 
-extern "C" int odit_attn_fwd_ex(const void* q, const void* k, const void* v, void* o, void* o_tail,
-                                int q_split, const uint8_t* key_mask, float* lse, int B, int Sq, int Sk,
-                                int H, int Hkv, int D, const int64_t q_strides[3],
+extern "C" int odit_attn_fwd_ex(const void* q, const void* k, const void* v, const void* v_tail, int k_split,
+                                void* o, void* o_tail, int q_split, const uint8_t* key_mask, float* lse,
+                                int B, int Sq, int Sk, int H, int Hkv, int D, const int64_t q_strides[3],
                                 const int64_t k_strides[3], const int64_t v_strides[3],
-                                const int64_t o_strides[3], const int64_t o_tail_strides[3], float scale,
-                                int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+                                const int64_t v_tail_strides[3], const int64_t o_strides[3],
+                                const int64_t o_tail_strides[3], float scale, int dtype, void* workspace,
+                                size_t workspace_bytes, void* stream) {
   using namespace odit;
   if (o_tail != nullptr) {
     ODIT_CHECK_ARG(o_tail_strides != nullptr, "odit_attn_fwd_ex: o_tail given without strides");
@@ -656,6 +658,16 @@ extern "C" int odit_attn_fwd_ex(const void* q, const void* k, const void* v, voi
     ODIT_CHECK_ARG(aligned16(o_tail) && o_tail_strides[0] % 8 == 0 && o_tail_strides[1] % 8 == 0 &&
                        o_tail_strides[2] % 8 == 0,
                    "odit_attn_fwd_ex: o_tail must be 16-byte aligned with strides multiple of 8");
+  }
+  if (v_tail != nullptr) {
+    ODIT_CHECK_ARG(v_tail_strides != nullptr && v_strides != nullptr, "odit_attn_fwd_ex: v_tail given without strides");
+    ODIT_CHECK_ARG(k_split > 0 && k_split < Sk && k_split % 64 == 0,
+                   "odit_attn_fwd_ex: k_split=%d must be a multiple of 64 inside (0, Sk=%d)", k_split, Sk);
+    ODIT_CHECK_ARG(v_tail_strides[1] == v_strides[1],
+                   "odit_attn_fwd_ex: v and v_tail must share the row stride (%lld vs %lld)",
+                   static_cast<long long>(v_strides[1]), static_cast<long long>(v_tail_strides[1]));
+    ODIT_CHECK_ARG(aligned16(v_tail) && v_tail_strides[0] % 8 == 0 && v_tail_strides[2] % 8 == 0,
+                   "odit_attn_fwd_ex: v_tail must be 16-byte aligned with strides multiple of 8");
   }
   ODIT_CHECK_ARG(q && k && v && o, "odit_attn_fwd: q/k/v/o must not be null");
   ODIT_CHECK_ARG(q_strides && k_strides && v_strides && o_strides, "odit_attn_fwd: null strides");
@@ -692,6 +704,9 @@ extern "C" int odit_attn_fwd_ex(const void* q, const void* k, const void* v, voi
   p.o_tail = o_tail; p.q_split = q_split;
   p.ts_b = o_tail ? o_tail_strides[0] : 0; p.ts_s = o_tail ? o_tail_strides[1] : 0; p.ts_h = o_tail ? o_tail_strides[2] : 0;
 
+  p.v_tail = v_tail; p.k_split = v_tail ? k_split : 0;
+  p.vt_b = v_tail ? v_tail_strides[0] : 0; p.vt_h = v_tail ? v_tail_strides[2] : 0;
+
   p.n_full = 0; p.key_chunks = 1; p.tiles_per_chunk = 0; p.ws = nullptr;
 
   int variant = attn_variant();
@@ -700,6 +715,11 @@ extern "C" int odit_attn_fwd_ex(const void* q, const void* k, const void* v, voi
     const int rc = launch_attn_dma(p, dtype, D, variant == 38 ? 8 : 4, st, workspace, workspace_bytes);
     if (rc != ODIT_ENOTSUP) return rc;
     variant = 28;  // tensors too large for 32-bit buffer offsets: pointer-addressed kernel
+  }
+  if (v_tail != nullptr) {
+    set_error("odit_attn_fwd_ex: values in two tensors need the buffer-addressed kernel (default variant, "
+              "key/value spans below 2 GiB per batch and head)");
+    return ODIT_ENOTSUP;
   }
   if (dtype == ODIT_BF16) {
     return D == 128 ? dispatch_attn<bf16_t, 128>(p, variant, st)

@@ -87,7 +87,11 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
 
   // buffer descriptors end right after the last valid key row: later rows read as zeros
   const uint32_t k_bytes = static_cast<uint32_t>(((p.Sk - 1) * p.ks_s + D) * 2);
-  const uint32_t v_bytes = static_cast<uint32_t>(((p.Sk - 1) * p.vs_s + D) * 2);
+  // value rows [0, k_split) come from v, rows [k_split, Sk) from v_tail (k_split is a whole number of
+  // tiles and both share the row stride): two descriptors, picked per tile with scalar selects
+  const int v_split_tiles = p.v_tail != nullptr ? p.k_split / BN : n_tiles_all;
+  const int v_rows = p.v_tail != nullptr ? p.k_split : p.Sk;
+  const uint32_t v_bytes = static_cast<uint32_t>(((v_rows - 1) * p.vs_s + D) * 2);
   // raw buffer descriptors {base[31:0], base[47:32] (stride 0), bytes, dword3 = 0x00020000}
   auto make_rsrc = [](const void* base, uint32_t bytes) {
     const uint64_t a = reinterpret_cast<uint64_t>(base);
@@ -97,6 +101,11 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   };
   const u32x4_v krsrc = make_rsrc(kbase, k_bytes);
   const u32x4_v vrsrc = make_rsrc(vbase, v_bytes);
+  u32x4_v vrsrc2 = vrsrc;
+  if (p.v_tail != nullptr) {
+    const T* vbase2 = static_cast<const T*>(p.v_tail) + b * p.vt_b + hkv * p.vt_h;
+    vrsrc2 = make_rsrc(vbase2, static_cast<uint32_t>(((p.Sk - p.k_split - 1) * p.vs_s + D) * 2));
+  }
 
   // per-lane global byte offsets of the chunks this lane moves, relative to the tile's first row
   uint32_t kvoff[IPW], vvoff[IPW];
@@ -128,6 +137,11 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
                    : "memory", "m0");
     }
 #endif
+  };
+
+  auto dma_v = [&](int jt, char* dst) {
+    const bool second = jt >= v_split_tiles;
+    dma_tile(second ? vrsrc2 : vrsrc, vvoff, static_cast<uint32_t>(second ? jt - v_split_tiles : jt) * v_tile_step, dst);
   };
 
   // ---- Q fragments stay in registers ----
@@ -230,7 +244,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
     const bool has_next = j + 1 < n_tiles;
     // buffers K[buf] (held K(j), consumed last tile) and V[buf^1] (held V(j-1)) are free now
     if (j + 2 < n_tiles) dma_tile(krsrc, kvoff, static_cast<uint32_t>(j + 2) * k_tile_step, Kb + buf * TILEB);
-    if (has_next) dma_tile(vrsrc, vvoff, static_cast<uint32_t>(j + 1) * v_tile_step, Vb + (buf ^ 1) * TILEB);
+    if (has_next) dma_v(j + 1, Vb + (buf ^ 1) * TILEB);
 
     const float mc = (m_run == -INFINITY) ? 0.f : m_run * c;
     uint32_t pf[2][2][4];
@@ -334,7 +348,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
 
   // ---- prologue (jt0 is even, so tile j always lives in buffer j & 1) ----
   dma_tile(krsrc, kvoff, static_cast<uint32_t>(jt0) * k_tile_step, Kb);
-  dma_tile(vrsrc, vvoff, static_cast<uint32_t>(jt0) * v_tile_step, Vb);
+  dma_v(jt0, Vb);
   if (jt0 + 1 < n_tiles) dma_tile(krsrc, kvoff, static_cast<uint32_t>(jt0 + 1) * k_tile_step, Kb + TILEB);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();

@@ -71,7 +71,7 @@ def _last_contig(t: torch.Tensor, name: str) -> None:
 def attn_fwd(
     q: torch.Tensor,
     k: torch.Tensor,
-    v: torch.Tensor,
+    v: torch.Tensor | tuple[torch.Tensor, torch.Tensor],
     scale: float,
     key_mask: torch.Tensor | None = None,
     return_lse: bool = False,
@@ -80,26 +80,51 @@ def attn_fwd(
 ):
     """softmax(q k^T * scale) v for q [B,Sq,H,D], k/v [B,Sk,Hkv,D] (BSHD, bf16/fp16).
 
+    ``v`` may be a pair (v_head [B,s,Hkv,D], v_tail [B,Sk-s,Hkv,D]) holding the value rows of keys
+    [0, s) and [s, Sk): the kernel reads both in place when s is a multiple of 64 and they share their
+    row stride (two fused-QKV projection outputs do); otherwise they are concatenated first.
+
     key_mask: optional [B,Sk] bool/uint8, False/0 = key excluded. Returns o [B,Sq,H,D]
     (and lse [B,H,Sq] float32 when return_lse). With ``split`` = s the output comes back as two dense
     tensors (o[:, :s], o[:, s:]) written directly by the kernel. ``use_workspace=False`` keeps the launch
     from cutting its last round of workgroups along the keys (no scratch buffer, one kernel).
     """
-    _dev(q, k, v, key_mask)
+    v_tail = None
+    if isinstance(v, (tuple, list)):
+        v, v_tail = v
+        if v.dim() != 4 or v_tail.dim() != 4 or k.dim() != 4 or v.shape[1] + v_tail.shape[1] != k.shape[1]:
+            raise ValueError(f"value pair {tuple(v.shape)} + {tuple(v_tail.shape)} does not cover k {tuple(k.shape)}")
+        direct = (v.dim() == 4 and v_tail.dim() == 4 and v.shape[1] % 64 == 0 and 0 < v.shape[1] and v_tail.shape[1] > 0
+                  and v.stride(1) == v_tail.stride(1) and v.dtype == v_tail.dtype
+                  and all(t.stride(-1) == 1 and all(x % 8 == 0 for x in t.stride()[:3]) and t.data_ptr() % 16 == 0
+                          for t in (v, v_tail))
+                  and attn_reads_value_pairs())
+        if not direct:
+            v, v_tail = torch.cat([v, v_tail], dim=1), None
+    _dev(q, k, v, v_tail, key_mask)
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("attn_fwd expects 4-D [B,S,H,D] tensors")
     if not (q.dtype == k.dtype == v.dtype):
         raise TypeError("q, k, v must share a dtype")
     B, Sq, H, D = q.shape
     Bk, Sk, Hkv, Dk = k.shape
-    if (Bk, Dk) != (B, D) or tuple(v.shape) != tuple(k.shape):
+    k_split = 0
+    if v_tail is not None:
+        k_split = v.shape[1]
+        if (v.shape[0], v.shape[2], v.shape[3]) != (B, Hkv, D) or tuple(v_tail.shape) != (B, Sk - k_split, Hkv, D):
+            raise ValueError(f"value pair {tuple(v.shape)} + {tuple(v_tail.shape)} does not cover k {tuple(k.shape)}")
+    elif (Bk, Dk) != (B, D) or tuple(v.shape) != tuple(k.shape):
         raise ValueError(f"shape mismatch: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
+    if Bk != B or Dk != D:
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)}, k {tuple(k.shape)}")
 
     def _prep(t):
         ok = t.stride(-1) == 1 and all(s % 8 == 0 for s in t.stride()[:3]) and t.data_ptr() % 16 == 0
         return t if ok else t.contiguous()
 
-    q, k, v = _prep(q), _prep(k), _prep(v)
+    q, k = _prep(q), _prep(k)
+    if v_tail is None:
+        v = _prep(v)
     if split is not None and not 0 <= split <= Sq:
         raise ValueError(f"split={split} outside [0, {Sq}]")
     o = torch.empty((B, Sq if split is None else split, H, D), dtype=q.dtype, device=q.device)
@@ -123,16 +148,28 @@ def attn_fwd(
     t_str = None if tail_t is None else _lib.i64_array(((Sq - cut) * H * D, H * D, D))
     ws = _attn_workspace(lib, q.device, B, Sq, Sk, H, D) if use_workspace else None
     rc = lib.odit_attn_fwd_ex(
-        q.data_ptr(), k.data_ptr(), v.data_ptr(), head_t.data_ptr(), _ptr(tail_t), cut,
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), _ptr(v_tail), k_split, head_t.data_ptr(), _ptr(tail_t), cut,
         _ptr(mask_u8), _ptr(lse), B, Sq, Sk, H, Hkv, D,
         _lib.i64_array(q.stride()[:3]), _lib.i64_array(k.stride()[:3]),
-        _lib.i64_array(v.stride()[:3]), _lib.i64_array(o_str), t_str,
+        _lib.i64_array(v.stride()[:3]), None if v_tail is None else _lib.i64_array(v_tail.stride()[:3]),
+        _lib.i64_array(o_str), t_str,
         float(scale), _code(q), _ptr(ws), 0 if ws is None else ws.numel(), _stream(),
     )
+    if rc == -2 and v_tail is not None:  # ODIT_ENOTSUP: spans too large for the kernel that reads value pairs
+        return attn_fwd(q, k, torch.cat([v, v_tail], dim=1), scale, key_mask=key_mask, return_lse=return_lse,
+                        split=split, use_workspace=use_workspace)
     _lib.check(rc, "odit_attn_fwd_ex")
     if split is None:
         return (o, lse) if return_lse else o
     return (o, o_tail, lse) if return_lse else (o, o_tail)
+
+
+def attn_reads_value_pairs() -> bool:
+    """Whether the selected attention kernel takes the values as two tensors (the default one does; the
+    earlier variants kept for cross-checks, chosen with ODIT_ATTN_VARIANT, do not)."""
+    import os
+
+    return os.environ.get("ODIT_ATTN_VARIANT", "34") in ("34", "38")
 
 
 _ATTN_SCRATCH: dict[tuple[int, int], torch.Tensor] = {}
