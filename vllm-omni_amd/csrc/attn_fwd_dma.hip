@@ -131,10 +131,15 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
 #pragma unroll
     for (int i = 0; i < IPW; ++i) {
       const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds0 + i * 1024);
+      // m0 (the LDS destination of the load) is a reserved register: naming it as clobbered draws a
+      // warning per expansion, and leaving it out would hide the write from the compiler
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                    :
                    : "s"(m0v), "v"(voff[i]), "s"(rsrc), "s"(soff)
                    : "memory", "m0");
+#pragma clang diagnostic pop
     }
 #endif
   };
