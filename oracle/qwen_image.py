@@ -120,25 +120,35 @@ def qwen_rope_freqs(cfg: QwenConfig, frame: int, height: int, width: int, txt_le
     return qwen_rope_freqs_images(cfg, [(frame, height, width)], txt_len)
 
 
-def qwen_rope_freqs_images(cfg: QwenConfig, shapes, txt_len: int):
+def qwen_rope_freqs_images(cfg: QwenConfig, shapes, txt_len: int, layer3d: bool = False):
     """The same tables for a sample made of several images (editing: source, then targets): image
     number ``idx`` takes frame positions idx .. idx+frame-1, its rows and columns are centred on its own
     grid, the token rows of all images are concatenated, and text positions start after the largest
-    half-extent of any image. qit.py:340-396."""
+    half-extent of any image. qit.py:340-396.
+
+    ``layer3d`` (QwenEmbedLayer3DRope, qit.py:183-296, the layered-image variant): the LAST image of the
+    list is the condition image and sits at frame position -1 instead of its list index, and the text
+    start is also at least the number of layers (= len(shapes) - 1)."""
     a0, a1, a2 = cfg.axes_dims_rope
     pos = torch.arange(4096)
     neg = torch.arange(4096).flip(0) * -1 - 1
     pos_f = [_axis_freqs(pos, a, cfg.theta) for a in (a0, a1, a2)]
     neg_f = [_axis_freqs(neg, a, cfg.theta) for a in (a0, a1, a2)]
     vids, start = [], 0
+    layer_num = len(shapes) - 1
     for idx, (frame, height, width) in enumerate(shapes):
-        f_frame = pos_f[0][idx:idx + frame].view(frame, 1, 1, -1).expand(frame, height, width, -1)
+        if layer3d and idx == layer_num:
+            f_frame = neg_f[0][-1:].view(frame, 1, 1, -1).expand(frame, height, width, -1)  # frame must be 1
+        else:
+            f_frame = pos_f[0][idx:idx + frame].view(frame, 1, 1, -1).expand(frame, height, width, -1)
         f_h = torch.cat([neg_f[1][-(height - height // 2):], pos_f[1][: height // 2]], dim=0)
         f_h = f_h.view(1, height, 1, -1).expand(frame, height, width, -1)
         f_w = torch.cat([neg_f[2][-(width - width // 2):], pos_f[2][: width // 2]], dim=0)
         f_w = f_w.view(1, 1, width, -1).expand(frame, height, width, -1)
         vids.append(torch.cat([f_frame, f_h, f_w], dim=-1).reshape(frame * height * width, -1))
         start = max(start, height // 2, width // 2)
+    if layer3d:
+        start = max(start, layer_num)
     txt = torch.cat(pos_f, dim=1)[start:start + txt_len].contiguous()
     return torch.cat(vids, dim=0).contiguous(), txt
 
@@ -213,20 +223,28 @@ def block_forward(w, i: int, cfg: QwenConfig, img, txt, temb, vid_freqs, txt_fre
     return txt, img
 
 
-def time_text_embed(w, timestep: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
-    """QwenTimestepProjEmbeddings: sinusoid(256, scale 1000) -> Linear -> SiLU -> Linear. qit.py:159-181."""
+def time_text_embed(w, timestep: torch.Tensor, dtype: torch.dtype, addition_t_cond=None) -> torch.Tensor:
+    """QwenTimestepProjEmbeddings: sinusoid(256, scale 1000) -> Linear -> SiLU -> Linear, plus, when the
+    checkpoint has ``addition_t_embedding`` (use_additional_t_cond), the row of that 2-entry table picked
+    by ``addition_t_cond`` [N] (integers 0/1). qit.py:159-181."""
     proj = ops.timestep_embedding(timestep).to(dtype)
     h = _lin(w, "time_text_embed.timestep_embedder.linear_1", proj)
-    return _lin(w, "time_text_embed.timestep_embedder.linear_2", F.silu(h))
+    out = _lin(w, "time_text_embed.timestep_embedder.linear_2", F.silu(h))
+    table = w.get("time_text_embed.addition_t_embedding.weight")
+    if table is not None:
+        if addition_t_cond is None:
+            raise ValueError("When additional_t_cond is True, addition_t_cond must be provided.")
+        out = out + F.embedding(addition_t_cond, table).to(dtype)
+    return out
 
 
-def stem(w, cfg: QwenConfig, latents, text, timestep):
+def stem(w, cfg: QwenConfig, latents, text, timestep, addition_t_cond=None):
     """img_in, txt_norm, txt_in, time_text_embed. qit.py:1003-1024."""
     img = _lin(w, "img_in", latents)
     timestep = timestep.to(dtype=img.dtype)
     txt = ops.rms_norm_head(text, w["txt_norm.weight"], cfg.eps)
     txt = _lin(w, "txt_in", txt)
-    temb = time_text_embed(w, timestep, img.dtype)
+    temb = time_text_embed(w, timestep, img.dtype, addition_t_cond)
     return img, txt, temb
 
 
@@ -244,7 +262,8 @@ def modulated_input(w, cfg: QwenConfig, img, temb):
 
 
 def transformer_forward(w, cfg: QwenConfig, latents, text, timestep, img_shape, key_mask=None,
-                        collect_blocks: bool = False, zero_cond_t: bool = False):
+                        collect_blocks: bool = False, zero_cond_t: bool = False, layer3d_rope: bool = False,
+                        addition_t_cond=None):
     """QwenImageTransformer2DModel.forward, qit.py:951-1071. latents [B,S_img,in], text [B,S_txt,J],
     timestep [B] in [0,1]; img_shape = (frame, height, width) of the patch grid, or a list of them when the
     sample is several images (rotary tables and, with ``zero_cond_t``, the per-token conditioning index
@@ -255,8 +274,8 @@ def transformer_forward(w, cfg: QwenConfig, latents, text, timestep, img_shape, 
     if zero_cond_t:
         timestep = torch.cat([timestep, timestep * 0], dim=0)
         index = modulate_index([shapes] * latents.shape[0]).to(latents.device)
-    img, txt, temb = stem(w, cfg, latents, text, timestep)
-    vid_freqs, txt_freqs = qwen_rope_freqs_images(cfg, shapes, txt_len=text.shape[1])
+    img, txt, temb = stem(w, cfg, latents, text, timestep, addition_t_cond)
+    vid_freqs, txt_freqs = qwen_rope_freqs_images(cfg, shapes, txt_len=text.shape[1], layer3d=layer3d_rope)
     per_block = []
     for i in range(cfg.num_layers):
         txt, img = block_forward(w, i, cfg, img, txt, temb, vid_freqs, txt_freqs, key_mask,

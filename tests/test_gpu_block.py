@@ -21,7 +21,7 @@ def _cosine(a, b):
     return float(torch.dot(a, b) / (a.norm() * b.norm()))
 
 
-def _build(gpu, dtype=torch.bfloat16, seed=0, bias_std=0.02, ref_rounding=False, **model_kwargs):
+def _build(gpu, dtype=torch.bfloat16, seed=0, bias_std=0.02, ref_rounding=False, load=True, **model_kwargs):
     from vllm_omni_amd.attention.selector import get_attn_backend
     from vllm_omni_amd.blocks.qwen_image import QwenImageTransformer2DModel
 
@@ -34,7 +34,8 @@ def _build(gpu, dtype=torch.bfloat16, seed=0, bias_std=0.02, ref_rounding=False,
         attention_head_dim=cfg.head_dim, num_attention_heads=cfg.num_heads,
         joint_attention_dim=cfg.joint_attention_dim, axes_dims_rope=cfg.axes_dims_rope,
         ref_rounding=ref_rounding, **model_kwargs).to(gpu).to(dtype)
-    model.load_flat_state(w_lp)
+    if load:
+        model.load_flat_state(w_lp)
     return cfg, w_lp, model
 
 
@@ -198,6 +199,35 @@ def test_editing_variant_per_token_conditioning(gpu, fuse):
     assert err <= 2e-2 and _cosine(got, want) >= 0.9995
     # the test would not notice a dropped index if the two models agreed anyway: they do not
     assert (plain - want).abs().max().item() > 10 * err
+
+
+def test_layered_variant_rope_and_additional_t_cond(gpu):
+    """use_layer3d_rope (condition image at frame -1, text start at least the layer count) and
+    use_additional_t_cond (a 2-entry learned embedding added to the timestep embedding)."""
+    cfg, w, model = _build(gpu, use_layer3d_rope=True, use_additional_t_cond=True, load=False)
+    g = torch.Generator().manual_seed(51)
+    w = dict(w)
+    w["time_text_embed.addition_t_embedding.weight"] = torch.randn(2, cfg.dim, generator=g).bfloat16()
+    # sharper attention (q/k norm weights 3 -> logits x9): with N(0, 0.02) projections the attention is close
+    # to uniform and positions would hardly matter
+    w = {k: (v * 3 if k.endswith(("norm_q.weight", "norm_k.weight")) else v) for k, v in w.items()}
+    model.load_flat_state(w)
+    shapes = [(1, 8, 8), (1, 8, 8), (1, 8, 8), (1, 8, 8)]   # three layers + the condition image, 256 tokens
+    lat, txt, t = _inputs(2, seed=52)
+    cond = torch.tensor([1, 0])
+    w32 = {k: v.float() for k, v in w.items()}
+    want = oq.transformer_forward(w32, cfg, lat.float(), txt.float(), t.float(), shapes, layer3d_rope=True,
+                                  addition_t_cond=cond)
+    other = oq.transformer_forward(w32, cfg, lat.float(), txt.float(), t.float(), shapes, addition_t_cond=cond)
+    with torch.inference_mode():
+        got = model(lat.to(gpu), txt.to(gpu), None, t.to(gpu), [shapes, shapes], [S_TXT],
+                    additional_t_cond=cond.to(gpu)).sample
+        with pytest.raises(ValueError, match="addition_t_cond"):
+            model(lat.to(gpu), txt.to(gpu), None, t.to(gpu), [shapes, shapes], [S_TXT])
+    err = (got.float().cpu() - want).abs().max().item()
+    print(f"layered variant: max-abs {err:.4f} cosine {_cosine(got, want):.6f}", flush=True)
+    assert err <= 2e-2 and _cosine(got, want) >= 0.9995
+    assert (other - want).abs().max().item() > 5 * err   # the frame position of the last image matters
 
 
 def test_teacache_refuses_the_editing_variant(gpu):

@@ -23,16 +23,20 @@ def _setup(seed=0, B=2, grid=(1, 4, 6), n_txt=7, dtype=torch.float64, bias_std=0
     return cfg, w, lat, txt, t
 
 
-def _expected_tables(cfg, shapes, txt_len):
+def _expected_tables(cfg, shapes, txt_len, layer3d=False):
     """Positions stated directly: image idx has frames idx.., rows y - ceil(h/2), columns x - ceil(w/2);
-    text token j sits at max over images of max(h//2, w//2), plus j, on all three axes."""
+    text token j sits at max over images of max(h//2, w//2), plus j, on all three axes. Layered variant:
+    the last image sits at frame -1 and the text start is at least the number of layers."""
     rows = []
     for idx, (f, h, w) in enumerate(shapes):
+        first = -1 if layer3d and idx == len(shapes) - 1 else idx
         for t in range(f):
             for y in range(h):
                 for x in range(w):
-                    rows.append((idx + t, y - (h + 1) // 2, x - (w + 1) // 2))
+                    rows.append((first + t, y - (h + 1) // 2, x - (w + 1) // 2))
     start = max(max(h // 2, w // 2) for _, h, w in shapes)
+    if layer3d:
+        start = max(start, len(shapes) - 1)
     txt_rows = [(start + j,) * 3 for j in range(txt_len)]
 
     def table(pos_rows):
@@ -57,6 +61,38 @@ def test_rotary_tables_against_numpy_positions():
     one = oq.qwen_rope_freqs(cfg, 1, 4, 6, txt_len=5)
     many = oq.qwen_rope_freqs_images(cfg, [(1, 4, 6)], txt_len=5)
     assert torch.equal(one[0], many[0]) and torch.equal(one[1], many[1])
+
+
+def test_layered_rotary_tables_against_numpy_positions():
+    cfg = oq.tiny_config()
+    for shapes in ([(1, 4, 6), (1, 4, 6), (1, 4, 6)], [(1, 2, 2)] * 5 + [(1, 2, 3)], [(1, 3, 3)]):
+        vid, txt = oq.qwen_rope_freqs_images(cfg, shapes, txt_len=4, layer3d=True)
+        want_v, want_t = _expected_tables(cfg, shapes, 4, layer3d=True)
+        np.testing.assert_allclose(vid.numpy(), want_v, atol=1e-5)
+        np.testing.assert_allclose(txt.numpy(), want_t, atol=1e-5)
+    # five 2x2 layers: the half-extents are 1, so the layer count (5) decides where the text starts
+    _, txt = oq.qwen_rope_freqs_images(cfg, [(1, 2, 2)] * 5 + [(1, 2, 3)], txt_len=1, layer3d=True)
+    _, txt_plain = oq.qwen_rope_freqs_images(cfg, [(1, 2, 2)] * 5 + [(1, 2, 3)], txt_len=6)
+    assert torch.equal(txt[0], txt_plain[4])  # plain start is 1: its row 4 is position 5
+
+
+def test_additional_t_cond_adds_the_picked_table_row():
+    cfg, w, lat, txt, t = _setup()
+    w = dict(w)
+    table = torch.randn(2, cfg.dim, generator=torch.Generator().manual_seed(9), dtype=torch.float64)
+    base = oq.time_text_embed(w, t, torch.float64)
+    w["time_text_embed.addition_t_embedding.weight"] = table
+    got = oq.time_text_embed(w, t, torch.float64, torch.tensor([1, 0]))
+    torch.testing.assert_close(got - base, table[[1, 0]], atol=1e-12, rtol=0)
+    import pytest
+    with pytest.raises(ValueError):
+        oq.time_text_embed(w, t, torch.float64)
+    # a zero table leaves the whole forward unchanged
+    w["time_text_embed.addition_t_embedding.weight"] = torch.zeros_like(table)
+    plain = {k: v for k, v in w.items() if "addition_t" not in k}
+    torch.testing.assert_close(
+        oq.transformer_forward(w, cfg, lat, txt, t, (1, 4, 6), addition_t_cond=torch.tensor([1, 1])),
+        oq.transformer_forward(plain, cfg, lat, txt, t, (1, 4, 6)), atol=0, rtol=0)
 
 
 def test_modulate_index_layout():

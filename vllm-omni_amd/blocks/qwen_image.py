@@ -115,6 +115,8 @@ class QwenEmbedRope(nn.Module):
     ``forward`` returns complex64 (vid_freqs, txt_freqs) like the reference; ``cos_sin`` returns the
     float32 [S, D/2] tables the fused kernel reads, cached per (shape, device)."""
 
+    layer3d = False  # QwenEmbedLayer3DRope sets it
+
     def __init__(self, theta: int, axes_dim: list[int], scale_rope: bool = True):
         super().__init__()
         self.theta, self.axes_dim, self.scale_rope = theta, list(axes_dim), scale_rope
@@ -132,10 +134,17 @@ class QwenEmbedRope(nn.Module):
         return torch.polar(torch.ones_like(ang), ang)
 
     def _video_freqs(self, frame: int, height: int, width: int, idx: int = 0) -> torch.Tensor:
+        """``idx`` = frame position of the image's first frame; -1 = the condition image of the layered
+        variant, which sits one frame before the origin (qit.py:278-296)."""
         halves = [d // 2 for d in self.axes_dim]
         fp = self.pos_freqs.split(halves, dim=1)
         fn = self.neg_freqs.split(halves, dim=1)
-        f_t = fp[0][idx:idx + frame].view(frame, 1, 1, -1).expand(frame, height, width, -1)
+        if idx < 0:
+            if frame != 1:
+                raise ValueError("the condition image of the layered variant has one frame")
+            f_t = fn[0][-1:].view(1, 1, 1, -1).expand(frame, height, width, -1)
+        else:
+            f_t = fp[0][idx:idx + frame].view(frame, 1, 1, -1).expand(frame, height, width, -1)
         if self.scale_rope:
             rows = torch.cat([fn[1][-(height - height // 2):], fp[1][: height // 2]], dim=0)
             cols = torch.cat([fn[2][-(width - width // 2):], fp[2][: width // 2]], dim=0)
@@ -147,9 +156,12 @@ class QwenEmbedRope(nn.Module):
 
     def _build(self, shapes: tuple[tuple[int, int, int], ...], txt_len: int, device: str):
         vids, start = [], 0
+        layer_num = len(shapes) - 1
         for idx, (f, h, w) in enumerate(shapes):
-            vids.append(self._video_freqs(f, h, w, idx))
+            vids.append(self._video_freqs(f, h, w, -1 if self.layer3d and idx == layer_num else idx))
             start = max(start, max(h // 2, w // 2) if self.scale_rope else max(h, w))
+        if self.layer3d:
+            start = max(start, layer_num)
         vid = torch.cat(vids, dim=0).to(device)
         txt = self.pos_freqs[start:start + txt_len].to(device)
         return vid, txt
@@ -164,6 +176,14 @@ class QwenEmbedRope(nn.Module):
 
     def forward(self, video_fhw, txt_seq_lens, device):
         return self._tables(self._norm_shapes(video_fhw), int(max(txt_seq_lens)), str(device))
+
+
+class QwenEmbedLayer3DRope(QwenEmbedRope):
+    """The layered-image variant's tables (qit.py:183-296): as QwenEmbedRope for the layers, the last
+    image of the list (the condition image) at frame position -1, text after the larger of the images'
+    half-extents and the number of layers."""
+
+    layer3d = True
 
 
 class RotaryTables:
@@ -337,11 +357,15 @@ class TimestepEmbedding(nn.Module):
 
 
 class QwenTimestepProjEmbeddings(nn.Module):
-    """Sinusoid(256 channels, cos first, scale 1000) -> MLP (qit.py:159-181)."""
+    """Sinusoid(256 channels, cos first, scale 1000) -> MLP, plus a 2-entry learned embedding picked by
+    ``addition_t_cond`` when ``use_additional_t_cond`` (qit.py:159-181)."""
 
-    def __init__(self, embedding_dim: int):
+    def __init__(self, embedding_dim: int, use_additional_t_cond: bool = False):
         super().__init__()
         self.timestep_embedder = TimestepEmbedding(256, embedding_dim)
+        self.use_additional_t_cond = use_additional_t_cond
+        if use_additional_t_cond:
+            self.addition_t_embedding = nn.Embedding(2, embedding_dim)
 
     @staticmethod
     def time_proj(t: torch.Tensor, dim: int = 256, max_period: int = 10000, scale: float = 1000.0):
@@ -353,7 +377,12 @@ class QwenTimestepProjEmbeddings(nn.Module):
         return torch.cat((torch.cos(arg), torch.sin(arg)), dim=-1)
 
     def forward(self, timestep: torch.Tensor, hidden_states: torch.Tensor, addition_t_cond=None):
-        return self.timestep_embedder(self.time_proj(timestep).to(hidden_states.dtype))
+        emb = self.timestep_embedder(self.time_proj(timestep).to(hidden_states.dtype))
+        if self.use_additional_t_cond:
+            if addition_t_cond is None:
+                raise ValueError("When additional_t_cond is True, addition_t_cond must be provided.")
+            emb = emb + self.addition_t_embedding(addition_t_cond).to(hidden_states.dtype)
+        return emb
 
 
 class AdaLayerNormContinuous(nn.Module):
@@ -380,13 +409,15 @@ class QwenImageTransformer2DModel(nn.Module):
                  num_layers: int = 60, attention_head_dim: int = 128, num_attention_heads: int = 24,
                  joint_attention_dim: int = 3584, axes_dims_rope: tuple[int, int, int] = (16, 56, 56),
                  mlp_ratio: int = 4, ref_rounding: bool = False, fuse_epilogues: bool = True,
-                 zero_cond_t: bool = False):
+                 zero_cond_t: bool = False, use_additional_t_cond: bool = False, use_layer3d_rope: bool = False):
         super().__init__()
         self.in_channels = in_channels
         self.out_channels = out_channels or in_channels
         self.inner_dim = num_attention_heads * attention_head_dim
-        self.pos_embed = QwenEmbedRope(theta=10000, axes_dim=list(axes_dims_rope), scale_rope=True)
-        self.time_text_embed = QwenTimestepProjEmbeddings(embedding_dim=self.inner_dim)
+        rope_cls = QwenEmbedLayer3DRope if use_layer3d_rope else QwenEmbedRope
+        self.pos_embed = rope_cls(theta=10000, axes_dim=list(axes_dims_rope), scale_rope=True)
+        self.time_text_embed = QwenTimestepProjEmbeddings(embedding_dim=self.inner_dim,
+                                                          use_additional_t_cond=use_additional_t_cond)
         self.txt_norm = RMSNorm(joint_attention_dim, eps=1e-6)
         self.img_in = nn.Linear(in_channels, self.inner_dim)
         self.txt_in = nn.Linear(joint_attention_dim, self.inner_dim)
@@ -403,7 +434,8 @@ class QwenImageTransformer2DModel(nn.Module):
         self.do_true_cfg = False
 
     # -- stages ---------------------------------------------------------------------------------
-    def prepare(self, hidden_states, encoder_hidden_states, timestep, img_shapes, txt_seq_lens):
+    def prepare(self, hidden_states, encoder_hidden_states, timestep, img_shapes, txt_seq_lens,
+                additional_t_cond=None):
         """Stem. With ``zero_cond_t`` (editing checkpoints) the timestep is doubled to [t, 0 * t], so temb
         has 2B rows: real-timestep conditioning, then timestep-zero conditioning (qit.py:141-145)."""
         img = self.img_in(hidden_states)
@@ -411,7 +443,9 @@ class QwenImageTransformer2DModel(nn.Module):
         if self.zero_cond_t:
             timestep = torch.cat([timestep, timestep * 0], dim=0)
         txt = self.txt_in(self.txt_norm(encoder_hidden_states))
-        temb = self.time_text_embed(timestep, img)
+        if additional_t_cond is not None and self.zero_cond_t:
+            additional_t_cond = torch.cat([additional_t_cond, additional_t_cond], dim=0)
+        temb = self.time_text_embed(timestep, img, additional_t_cond)
         if txt_seq_lens is None:
             txt_seq_lens = [encoder_hidden_states.shape[1]]
         vid_freqs, txt_freqs = self.pos_embed(img_shapes, txt_seq_lens, device=img.device)
@@ -502,7 +536,8 @@ class QwenImageTransformer2DModel(nn.Module):
                 encoder_hidden_states_mask: torch.Tensor = None, timestep: torch.Tensor = None,
                 img_shapes=None, txt_seq_lens=None, guidance: torch.Tensor = None,
                 attention_kwargs: dict[str, Any] | None = None, additional_t_cond=None, return_dict: bool = True):
-        img, txt, temb, rotary = self.prepare(hidden_states, encoder_hidden_states, timestep, img_shapes, txt_seq_lens)
+        img, txt, temb, rotary = self.prepare(hidden_states, encoder_hidden_states, timestep, img_shapes, txt_seq_lens,
+                                              additional_t_cond)
         index = self.modulate_index(img_shapes, img.device)
         img, txt = self.run_blocks(img, txt, temb, rotary, encoder_hidden_states_mask, attention_kwargs,
                                    modulate_index=index)

@@ -64,7 +64,8 @@ def extract_qwen_context(module: nn.Module, hidden_states: torch.Tensor,
         # the reference's extractor passes no per-token index to the blocks either (extractors.py:245-254):
         # an editing model under it would silently be modulated wrongly, so refuse instead
         raise NotImplementedError("TeaCache has no extractor for the zero_cond_t (editing) variant")
-    img, txt, temb, rotary = module.prepare(hidden_states, encoder_hidden_states, timestep, img_shapes, txt_seq_lens)
+    img, txt, temb, rotary = module.prepare(hidden_states, encoder_hidden_states, timestep, img_shapes, txt_seq_lens,
+                                            additional_t_cond)
     block0 = module.transformer_blocks[0]
     mod1 = block0.img_mod(temb).chunk(2, dim=-1)[0]
     modulated, _ = block0.img_norm1(img, mod1)
