@@ -365,3 +365,31 @@ def test_custom_ops_trace_with_fake_tensors():
         assert torch.ops.omni_dit.adaln_modulate(x, m, m, 1e-6).shape == x.shape
         t = torch.empty(70, 32, device="cuda")
         assert torch.ops.omni_dit.rotary(q, t, t, False).shape == q.shape
+
+
+def test_models_take_the_reference_constructor_calls():
+    """Pipelines build ``Model(od_config=od_config, **transformer_kwargs)`` (pipeline_qwen_image_edit.py:253):
+    the config object is accepted, a parallel degree above one is refused, Wan exposes ``.config``."""
+    from types import SimpleNamespace as NS
+
+    from vllm_omni_amd.blocks.flux import FluxTransformer2DModel
+    from vllm_omni_amd.blocks.qwen_image import QwenImageTransformer2DModel
+    from vllm_omni_amd.blocks.wan import WanTransformer3DModel
+
+    one = NS(parallel_config=NS(tensor_parallel_size=1, sequence_parallel_size=None, ulysses_degree=1, ring_degree=1,
+                                cfg_parallel_size=1), tf_model_config=NS(num_layers=1))
+    tiny = dict(num_layers=2, attention_head_dim=64, num_attention_heads=2, joint_attention_dim=32)
+    m = QwenImageTransformer2DModel(od_config=one, zero_cond_t=True, use_additional_t_cond=True, use_layer3d_rope=True,
+                                    guidance_embeds=False, quant_config=None, **tiny)
+    assert m.parallel_config is one.parallel_config and len(m.transformer_blocks) == 2
+    assert m.time_text_embed.addition_t_embedding.weight.shape == (2, 128) and m.pos_embed.layer3d
+    f = FluxTransformer2DModel(od_config=one, num_single_layers=1, pooled_projection_dim=16, **tiny)
+    assert len(f.transformer_blocks) == 1   # tf_model_config.num_layers wins, as in the reference
+    two = NS(parallel_config=NS(tensor_parallel_size=1, ulysses_degree=2))
+    for cls in (QwenImageTransformer2DModel, FluxTransformer2DModel):
+        with pytest.raises(NotImplementedError, match="ulysses_degree"):
+            cls(od_config=two, **tiny)
+    with pytest.raises(NotImplementedError, match="quantised"):
+        QwenImageTransformer2DModel(quant_config=object(), **tiny)
+    w = WanTransformer3DModel(num_attention_heads=2, attention_head_dim=64, ffn_dim=64, num_layers=1, text_dim=32)
+    assert w.config.patch_size == (1, 2, 2) and w.config.num_layers == 1 and w.config.image_dim is None

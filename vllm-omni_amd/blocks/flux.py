@@ -32,7 +32,7 @@ from ..attention.layer import Attention
 from ..layers.rmsnorm import RMSNorm
 from ..layers.rope import RotaryEmbedding
 from .qwen_image import (AdaLayerNormContinuous, FeedForward, QwenTimestepProjEmbeddings, TimestepEmbedding,
-                         Transformer2DModelOutput, project_residual)
+                         Transformer2DModelOutput, _require_single_gpu, project_residual)
 
 
 class FluxRotary:
@@ -326,12 +326,19 @@ class FluxTransformer2DModel(nn.Module):
 
     _repeated_blocks = ["FluxTransformerBlock"]
 
-    def __init__(self, patch_size: int = 1, in_channels: int = 64, out_channels: int | None = None,
-                 num_layers: int = 19, num_single_layers: int = 38, attention_head_dim: int = 128,
-                 num_attention_heads: int = 24, joint_attention_dim: int = 4096, pooled_projection_dim: int = 768,
-                 guidance_embeds: bool = True, axes_dims_rope: tuple[int, int, int] = (16, 56, 56),
-                 ref_rounding: bool = False):
+    def __init__(self, od_config: Any | None = None, patch_size: int = 1, in_channels: int = 64,
+                 out_channels: int | None = None, num_layers: int = 19, num_single_layers: int = 38,
+                 attention_head_dim: int = 128, num_attention_heads: int = 24, joint_attention_dim: int = 4096,
+                 pooled_projection_dim: int = 768, guidance_embeds: bool = True,
+                 axes_dims_rope: tuple[int, int, int] = (16, 56, 56), ref_rounding: bool = False):
+        """The reference's arguments (flux.py:436-450), ``od_config`` included: its ``tf_model_config.num_layers``
+        overrides ``num_layers`` as there, its ``parallel_config`` has to describe one GPU."""
         super().__init__()
+        _require_single_gpu(od_config)
+        tf_cfg = getattr(od_config, "tf_model_config", None)
+        if tf_cfg is not None and getattr(tf_cfg, "num_layers", None) is not None:
+            num_layers = tf_cfg.num_layers
+        self.parallel_config = getattr(od_config, "parallel_config", None)
         self.in_channels = in_channels
         self.out_channels = out_channels or in_channels
         self.inner_dim = num_attention_heads * attention_head_dim

@@ -31,6 +31,19 @@ from ..layers.rmsnorm import RMSNorm
 from ..layers.rope import RotaryEmbedding
 
 
+def _require_single_gpu(od_config: Any | None) -> None:
+    """The reference models read their parallel degrees from ``od_config.parallel_config``
+    (vllm_omni/diffusion/data.py); this package runs one GPU and refuses anything else."""
+    pc = getattr(od_config, "parallel_config", None)
+    if pc is None:
+        return
+    for name in ("sequence_parallel_size", "ulysses_degree", "ring_degree", "tensor_parallel_size",
+                 "cfg_parallel_size", "pipeline_parallel_size", "data_parallel_size"):
+        degree = getattr(pc, name, 1)
+        if degree not in (None, 1):
+            raise NotImplementedError(f"{name}={degree}: this package runs on one GPU")
+
+
 class Transformer2DModelOutput:
     """Minimal stand-in for diffusers' output object: ``.sample`` and ``[0]`` both work."""
 
@@ -405,12 +418,20 @@ class QwenImageTransformer2DModel(nn.Module):
 
     _repeated_blocks = ["QwenImageTransformerBlock"]
 
-    def __init__(self, patch_size: int = 2, in_channels: int = 64, out_channels: int | None = 16,
-                 num_layers: int = 60, attention_head_dim: int = 128, num_attention_heads: int = 24,
-                 joint_attention_dim: int = 3584, axes_dims_rope: tuple[int, int, int] = (16, 56, 56),
-                 mlp_ratio: int = 4, ref_rounding: bool = False, fuse_epilogues: bool = True,
-                 zero_cond_t: bool = False, use_additional_t_cond: bool = False, use_layer3d_rope: bool = False):
+    def __init__(self, od_config: Any | None = None, patch_size: int = 2, in_channels: int = 64,
+                 out_channels: int | None = 16, num_layers: int = 60, attention_head_dim: int = 128,
+                 num_attention_heads: int = 24, joint_attention_dim: int = 3584, guidance_embeds: bool = False,
+                 axes_dims_rope: tuple[int, int, int] = (16, 56, 56), zero_cond_t: bool = False,
+                 use_additional_t_cond: bool = False, use_layer3d_rope: bool = False, quant_config: Any | None = None,
+                 mlp_ratio: int = 4, ref_rounding: bool = False, fuse_epilogues: bool = True):
+        """Arguments up to ``quant_config`` are the reference's (qit.py:885-901), ``od_config`` included so a
+        pipeline's ``Model(od_config=..., **transformer_kwargs)`` call works unchanged; only its
+        ``parallel_config`` is looked at, and it has to describe one GPU."""
         super().__init__()
+        _require_single_gpu(od_config)
+        if quant_config is not None:
+            raise NotImplementedError("quantised linears are not part of this package")
+        self.guidance_embeds = guidance_embeds
         self.in_channels = in_channels
         self.out_channels = out_channels or in_channels
         self.inner_dim = num_attention_heads * attention_head_dim
@@ -430,7 +451,7 @@ class QwenImageTransformer2DModel(nn.Module):
         self.proj_out = nn.Linear(self.inner_dim, patch_size * patch_size * self.out_channels, bias=True)
         self.zero_cond_t = zero_cond_t
         self._res_bias = None
-        self.parallel_config = None
+        self.parallel_config = getattr(od_config, "parallel_config", None)
         self.do_true_cfg = False
 
     # -- stages ---------------------------------------------------------------------------------

@@ -424,6 +424,13 @@ class WanTransformer3DModel(nn.Module):
                  rope_max_seq_len: int = 1024, pos_embed_seq_len: int | None = None,
                  text_context_len: int = 512):
         super().__init__()
+        # attribute bag with the constructor arguments, as pipelines read it (wan.py:775-797)
+        self.config = type("Config", (), dict(
+            patch_size=patch_size, num_attention_heads=num_attention_heads, attention_head_dim=attention_head_dim,
+            in_channels=in_channels, out_channels=out_channels, text_dim=text_dim, freq_dim=freq_dim, ffn_dim=ffn_dim,
+            num_layers=num_layers, cross_attn_norm=cross_attn_norm, eps=eps, image_dim=image_dim,
+            added_kv_proj_dim=added_kv_proj_dim, rope_max_seq_len=rope_max_seq_len,
+            pos_embed_seq_len=pos_embed_seq_len))()
         inner_dim = num_attention_heads * attention_head_dim
         self.patch_size, self.inner_dim, self.eps = tuple(patch_size), inner_dim, eps
         self.in_channels, self.out_channels = in_channels, out_channels or in_channels
