@@ -382,9 +382,11 @@ def test_models_take_the_reference_constructor_calls():
     m = QwenImageTransformer2DModel(od_config=one, zero_cond_t=True, use_additional_t_cond=True, use_layer3d_rope=True,
                                     guidance_embeds=False, quant_config=None, **tiny)
     assert m.parallel_config is one.parallel_config and len(m.transformer_blocks) == 2
+    assert m.dtype == torch.float32 and m.in_channels == 64 and m.guidance_embeds is False and m.do_true_cfg is False
     assert m.time_text_embed.addition_t_embedding.weight.shape == (2, 128) and m.pos_embed.layer3d
     f = FluxTransformer2DModel(od_config=one, num_single_layers=1, pooled_projection_dim=16, **tiny)
     assert len(f.transformer_blocks) == 1   # tf_model_config.num_layers wins, as in the reference
+    assert f.dtype == torch.float32 and f.guidance_embeds is True
     two = NS(parallel_config=NS(tensor_parallel_size=1, ulysses_degree=2))
     for cls in (QwenImageTransformer2DModel, FluxTransformer2DModel):
         with pytest.raises(NotImplementedError, match="ulysses_degree"):

@@ -362,6 +362,10 @@ class FluxTransformer2DModel(nn.Module):
         self._res_bias = None
 
     # -- stages ---------------------------------------------------------------------------------
+    @property
+    def dtype(self) -> torch.dtype:
+        return next(self.parameters()).dtype
+
     def prepare(self, hidden_states, encoder_hidden_states, pooled_projections, timestep, img_ids, txt_ids,
                 guidance=None):
         img = self.x_embedder(hidden_states)

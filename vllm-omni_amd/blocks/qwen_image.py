@@ -454,6 +454,10 @@ class QwenImageTransformer2DModel(nn.Module):
         self.parallel_config = getattr(od_config, "parallel_config", None)
         self.do_true_cfg = False
 
+    @property
+    def dtype(self) -> torch.dtype:
+        return next(self.parameters()).dtype
+
     # -- stages ---------------------------------------------------------------------------------
     def prepare(self, hidden_states, encoder_hidden_states, timestep, img_shapes, txt_seq_lens,
                 additional_t_cond=None):
