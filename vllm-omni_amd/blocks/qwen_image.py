@@ -417,6 +417,7 @@ class QwenImageTransformer2DModel(nn.Module):
     are the three stages TeaCache needs to call separately (cache/teacache/extractors.py:147-279)."""
 
     _repeated_blocks = ["QwenImageTransformerBlock"]
+    enable_separate_cfg = True   # class attribute of the reference's CachedTransformer base (cache/base.py:105-112)
 
     def __init__(self, od_config: Any | None = None, patch_size: int = 2, in_channels: int = 64,
                  out_channels: int | None = 16, num_layers: int = 60, attention_head_dim: int = 128,
