@@ -79,6 +79,26 @@ def test_tiny_model_per_block_parity(gpu, monkeypatch, fuse_min_rows):
     assert torch.equal(out2, out)
 
 
+@pytest.mark.parametrize("B,grid,n_txt", [(2, (1, 12, 20), 37), (1, (1, 7, 9), 128), (3, (1, 16, 16), 5)])
+def test_tiny_model_ragged_shapes(gpu, B, grid, n_txt):
+    """Non-square grids, odd token counts, a text length that is not a multiple of the 64-key tile (the
+    values are then copied into the joint buffer instead of being read in place), batch 3."""
+    cfg, w, model = _build(gpu)
+    model.fuse_modulation()
+    g = torch.Generator().manual_seed(61)
+    n_img = grid[0] * grid[1] * grid[2]
+    lat = torch.randn(B, n_img, 64, generator=g).bfloat16()
+    txt = torch.randn(B, n_txt, 256, generator=g).bfloat16()
+    t = torch.rand(B, generator=g).bfloat16()
+    w32 = {k: v.float() for k, v in w.items()}
+    want = oq.transformer_forward(w32, cfg, lat.float(), txt.float(), t.float(), grid)
+    with torch.inference_mode():
+        got = model(lat.to(gpu), txt.to(gpu), None, t.to(gpu), [grid], [n_txt]).sample
+    err = (got.float().cpu() - want).abs().max().item()
+    print(f"B={B} grid={grid} text={n_txt}: max-abs {err:.4f} cosine {_cosine(got, want):.6f}", flush=True)
+    assert err <= 2e-2 and _cosine(got, want) >= 0.9995
+
+
 def test_headline_shape_block_against_oracle(gpu):
     """One block at the width and sequence the metric is quoted on (hidden 3072 = 24 heads x 128, MLP 12288,
     batch 2, 4096 image + 256 text tokens, 64x64 rotary grid) against the fp32 oracle of the same block: the
