@@ -4,15 +4,17 @@
  *
  * Conventions
  *   - Every pointer except `stream` is a DEVICE pointer owned by the caller. No entry point
- *     allocates, frees or synchronises; all work is enqueued on `stream` (a hipStream_t; NULL = the
- *     legacy default stream).
+ *     allocates or frees device memory, and none synchronises except odit_linear_tune (a set-up
+ *     call that times kernels); all work is enqueued on `stream` (a hipStream_t; NULL = the legacy
+ *     default stream).
  *   - Tensors are row-major with the innermost dimension contiguous. Strides are in ELEMENTS.
  *   - `dtype` is one of ODIT_BF16 / ODIT_F16 / ODIT_F32 and names the element type of the activation
  *     tensors. Arithmetic inside every kernel is fp32.
  *   - Return value: 0 on success, a negative ODIT_E* code on failure; odit_last_error() then returns a
  *     thread-local, NUL-terminated description. Argument errors are detected on the host BEFORE any
  *     launch, so a failing call enqueues nothing.
- *   - Re-entrant; no global mutable state apart from the thread-local error string.
+ *   - Re-entrant; the only state kept between calls is thread-local: the error string, and in
+ *     odit_linear the library handle with the matmul descriptors of the problems seen so far.
  *
  * The reference (Flink-ddd/vllm-omni) is pure Python and has no FFI of its own for this path; each
  * entry point below replaces the third-party kernel call(s) made at the cited reference lines.
