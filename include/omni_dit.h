@@ -14,7 +14,8 @@
  *     thread-local, NUL-terminated description. Argument errors are detected on the host BEFORE any
  *     launch, so a failing call enqueues nothing.
  *   - Re-entrant; the only state kept between calls is thread-local: the error string, and in
- *     odit_linear the library handle with the matmul descriptors of the problems seen so far.
+ *     odit_linear the library handle with the matmul descriptors of the problems seen so far
+ *     (plus a process-wide, write-once table of each device's compute-unit count).
  *
  * The reference (Flink-ddd/vllm-omni) is pure Python and has no FFI of its own for this path; each
  * entry point below replaces the third-party kernel call(s) made at the cited reference lines.
