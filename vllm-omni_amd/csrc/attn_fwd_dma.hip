@@ -413,6 +413,8 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
 // Merge of the key-split tail: one wavefront per query row adds the row's key_chunks partial results,
 //   O = sum_c 2^((m_c - m) c) O_c / sum_c 2^((m_c - m) c) l_c,   m = max_c m_c,
 // and writes the row (and its log-sum-exp) where the unsplit kernel would have.
+constexpr int kMergeMaxChunks = 16;  // = kMaxKeyChunks below
+
 template <typename T, int D, int BM>
 __global__ __launch_bounds__(256) void attn_merge_kernel(const AttnParams p, int n_parts) {
   using M = Mma<T>;
@@ -426,22 +428,36 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const AttnParams p, int
   const int row = qb * BM + r;
   if (row >= p.Sq) return;
   const float* ml = p.ws + static_cast<int64_t>(n_parts) * BM * D;
-  float m = -INFINITY;
-  for (int cidx = 0; cidx < p.key_chunks; ++cidx)
-    m = fmaxf(m, ml[(static_cast<int64_t>(unit * p.key_chunks + cidx) * BM + r) * 2]);
-  const float m_safe = m == -INFINITY ? 0.f : m;
+  // every load of the row is issued before the first use: the loop bounds are compile-time (kMergeMaxChunks
+  // is the most ranges plan_tail hands out) and the ranges beyond key_chunks are predicated off, so the
+  // kernel pays one memory latency, not one per range
   constexpr int EPL = D / 64;  // consecutive elements per lane
+  float mc[kMergeMaxChunks], lc[kMergeMaxChunks], part[kMergeMaxChunks][EPL];
+#pragma unroll
+  for (int cidx = 0; cidx < kMergeMaxChunks; ++cidx) {
+    const bool on = cidx < p.key_chunks;
+    const int64_t pr = static_cast<int64_t>(unit * p.key_chunks + (on ? cidx : 0)) * BM + r;
+    mc[cidx] = on ? ml[pr * 2] : -INFINITY;
+    lc[cidx] = on ? ml[pr * 2 + 1] : 0.f;
+    const float* src = p.ws + pr * D + lane * EPL;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) part[cidx][e] = on ? src[e] : 0.f;
+  }
+  float m = -INFINITY;
+#pragma unroll
+  for (int cidx = 0; cidx < kMergeMaxChunks; ++cidx) m = fmaxf(m, mc[cidx]);
+  const float m_safe = m == -INFINITY ? 0.f : m;
   float acc[EPL];
 #pragma unroll
   for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
   float l = 0.f;
-  for (int cidx = 0; cidx < p.key_chunks; ++cidx) {
-    const int64_t pr = static_cast<int64_t>(unit * p.key_chunks + cidx) * BM + r;
-    const float wgt = __builtin_amdgcn_exp2f((ml[pr * 2] - m_safe) * p.scale_log2);  // 0 for an empty range
-    l = fmaf(wgt, ml[pr * 2 + 1], l);
-    const float* src = p.ws + pr * D + lane * EPL;
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) acc[e] = fmaf(wgt, src[e], acc[e]);
+  for (int cidx = 0; cidx < kMergeMaxChunks; ++cidx) {
+    // same order of accumulation as a loop over the ranges; weight 0 for an empty or absent range
+    const float wgt = cidx < p.key_chunks ? __builtin_amdgcn_exp2f((mc[cidx] - m_safe) * p.scale_log2) : 0.f;
+    l = fmaf(wgt, lc[cidx], l);
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) acc[e] = fmaf(wgt, part[cidx][e], acc[e]);
   }
   const float inv = l > 0.f ? 1.f / l : 0.f;
   T* op = out_row_ptr<T>(p, b, h, row) + lane * EPL;
@@ -465,7 +481,7 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const AttnParams p, int
 // a side stream, concurrently with the full units, gave nothing over the same-stream order.
 struct TailPlan { int rem, key_chunks, tiles_per_chunk; };
 constexpr int kMinTilesPerChunk = 8;
-constexpr int kMaxKeyChunks = 16;
+constexpr int kMaxKeyChunks = kMergeMaxChunks;
 
 static int device_slots(int nw) {
   static int cus[64] = {0};
