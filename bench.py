@@ -308,6 +308,10 @@ def kernel_rooflines(torch):
     bw("gated_residual", [lambda i=i: kernels.gated_residual(xs[i], ys[i], gate, out=os_[i]) for i in range(NSET)],
        3 * n_el * 2)
     bw("rel_l1", [lambda i=i: kernels.rel_l1_sums(xs[i], ys[i]) for i in range(NSET)], 2 * n_el * 2)
+    # reference point, not a kernel of the path: what a plain device copy of the same 50 MB tensors reaches on
+    # this box with the same rotation of buffers (torch's copy kernel; gated residual with a gate of ones is
+    # this library's own streaming pass over three such tensors)
+    bw("reference_copy_50MB", [lambda i=i: os_[i].copy_(xs[i]) for i in range(NSET)], 2 * n_el * 2)
     del ys
     qkvs = [torch.randn(B, S_IMG, 3, HEADS, HEAD_DIM, device=dev, dtype=bf) for _ in range(NSET)]
     jqs = [[torch.empty(B, S_IMG + S_TXT, HEADS, HEAD_DIM, device=dev, dtype=bf) for _ in range(3)] for _ in range(NSET)]

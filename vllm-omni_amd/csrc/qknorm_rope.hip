@@ -119,7 +119,9 @@ template <typename T> __device__ __forceinline__ u32x4 pack_vec(const float (&x)
 }
 
 // ---- per-head (or no) statistics: one vector per lane, grid (vectors / 256, parts) ---------------
-template <typename T, typename TW, int NORM_MODE, bool GENERAL>
+// IDX32: vector and token numbers fit 32 bits (every launch short of 2^31 vectors), which spares each
+// lane two 64-bit integer divisions.
+template <typename T, typename TW, int NORM_MODE, bool GENERAL, bool IDX32>
 __global__ __launch_bounds__(256) void qknorm_flat_kernel(
     const T* __restrict__ q_in, const T* __restrict__ k_in, const T* __restrict__ v_in,
     T* __restrict__ q_out, T* __restrict__ k_out, T* __restrict__ v_out,
@@ -134,10 +136,19 @@ __global__ __launch_bounds__(256) void qknorm_flat_kernel(
   const int64_t i_raw = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   const bool valid = i_raw < total_vec;
   const int64_t i = valid ? i_raw : total_vec - 1;  // clamped lanes compute, never store
-  const int64_t tok = i / vec_per_row;
-  const int e0 = static_cast<int>(i - tok * vec_per_row) * EPV;
-  const int b = static_cast<int>(tok / S);
-  const int s = static_cast<int>(tok - static_cast<int64_t>(b) * S);
+  int e0, b, s;
+  if constexpr (IDX32) {
+    const unsigned iu = static_cast<unsigned>(i), vpr = static_cast<unsigned>(vec_per_row);
+    const unsigned tok = iu / vpr;
+    e0 = static_cast<int>(iu - tok * vpr) * EPV;
+    b = static_cast<int>(tok / static_cast<unsigned>(S));
+    s = static_cast<int>(tok - static_cast<unsigned>(b) * static_cast<unsigned>(S));
+  } else {
+    const int64_t tok = i / vec_per_row;
+    e0 = static_cast<int>(i - tok * vec_per_row) * EPV;
+    b = static_cast<int>(tok / S);
+    s = static_cast<int>(tok - static_cast<int64_t>(b) * S);
+  }
   const int64_t in_off = b * is_b + s * is_s + e0;
   const int64_t out_off = (static_cast<int64_t>(b) * S_total + out_seq_offset + s) * HD + e0;
   if (kind == 2) {  // block-uniform
@@ -149,7 +160,7 @@ __global__ __launch_bounds__(256) void qknorm_flat_kernel(
   float x[EPV];
 #pragma unroll
   for (int j = 0; j < EPV; ++j) x[j] = Raw<T>::get(r, j);
-  const int d0 = e0 % D;
+  const int d0 = (D & (D - 1)) == 0 ? (e0 & (D - 1)) : e0 % D;  // head sizes are powers of two in practice
   float rstd = 1.f;
   if constexpr (NORM_MODE == ODIT_NORM_HEAD) {
     float sq = 0.f;
@@ -265,12 +276,15 @@ template <typename T, typename TW, int NORM_MODE, bool GENERAL> static int qk_fl
   const int64_t total = static_cast<int64_t>(a.B) * a.S * vpr;
   const int nparts = 1 + (a.k_in != nullptr) + (a.v_in != nullptr);
   const dim3 grid(static_cast<unsigned>((total + 255) / 256), nparts);
-  hipLaunchKernelGGL((qknorm_flat_kernel<T, TW, NORM_MODE, GENERAL>), grid, dim3(256), 0, a.stream,
-                     static_cast<const T*>(a.q_in), static_cast<const T*>(a.k_in),
-                     static_cast<const T*>(a.v_in), static_cast<T*>(a.q_out), static_cast<T*>(a.k_out),
-                     static_cast<T*>(a.v_out), static_cast<const TW*>(a.wq), static_cast<const TW*>(a.wk),
-                     a.cos, a.sin, a.S, a.HD, a.D, a.rot, a.is_b, a.is_s, a.out_seq_offset, a.S_total,
-                     a.eps, vpr, total, a.neox, a.ref_round);
+#define ODIT_QK_FLAT(I32)                                                                          \
+  hipLaunchKernelGGL((qknorm_flat_kernel<T, TW, NORM_MODE, GENERAL, I32>), grid, dim3(256), 0, a.stream, \
+                     static_cast<const T*>(a.q_in), static_cast<const T*>(a.k_in),                  \
+                     static_cast<const T*>(a.v_in), static_cast<T*>(a.q_out), static_cast<T*>(a.k_out), \
+                     static_cast<T*>(a.v_out), static_cast<const TW*>(a.wq), static_cast<const TW*>(a.wk), \
+                     a.cos, a.sin, a.S, a.HD, a.D, a.rot, a.is_b, a.is_s, a.out_seq_offset, a.S_total, \
+                     a.eps, vpr, total, a.neox, a.ref_round)
+  if (total < (1ll << 31)) ODIT_QK_FLAT(true); else ODIT_QK_FLAT(false);
+#undef ODIT_QK_FLAT
   return check_launch("odit_qknorm_rope");
 }
 
