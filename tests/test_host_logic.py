@@ -395,3 +395,60 @@ def test_models_take_the_reference_constructor_calls():
         QwenImageTransformer2DModel(quant_config=object(), **tiny)
     w = WanTransformer3DModel(num_attention_heads=2, attention_head_dim=64, ffn_dim=64, num_layers=1, text_dim=32)
     assert w.config.patch_size == (1, 2, 2) and w.config.num_layers == 1 and w.config.image_dim is None
+
+
+# ------------------------------------------------------- cache backends, after the reference's own tests
+def test_cache_backend_and_selector_like_the_reference_tests(monkeypatch):
+    """tests/diffusion/cache/test_cache_backends.py:126-222 of the reference, against this package:
+    TeaCacheBackend init / enable / enable with coefficients / refresh, and the selector."""
+    from unittest.mock import Mock
+
+    from vllm_omni_amd.cache.base import DiffusionCacheConfig
+    from vllm_omni_amd.cache.selector import get_cache_backend
+    from vllm_omni_amd.cache.teacache import backend as backend_mod
+    from vllm_omni_amd.cache.teacache.backend import TeaCacheBackend
+
+    backend = TeaCacheBackend(DiffusionCacheConfig(rel_l1_thresh=0.3))
+    assert backend.config.rel_l1_thresh == 0.3 and backend.enabled is False and backend.is_enabled() is False
+
+    def pipeline():
+        p, t = Mock(), Mock()
+        p.__class__.__name__ = "QwenImagePipeline"
+        t.__class__.__name__ = "QwenImageTransformer2DModel"
+        p.transformer = t
+        return p, t
+
+    for cfg in (DiffusionCacheConfig(rel_l1_thresh=0.3),
+                DiffusionCacheConfig(rel_l1_thresh=0.3, coefficients=[1.0, 0.5, 0.2, 0.1, 0.05])):
+        applied = Mock()
+        monkeypatch.setattr(backend_mod, "apply_teacache_hook", applied)
+        backend = TeaCacheBackend(cfg)
+        p, t = pipeline()
+        backend.enable(p)
+        assert backend.enabled is True
+        applied.assert_called_once()
+        module, tc = applied.call_args[0]
+        assert module is t and tc.transformer_type == "QwenImageTransformer2DModel" and tc.rel_l1_thresh == 0.3
+        assert list(tc.coefficients) == (cfg.coefficients or [-4.5e2, 2.8e2, -4.5e1, 3.2, -2.0e-2])
+        assert backend.config is cfg   # the given object stays the backend's config
+    # a transformer class without coefficients is a configuration error, reported as ValueError
+    p, t = pipeline()
+    t.__class__.__name__ = "SomethingElse"
+    with pytest.raises(ValueError, match="Invalid TeaCache configuration"):
+        TeaCacheBackend(DiffusionCacheConfig()).enable(p)
+    # refresh resets the hook through the registry
+    p, t = pipeline()
+    t._hook_registry = Mock()
+    backend = TeaCacheBackend(DiffusionCacheConfig())
+    backend.enable(p)
+    backend.refresh(p, num_inference_steps=50)
+    t._hook_registry.reset_hook.assert_called_once()
+    # selector
+    assert get_cache_backend(None, None) is None and get_cache_backend("none", None) is None
+    b = get_cache_backend("tea_cache", {"rel_l1_thresh": 0.3, "Fn_compute_blocks": 4})
+    assert isinstance(b, TeaCacheBackend) and b.config.rel_l1_thresh == 0.3
+    with pytest.raises(ValueError, match="Unsupported cache backend"):
+        get_cache_backend("invalid_backend", {})
+    with pytest.raises(NotImplementedError):
+        get_cache_backend("cache_dit", {})
+    assert DiffusionCacheConfig.from_dict({}).rel_l1_thresh == 0.2

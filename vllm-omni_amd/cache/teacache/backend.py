@@ -6,24 +6,29 @@ from __future__ import annotations
 from typing import Any
 
 from ...hooks.base import HookRegistry
+from ..base import CacheBackend, DiffusionCacheConfig
 from .config import TeaCacheConfig
 from .hook import TeaCacheHook, apply_teacache_hook
 
 
-class TeaCacheBackend:
-    def __init__(self, config: dict[str, Any] | TeaCacheConfig | None = None):
-        self.config = config
-        self.enabled = False
+class TeaCacheBackend(CacheBackend):
+    def __init__(self, config: DiffusionCacheConfig | dict[str, Any] | TeaCacheConfig | None = None):
+        """``config``: the reference's DiffusionCacheConfig (or a dict of its fields); a ready TeaCacheConfig is
+        taken as it is. ``self.config`` keeps what was given, as in the reference."""
+        if config is None or isinstance(config, dict):
+            config = DiffusionCacheConfig.from_dict(config)
+        super().__init__(config)
 
     def enable(self, pipeline: Any) -> None:
         transformer = pipeline.transformer
         cfg = self.config
         if not isinstance(cfg, TeaCacheConfig):
-            kw = dict(cfg or {})
-            kw.setdefault("transformer_type", transformer.__class__.__name__)
-            cfg = TeaCacheConfig(**{k: v for k, v in kw.items()
-                                    if k in ("rel_l1_thresh", "coefficients", "transformer_type")})
-        self.config = cfg
+            try:
+                cfg = TeaCacheConfig(transformer_type=transformer.__class__.__name__,
+                                     rel_l1_thresh=cfg.rel_l1_thresh, coefficients=cfg.coefficients)
+            except Exception as e:
+                raise ValueError(f"Invalid TeaCache configuration: {e}. Expected keys: rel_l1_thresh, coefficients "
+                                 "(optional); transformer_type comes from pipeline.transformer.__class__.__name__.") from e
         apply_teacache_hook(transformer, cfg)
         self.enabled = True
 
@@ -32,9 +37,6 @@ class TeaCacheBackend:
         reg = getattr(pipeline.transformer, "_hook_registry", None)
         if reg is not None:
             reg.reset_hook(TeaCacheHook._HOOK_NAME)
-
-    def is_enabled(self) -> bool:
-        return self.enabled
 
     @staticmethod
     def hook_of(pipeline: Any) -> TeaCacheHook | None:
