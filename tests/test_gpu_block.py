@@ -3,6 +3,7 @@
 oracle, per block (max-abs <= 2e-2, cosine >= 0.9995); TeaCache decisions against the oracle's
 sequential-CFG state machine; CFG-batched against sequential calls."""
 
+import numpy as np
 import pytest
 import torch
 
@@ -376,3 +377,44 @@ def test_cfg_batched_equals_sequential(gpu):
     for i in range(2):
         d = (both[i:i + 1].float() - one[i].float()).abs().max().item()
         assert d <= 2e-2, d   # GEMM tiling may differ with M; everything else is row-independent
+
+
+def test_cfg_mixin_diffuse_one_call_against_two(gpu):
+    """The reference's step loop (QwenImageCFGParallelMixin.diffuse) around the HIP transformer, prompts of
+    different lengths: the one-call schedule (negative prompt padded and masked) against the reference's two
+    sequential calls, and, for equal lengths, against this package's own loop."""
+    from vllm_omni_amd import denoise
+
+    cfg, w, model = _build(gpu)
+    steps = 4
+    g = torch.Generator().manual_seed(21)
+    lat0 = torch.randn(1, S_IMG, 64, generator=g).bfloat16().to(gpu)
+    pos = torch.randn(1, S_TXT, 256, generator=g).bfloat16().to(gpu)
+    neg = torch.randn(1, S_TXT, 256, generator=g).bfloat16().to(gpu)
+
+    class Pipe(denoise.QwenImageCFGParallelMixin):
+        transformer = model
+
+    def run(batched, negative):
+        pipe = Pipe()
+        pipe.batch_cfg_branches = batched
+        pipe.scheduler = denoise.FlowMatchEulerScheduler()
+        pipe.scheduler.set_timesteps(sigmas=np.linspace(1.0, 1.0 / steps, steps), device=gpu,
+                                     mu=denoise.calculate_shift(S_IMG))
+        with torch.inference_mode():
+            return pipe.diffuse(pos, None, negative, None, lat0, [[IMG_SHAPE]], [S_TXT], [negative.shape[1]],
+                                pipe.scheduler.timesteps, True, None, 4.0, cfg_normalize=True,
+                                additional_transformer_kwargs={"return_dict": False})
+
+    short = neg[:, :40]
+    one_call, two_calls = run(True, short), run(False, short)
+    assert model.cfg_batched_branches is None          # the last run made two calls per step
+    d = (one_call.float() - two_calls.float()).abs().max().item()
+    print(f"ragged prompts, {steps} steps: one call vs two, max-abs {d:.4f}", flush=True)
+    assert d <= 5e-2 and _cosine(one_call, two_calls) >= 0.9995
+    # the padding must not leak: other padding values, same answer
+    same_len = run(True, neg)
+    with torch.inference_mode():
+        own = denoise.diffuse(model, denoise.DenoiseInputs(lat0, pos, neg, IMG_SHAPE), steps, 4.0, True)
+    assert torch.equal(same_len, own)
+    assert (same_len.float() - one_call.float()).abs().max().item() > 1e-2   # 24 more negative tokens matter

@@ -452,3 +452,149 @@ def test_cache_backend_and_selector_like_the_reference_tests(monkeypatch):
     with pytest.raises(NotImplementedError):
         get_cache_backend("cache_dit", {})
     assert DiffusionCacheConfig.from_dict({}).rel_l1_thresh == 0.2
+
+
+# ----------------------------------------------------------------------------------- CFG mixin
+class _RowMixer(torch.nn.Module):
+    """A per-sample token mixer (softmax over a sample's own positions): what one sample yields does
+    not depend on which other samples share its batch, as for a DiT."""
+
+    def __init__(self, channels: int = 4, width: int = 128, seed: int = 42):
+        super().__init__()
+        g = torch.Generator().manual_seed(seed)
+        self.w_in = torch.nn.Parameter(torch.randn(channels, width, generator=g) * 0.3)
+        self.w_qk = torch.nn.Parameter(torch.randn(width, width, generator=g) * 0.1)
+        self.w_out = torch.nn.Parameter(torch.randn(width, channels, generator=g) * 0.3)
+
+    def forward(self, x: torch.Tensor, **kwargs):
+        b, c, h, w = x.shape
+        s = x.flatten(2).transpose(1, 2) @ self.w_in
+        p = torch.softmax((s @ self.w_qk) @ s.transpose(1, 2) / s.shape[-1] ** 0.5, dim=-1)
+        s = torch.nn.functional.layer_norm(s + p @ s, (s.shape[-1],))
+        return ((s @ self.w_out).transpose(1, 2).reshape(b, c, h, w),)
+
+
+class _Pipe(denoise.CFGParallelMixin):
+    def __init__(self, batch_branches: bool):
+        self.transformer = _RowMixer().double().eval()
+        self.batch_cfg_branches = batch_branches
+
+
+@pytest.mark.parametrize("cfg_normalize", [False, True])
+def test_predict_noise_maybe_with_cfg_batched_equals_sequential(cfg_normalize):
+    """The reference's test of its mixin (tests/diffusion/distributed/test_cfg_parallel.py:293-372: batch 2,
+    4 channels, 16x16, width 128, scale 7.5, seeds 42/123, both settings of cfg_normalize) with the one-call
+    schedule in the place of the two-rank one; the sequential result is also checked against the formula."""
+    x_pos = torch.randn(2, 4, 16, 16, dtype=torch.float64, generator=torch.Generator().manual_seed(123))
+    x_neg = torch.randn(2, 4, 16, 16, dtype=torch.float64, generator=torch.Generator().manual_seed(124))
+    outs = []
+    for batched in (True, False):
+        pipe = _Pipe(batched)
+        calls = []
+        pipe.transformer.register_forward_hook(lambda m, a, kw, o: calls.append(kw["x"].shape[0]), with_kwargs=True)
+        with torch.no_grad():
+            outs.append(pipe.predict_noise_maybe_with_cfg(True, 7.5, {"x": x_pos}, {"x": x_neg}, cfg_normalize))
+        assert calls == ([4] if batched else [2, 2])
+    assert outs[0].shape == x_pos.shape
+    torch.testing.assert_close(outs[0], outs[1], atol=1e-12, rtol=1e-12)
+    with torch.no_grad():
+        p, n = pipe.transformer(x=x_pos)[0], pipe.transformer(x=x_neg)[0]
+    want = n + 7.5 * (p - n)
+    if cfg_normalize:
+        want = want * (p.norm(dim=-1, keepdim=True) / want.norm(dim=-1, keepdim=True))
+        torch.testing.assert_close(outs[1].norm(dim=-1), p.norm(dim=-1))
+    torch.testing.assert_close(outs[1], want, atol=1e-12, rtol=1e-12)
+
+
+def test_predict_noise_without_cfg():
+    """do_true_cfg = False: the positive prediction alone, one call, negative arguments untouched
+    (test_cfg_parallel.py:375-431), and output_slice keeps the leading positions of axis 1."""
+    pipe = _Pipe(True)
+    x = torch.randn(1, 4, 16, 16, dtype=torch.float64, generator=torch.Generator().manual_seed(123))
+    with torch.no_grad():
+        got = pipe.predict_noise_maybe_with_cfg(False, 7.5, {"x": x}, None)
+        want = pipe.transformer(x=x)[0]
+        cut = pipe.predict_noise_maybe_with_cfg(False, 7.5, {"x": x}, None, output_slice=3)
+    assert torch.equal(got, want) and torch.equal(cut, want[:, :3])
+
+
+def test_batch_cfg_kwargs_pads_and_masks_prompts():
+    lat = torch.randn(1, 6, 8)
+    pos = {"hidden_states": lat, "timestep": torch.tensor([0.5]), "guidance": None,
+           "encoder_hidden_states": torch.randn(1, 5, 3), "encoder_hidden_states_mask": None,
+           "img_shapes": [[(1, 2, 3)]], "txt_seq_lens": [5], "return_dict": False}
+    neg = dict(pos, encoder_hidden_states=torch.randn(1, 2, 3), txt_seq_lens=[2])
+    both = denoise.batch_cfg_kwargs(pos, neg)
+    assert both["hidden_states"].shape == (2, 6, 8) and torch.equal(both["hidden_states"][1], lat[0])
+    assert both["timestep"].tolist() == [0.5, 0.5] and both["guidance"] is None and both["return_dict"] is False
+    assert both["img_shapes"] == [[(1, 2, 3)], [(1, 2, 3)]] and both["txt_seq_lens"] == [5, 5]
+    text, mask = both["encoder_hidden_states"], both["encoder_hidden_states_mask"]
+    assert text.shape == (2, 5, 3) and torch.equal(text[1, :2], neg["encoder_hidden_states"][0])
+    assert torch.count_nonzero(text[1, 2:]) == 0
+    assert mask.tolist() == [[True] * 5, [True, True, False, False, False]]
+    # equal lengths and no masks: nothing to mask
+    same = denoise.batch_cfg_kwargs(pos, dict(pos))
+    assert same["encoder_hidden_states_mask"] is None and same["img_shapes"] == [[(1, 2, 3)]] * 2
+    # a given mask is kept and extended by the padding
+    neg_m = dict(neg, encoder_hidden_states_mask=torch.tensor([[1, 0]]))
+    assert denoise.batch_cfg_kwargs(pos, neg_m)["encoder_hidden_states_mask"][1].tolist() == [True, False, False, False, False]
+    # what cannot be stacked is left to two calls
+    assert denoise.batch_cfg_kwargs(pos, dict(pos, hidden_states=torch.randn(1, 7, 8))) is None
+    assert denoise.batch_cfg_kwargs(pos, dict(pos, return_dict=True)) is None
+    assert denoise.batch_cfg_kwargs(pos, {"hidden_states": lat}) is None
+
+
+def test_flow_match_scheduler_follows_the_sigma_table():
+    n, s_img = 9, 1024
+    sched = denoise.FlowMatchEulerScheduler()
+    sched.set_timesteps(sigmas=np.linspace(1.0, 1.0 / n, n), mu=denoise.calculate_shift(s_img))
+    sig = denoise.flow_match_sigmas(n, s_img)
+    np.testing.assert_allclose(sched.sigmas, sig, rtol=1e-6)
+    np.testing.assert_allclose(sched.timesteps.numpy(), sig[:-1] * 1000, rtol=1e-6)
+    x = torch.randn(1, 5, 4, generator=torch.Generator().manual_seed(2))
+    want = x.clone()
+    sched.set_begin_index(0)
+    for i, t in enumerate(sched.timesteps):
+        v = torch.full_like(x, float(i + 1))
+        x = sched.step(v, t, x, return_dict=False)[0]
+        want = want + (float(sig[i + 1]) - float(sig[i])) * v
+    torch.testing.assert_close(x, want)
+    # constant velocity: the steps telescope to x0 - sigma_0 v
+    sched.set_begin_index(0)
+    y = torch.zeros(3)
+    for t in sched.timesteps:
+        y = sched.step(torch.ones(3), t, y, return_dict=False)[0]
+    torch.testing.assert_close(y, torch.full((3,), -1.0))
+
+
+def test_qwen_mixin_diffuse_feeds_the_transformer_like_the_reference():
+    """Arguments per step (cfg_parallel.py:86-123 of the reference's qwen_image package): timestep / 1000 in
+    the latent dtype, latents joined with the image latents on axis 1 and the prediction cut back to the
+    latents' length, scheduler restarted at index 0."""
+    seen = []
+
+    class Net(torch.nn.Module):
+        def forward(self, hidden_states, timestep, encoder_hidden_states, **kw):
+            seen.append((hidden_states.shape, timestep.clone(), encoder_hidden_states.shape, kw))
+            return (hidden_states * 0 + encoder_hidden_states.mean(dim=(1, 2), keepdim=True),)
+
+    class Pipe(denoise.QwenImageCFGParallelMixin):
+        pass
+
+    pipe = Pipe()
+    pipe.transformer, pipe.scheduler = Net(), denoise.FlowMatchEulerScheduler()
+    pipe.scheduler.set_timesteps(3)
+    pipe.scheduler.set_begin_index(2)
+    lat, cond = torch.zeros(1, 4, 2), torch.ones(1, 3, 2)
+    pos, neg = torch.full((1, 5, 2), 2.0), torch.full((1, 2, 2), -1.0)
+    out = pipe.diffuse(pos, None, neg, None, lat, [[(1, 2, 2), (1, 1, 3)]], [5], [2], pipe.scheduler.timesteps,
+                       True, None, 2.0, image_latents=cond, cfg_normalize=False,
+                       additional_transformer_kwargs={"return_dict": False})
+    assert len(seen) == 3 and pipe.transformer.do_true_cfg is True
+    shape, t, tshape, kw = seen[0]
+    assert shape == (2, 7, 2) and tshape == (2, 5, 2) and t.tolist() == [1.0, 1.0]
+    assert kw["txt_seq_lens"] == [5, 5] and kw["return_dict"] is False and kw["guidance"] is None
+    assert kw["encoder_hidden_states_mask"].sum(dim=1).tolist() == [5, 2]
+    assert out.shape == lat.shape
+    # velocity per branch: mean of the (padded) prompt = 2 and -2/5; combined -0.4 + 2 * 2.4 = 4.4; sum of dsigma = -1
+    torch.testing.assert_close(out, torch.full_like(lat, -4.4))
