@@ -356,6 +356,43 @@ def kernel_rooflines(torch):
     return out
 
 
+def counter_probe(torch, kernels, dev):
+    """Three launches of each kernel of the path at the headline shapes on N(0,1) data, nothing else: short
+    enough for a hardware-counter pass (counters serialise the dispatches)."""
+    from vllm_omni_amd._lib import ODIT_NORM_HEAD
+
+    bf = torch.bfloat16
+    S = S_IMG + S_TXT
+    q = torch.randn(B, S, HEADS, HEAD_DIM, device=dev, dtype=bf)
+    k, v = torch.randn_like(q), torch.randn_like(q)
+    x = torch.randn(B, S_IMG, C, device=dev, dtype=bf)
+    y, o = torch.randn_like(x), torch.empty_like(x)
+    shift, scale, gate = torch.randn(B, 3 * C, device=dev, dtype=bf).chunk(3, dim=-1)
+    qkv = torch.randn(B, S_IMG, 3, HEADS, HEAD_DIM, device=dev, dtype=bf)
+    jq, jk = torch.empty_like(q), torch.empty_like(q)
+    w = torch.ones(HEAD_DIM, device=dev, dtype=bf)
+    cos, sin = torch.rand(S_IMG, HEAD_DIM // 2, device=dev), torch.rand(S_IMG, HEAD_DIM // 2, device=dev)
+    x2 = x.view(B * S_IMG, C)
+    w_up = torch.randn(MLP_RATIO * C, C, device=dev, dtype=bf) * 0.02
+    b_up = torch.zeros(MLP_RATIO * C, device=dev, dtype=bf)
+    w_qkv = torch.randn(3 * C, C, device=dev, dtype=bf) * 0.02
+    b_qkv = torch.zeros(3 * C, device=dev, dtype=bf)
+    for _ in range(3):
+        kernels.attn_fwd(q, k, v, 1.0 / math.sqrt(HEAD_DIM))
+        kernels.qknorm_rope(qkv[:, :, 0], qkv[:, :, 1], None, jq, jk, None, w, w, cos, sin, out_seq_offset=S_TXT,
+                            norm_mode=ODIT_NORM_HEAD)
+        kernels.adaln_modulate(x, shift, scale, out=o)
+        kernels.gated_residual(x, y, gate, out=o)
+        kernels.rel_l1_sums(x, y)
+        kernels.linear(x2, w_up, b_up, activation="gelu_tanh")
+        torch.nn.functional.linear(x2, w_qkv, b_qkv)
+    torch.cuda.synchronize()
+    print(json.dumps({"probe": "attention, qknorm+rope, adaLN, gated residual, rel-L1, MLP-up GEMM (GELU epilogue), "
+                               "QKV GEMM at the Qwen-Image shape, 3 launches each",
+                      "attention_flop": 4.0 * B * HEADS * S * S * HEAD_DIM,
+                      "mlp_up_flop": 2.0 * B * S_IMG * C * MLP_RATIO * C, "qkv_flop": 2.0 * B * S_IMG * C * 3 * C}))
+
+
 def mfma_ceiling(torch):
     """Sustained rate of the bf16 MFMA this path uses with nothing else in the loop, for constant and for
     random operand data (the part is power-limited: the two differ by about 30 %)."""
@@ -437,6 +474,9 @@ def main():
     ap.add_argument("--traffic-probe", action="store_true",
                     help="launch only the headline attention shape and a plain 512 MiB copy, a few times each: the "
                          "program to run under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`")
+    ap.add_argument("--counter-probe", action="store_true",
+                    help="launch each hand-written kernel and the two large GEMMs at the headline shapes three "
+                         "times: the program to run under `rocprofv3 --pmc <SQ counters>`")
     ap.add_argument("--unfused-epilogues", action="store_true",
                     help="A/B switch: GELU and gated residuals as separate kernels after plain GEMMs")
     ap.add_argument("--autotune", type=int, default=0,
@@ -474,6 +514,8 @@ def main():
         print(json.dumps({"probe": "attention B=2 S=4352 24x128 bf16 x4, copy 512 MiB x4",
                           "attention_min_bytes": 4 * q.numel() * 2, "copy_bytes_each_way": src.numel()}))
         return
+    if args.counter_probe:
+        return counter_probe(torch, kernels, dev)
     if args.workload != "qwen":
         return run_secondary(torch, kernels, args)
     model = build_model(torch, args.blocks, fuse_epilogues=not args.unfused_epilogues)
