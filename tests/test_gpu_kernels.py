@@ -243,6 +243,44 @@ def test_qknorm_rope_joint(gpu, dtype, H, D):
         assert (jq.cpu() == torch.cat(want_q_rr, 1)).float().mean().item() > 0.95
 
 
+def test_qknorm_rope_q_alone_and_offsets_beyond_31_bits(gpu):
+    """q without k, and the same inputs as views whose batch stride exceeds 2^31 elements (the kernel's 64-bit
+    indexing, which ordinary shapes never reach): identical bits to the compact call."""
+    from vllm_omni_amd import kernels
+    from vllm_omni_amd._lib import ODIT_NORM_HEAD
+
+    B, S, H, D, off = 2, 37, 3, 128, 5
+    dtype = torch.bfloat16
+    qkv = _rand(B, S, 3, H, D, seed=31, dtype=dtype).to(gpu)
+    w = (_rand(D, seed=32, dtype=torch.float32) * 0.2 + 1).to(dtype).to(gpu)
+    cos, sin = (t.to(gpu) for t in _cos_sin(S, D // 2, seed=33))
+
+    def run(q, k, v):
+        outs = [torch.zeros(B, S + off, H, D, dtype=dtype, device=gpu) if t is not None else None for t in (q, k, v)]
+        kernels.qknorm_rope(q, k, v, outs[0], outs[1], outs[2], w, w, cos, sin, eps=1e-6, out_seq_offset=off,
+                            norm_mode=ODIT_NORM_HEAD)
+        return outs
+
+    q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+    full = run(q, k, v)
+    want_q = ops.apply_rotary(ops.rms_norm_head(q.float().cpu(), w.float().cpu()), cos.cpu(), sin.cpu())
+    _close(full[0][:, off:], want_q, atol=2e-2, rtol=2e-2, what="q of the q+k+v call")
+    alone = run(q, None, None)
+    assert torch.equal(alone[0], full[0])
+    pair = run(q, k, None)
+    assert torch.equal(pair[0], full[0]) and torch.equal(pair[1], full[1])
+    # batch stride 2^31 + 4096 elements: one 4.3 GB buffer holding both batch rows far apart
+    row = S * 3 * H * D
+    stride_b = (1 << 31) + 4096
+    big = torch.empty(stride_b + row, dtype=dtype, device=gpu)
+    far = torch.as_strided(big, (B, S, 3, H, D), (stride_b, 3 * H * D, H * D, D, 1))
+    far.copy_(qkv)
+    got = run(far[:, :, 0], far[:, :, 1], far[:, :, 2])
+    del big, far
+    for a, b, name in zip(got, full, "qkv"):
+        assert torch.equal(a, b), name
+
+
 def test_rotary_layer_and_neox_and_partial(gpu):
     from vllm_omni_amd.layers.rope import RotaryEmbedding
 

@@ -13,6 +13,8 @@
 // (token, part) holding the row in registers, reduced across the wavefront.
 // Interleaved rotary pairs (2i, 2i+1) live inside one lane's vector; NeoX pairs are fetched from the
 // lane rot/(2*EPV) away with a shuffle.
+#include <type_traits>
+
 #include "odit_common.h"
 
 namespace odit {
@@ -118,9 +120,27 @@ template <typename T> __device__ __forceinline__ u32x4 pack_vec(const float (&x)
   return o;
 }
 
+// Division of n < 2^31 by a launch constant d as one multiply-high and a shift: with l = ceil(log2 d) >= 1
+// and mul = ceil(2^(31+l) / d) < 2^32, floor(n * mul / 2^(31+l)) = floor(n / d) exactly (the excess
+// n * (mul - 2^(31+l)/d) / 2^(31+l) stays below 2^-l <= 1/d). d = 1 is the identity (mul = 0 marks it).
+struct FastDiv {
+  uint32_t mul, shift;
+  static FastDiv make(uint32_t d) {
+    if (d <= 1) return {0u, 0u};
+    uint32_t l = 1;
+    while ((1ull << l) < d) ++l;
+    const uint64_t p2 = 1ull << (31 + l);
+    return {static_cast<uint32_t>((p2 + d - 1) / d), l - 1};
+  }
+  __device__ __forceinline__ uint32_t div(uint32_t n) const {
+    return mul == 0u ? n : (__umulhi(n, mul) >> shift);
+  }
+};
+
 // ---- per-head (or no) statistics: one vector per lane, grid (vectors / 256, parts) ---------------
-// IDX32: vector and token numbers fit 32 bits (every launch short of 2^31 vectors), which spares each
-// lane two 64-bit integer divisions.
+// IDX32: vector numbers, token numbers and element offsets fit 31 bits: the two divisions per lane (by
+// vectors per row, by tokens per batch row) become a multiply-high and a shift each and the addresses are a
+// base pointer plus a 32-bit offset.
 template <typename T, typename TW, int NORM_MODE, bool GENERAL, bool IDX32>
 __global__ __launch_bounds__(256) void qknorm_flat_kernel(
     const T* __restrict__ q_in, const T* __restrict__ k_in, const T* __restrict__ v_in,
@@ -128,20 +148,21 @@ __global__ __launch_bounds__(256) void qknorm_flat_kernel(
     const TW* __restrict__ wq, const TW* __restrict__ wk, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, int S, int HD, int D, int rot, int64_t is_b, int64_t is_s,
     int out_seq_offset, int S_total, float eps, int vec_per_row, int64_t total_vec, bool neox,
-    bool ref_round) {
+    bool ref_round, FastDiv by_vpr, FastDiv by_s, float inv_d) {
   constexpr int EPV = Vec16<T>::N;
   const int lane = threadIdx.x & 63;
-  // part: 0 = q, 1 = k, 2 = v (k and v may be absent)
-  const int kind = blockIdx.y == 0 ? 0 : (blockIdx.y == 1 && k_in != nullptr ? 1 : 2);
+  // grid.y: 0 = q together with k (when there is one), 1 = the copy of v. A lane takes the SAME vector
+  // position of q and of k: one index computation, one pair of cos/sin loads, two loads in flight.
+  const bool copy_v = blockIdx.y != 0;
   const int64_t i_raw = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   const bool valid = i_raw < total_vec;
   const int64_t i = valid ? i_raw : total_vec - 1;  // clamped lanes compute, never store
   int e0, b, s;
   if constexpr (IDX32) {
     const unsigned iu = static_cast<unsigned>(i), vpr = static_cast<unsigned>(vec_per_row);
-    const unsigned tok = iu / vpr;
+    const unsigned tok = by_vpr.div(iu);
     e0 = static_cast<int>(iu - tok * vpr) * EPV;
-    b = static_cast<int>(tok / static_cast<unsigned>(S));
+    b = static_cast<int>(by_s.div(tok));
     s = static_cast<int>(tok - static_cast<unsigned>(b) * static_cast<unsigned>(S));
   } else {
     const int64_t tok = i / vec_per_row;
@@ -149,41 +170,58 @@ __global__ __launch_bounds__(256) void qknorm_flat_kernel(
     b = static_cast<int>(tok / S);
     s = static_cast<int>(tok - static_cast<int64_t>(b) * S);
   }
-  const int64_t in_off = b * is_b + s * is_s + e0;
-  const int64_t out_off = (static_cast<int64_t>(b) * S_total + out_seq_offset + s) * HD + e0;
-  if (kind == 2) {  // block-uniform
+  // IDX32 also means that every element offset below fits 31 bits (checked by the launcher)
+  using off_t = typename std::conditional<IDX32, unsigned, int64_t>::type;
+  const off_t in_off = static_cast<off_t>(b) * static_cast<off_t>(is_b) + static_cast<off_t>(s) * static_cast<off_t>(is_s) +
+                       static_cast<off_t>(e0);
+  const off_t out_off = (static_cast<off_t>(b) * static_cast<off_t>(S_total) + static_cast<off_t>(out_seq_offset + s)) *
+                            static_cast<off_t>(HD) + static_cast<off_t>(e0);
+  if (copy_v) {  // block-uniform
     const u32x4 r = load_raw(v_in + in_off);
     if (valid) __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(v_out + out_off));
     return;
   }
-  const u32x4 r = load_raw((kind == 0 ? q_in : k_in) + in_off);
-  float x[EPV];
+  const bool has_k = k_in != nullptr;  // launch-uniform
+  const u32x4 rq = load_raw(q_in + in_off);
+  const u32x4 rk = has_k ? load_raw(k_in + in_off) : u32x4{0u, 0u, 0u, 0u};
+  float xq[EPV], xk[EPV];
 #pragma unroll
-  for (int j = 0; j < EPV; ++j) x[j] = Raw<T>::get(r, j);
+  for (int j = 0; j < EPV; ++j) { xq[j] = Raw<T>::get(rq, j); xk[j] = Raw<T>::get(rk, j); }
   const int d0 = (D & (D - 1)) == 0 ? (e0 & (D - 1)) : e0 % D;  // head sizes are powers of two in practice
-  float rstd = 1.f;
+  float rstd_q = 1.f, rstd_k = 1.f;
   if constexpr (NORM_MODE == ODIT_NORM_HEAD) {
-    float sq = 0.f;
+    float sq = 0.f, sk = 0.f;
 #pragma unroll
-    for (int j = 0; j < EPV; ++j) sq = fmaf(x[j], x[j], sq);
+    for (int j = 0; j < EPV; ++j) { sq = fmaf(xq[j], xq[j], sq); sk = fmaf(xk[j], xk[j], sk); }
     switch (D / EPV) {  // lanes per head row: wave-uniform
-      case 64: sq = group_sum<64>(sq); break;
-      case 32: sq = group_sum<32>(sq); break;
-      case 16: sq = group_sum<16>(sq); break;
-      case 8: sq = group_sum<8>(sq); break;
-      case 4: sq = group_sum<4>(sq); break;
-      case 2: sq = group_sum<2>(sq); break;
+      case 64: sq = group_sum<64>(sq); sk = group_sum<64>(sk); break;
+      case 32: sq = group_sum<32>(sq); sk = group_sum<32>(sk); break;
+      case 16: sq = group_sum<16>(sq); sk = group_sum<16>(sk); break;
+      case 8: sq = group_sum<8>(sq); sk = group_sum<8>(sk); break;
+      case 4: sq = group_sum<4>(sq); sk = group_sum<4>(sk); break;
+      case 2: sq = group_sum<2>(sq); sk = group_sum<2>(sk); break;
       default: break;
     }
-    rstd = rsqrtf(sq / static_cast<float>(D) + eps);
+    // a power-of-two head size divides exactly as a multiplication; any other keeps the division's rounding
+    if ((D & (D - 1)) == 0) {  // launch-uniform
+      rstd_q = rsqrtf(sq * inv_d + eps);
+      rstd_k = rsqrtf(sk * inv_d + eps);
+    } else {
+      rstd_q = rsqrtf(sq / static_cast<float>(D) + eps);
+      rstd_k = rsqrtf(sk / static_cast<float>(D) + eps);
+    }
   }
-  const TW* w = kind == 0 ? wq : wk;
   const float* cr = cos_t ? cos_t + static_cast<int64_t>(s) * (rot >> 1) : nullptr;
   const float* sr = sin_t ? sin_t + static_cast<int64_t>(s) * (rot >> 1) : nullptr;
-  transform_vec<T, TW, NORM_MODE != ODIT_NORM_NONE, true, GENERAL>(x, rstd, w ? w + d0 : nullptr, cr, sr, d0,
+  transform_vec<T, TW, NORM_MODE != ODIT_NORM_NONE, true, GENERAL>(xq, rstd_q, wq ? wq + d0 : nullptr, cr, sr, d0,
                                                                    rot, true, lane, neox, ref_round);
-  if (valid)
-    __builtin_nontemporal_store(pack_vec<T>(x), reinterpret_cast<u32x4*>((kind == 0 ? q_out : k_out) + out_off));
+  if (has_k)
+    transform_vec<T, TW, NORM_MODE != ODIT_NORM_NONE, true, GENERAL>(xk, rstd_k, wk ? wk + d0 : nullptr, cr, sr, d0,
+                                                                     rot, true, lane, neox, ref_round);
+  if (valid) {
+    __builtin_nontemporal_store(pack_vec<T>(xq), reinterpret_cast<u32x4*>(q_out + out_off));
+    if (has_k) __builtin_nontemporal_store(pack_vec<T>(xk), reinterpret_cast<u32x4*>(k_out + out_off));
+  }
 }
 
 // ---- whole-row statistics: one wavefront per (token, part), row held in registers ---------------
@@ -274,7 +312,7 @@ template <typename T, typename TW, int NORM_MODE, bool GENERAL> static int qk_fl
   constexpr int EPV = Vec16<T>::N;
   const int vpr = a.HD / EPV;
   const int64_t total = static_cast<int64_t>(a.B) * a.S * vpr;
-  const int nparts = 1 + (a.k_in != nullptr) + (a.v_in != nullptr);
+  const int nparts = 1 + (a.v_in != nullptr);  // q (with k) | v
   const dim3 grid(static_cast<unsigned>((total + 255) / 256), nparts);
 #define ODIT_QK_FLAT(I32)                                                                          \
   hipLaunchKernelGGL((qknorm_flat_kernel<T, TW, NORM_MODE, GENERAL, I32>), grid, dim3(256), 0, a.stream, \
@@ -282,8 +320,13 @@ template <typename T, typename TW, int NORM_MODE, bool GENERAL> static int qk_fl
                      static_cast<const T*>(a.v_in), static_cast<T*>(a.q_out), static_cast<T*>(a.k_out), \
                      static_cast<T*>(a.v_out), static_cast<const TW*>(a.wq), static_cast<const TW*>(a.wk), \
                      a.cos, a.sin, a.S, a.HD, a.D, a.rot, a.is_b, a.is_s, a.out_seq_offset, a.S_total, \
-                     a.eps, vpr, total, a.neox, a.ref_round)
-  if (total < (1ll << 31)) ODIT_QK_FLAT(true); else ODIT_QK_FLAT(false);
+                     a.eps, vpr, total, a.neox, a.ref_round, FastDiv::make(static_cast<uint32_t>(vpr)), \
+                     FastDiv::make(static_cast<uint32_t>(a.S)), 1.f / static_cast<float>(a.D))
+  // 32-bit indexing: vector numbers and every element offset of the inputs and of the joint outputs below 2^31
+  const int64_t in_span = (a.B - 1) * a.is_b + (a.S - 1) * a.is_s + a.HD;
+  const int64_t out_span = static_cast<int64_t>(a.B) * a.S_total * a.HD;
+  const bool idx32 = total < (1ll << 31) && in_span < (1ll << 31) && out_span < (1ll << 31) && a.is_b >= 0 && a.is_s >= 0;
+  if (idx32) ODIT_QK_FLAT(true); else ODIT_QK_FLAT(false);
 #undef ODIT_QK_FLAT
   return check_launch("odit_qknorm_rope");
 }
