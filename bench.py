@@ -29,6 +29,12 @@ PEAK_HBM_GBS = 8000.0            # MI355X HBM3E, vendor figure
 # (FETCH_SIZE x2.0, WRITE_SIZE x1.0). One call = three launches: the full units (203.7 MB fetched + 51.9 MB
 # written), the key ranges of the last round (74.0 + 36.4 MB) and their merge (33.5 + 3.1 MB).
 ATTN_TRAFFIC_BYTES = 402.6e6
+# Matrix-pipe counters of the attention main launch at the headline shape, from a rocprofv3 SQ-counter pass over
+# `bench.py --counter-probe` (not measured live): share of the launch's cycles with the MFMA pipe busy
+# (SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE / 8 x 1024 SIMDs)) and the clock those cycles ran at
+# (GRBM_GUI_ACTIVE / 8 / duration); the nominal peak assumes 2400 MHz.
+ATTN_MFMA_BUSY_FRAC = 0.560
+ATTN_CLOCK_MHZ = 1771.0
 
 # Qwen-Image shape at 1024x1024 (BASELINE.json configs[2])
 LAYERS, HEADS, HEAD_DIM, MLP_RATIO = 60, 24, 128, 4
@@ -579,6 +585,8 @@ def main():
                      "achieved": attn_tflops, "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": attn_tflops / PEAK_MFMA_BF16_TFLOPS,
                      "traffic": ATTN_TRAFFIC_BYTES if args.blocks == LAYERS else None,
+                     "counters": {"mfma_busy_frac_of_cycles": ATTN_MFMA_BUSY_FRAC, "clock_MHz_in_kernel": ATTN_CLOCK_MHZ,
+                                  "source": "rocprofv3 --pmc pass over bench.py --counter-probe, not live"},
                      "launches_timed": n_attn, "avg_ms": attn_ms, "flop_per_launch": attn_flop},
         "step_flop": None,
     }
