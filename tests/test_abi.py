@@ -84,3 +84,48 @@ def test_wrappers_refuse_cpu_tensors():
         kernels.adaln_modulate(x, None, None)
     with pytest.raises(RuntimeError, match="GPU"):
         kernels.gelu_tanh(x)
+
+
+def test_product_code_never_reaches_the_oracle():
+    """The oracle is test infrastructure: nothing in the package, and in bench.py / __graft_entry__.py only the
+    CPU-baseline leg and smoke(), may import it (checked on the syntax trees, so comments do not count)."""
+    import ast
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parents[1]
+
+    def oracle_imports(path):
+        found = []
+        for node in ast.walk(ast.parse(path.read_text())):
+            names = []
+            if isinstance(node, ast.Import):
+                names = [a.name for a in node.names]
+            elif isinstance(node, ast.ImportFrom):
+                names = [node.module or ""]
+            found += [(node.lineno, n) for n in names if n == "oracle" or n.startswith("oracle.")]
+        return found
+
+    package = {p.resolve() for p in root.iterdir() if p.is_dir() and (p / "kernels.py").exists()}  # dir + its import alias
+    assert len(package) == 1
+    for path in package.pop().rglob("*.py"):
+        assert oracle_imports(path) == [], path
+    allowed = {"bench.py": "cpu_baseline", "__graft_entry__.py": "smoke"}
+    for name, func in allowed.items():
+        tree = ast.parse((root / name).read_text())
+        inside = set()
+        for node in ast.walk(tree):
+            if isinstance(node, ast.FunctionDef) and node.name == func:
+                inside = {n.lineno for n in ast.walk(node) if isinstance(n, (ast.Import, ast.ImportFrom))}
+        for lineno, _ in oracle_imports(root / name):
+            assert lineno in inside, f"{name}:{lineno} imports the oracle outside {func}()"
+
+
+def test_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "libomni_dit_hip.so")
+    monkeypatch.setattr(_lib, "_lib", None)
+    with pytest.raises(_lib.OmniDitLibraryError, match="no fallback"):
+        _lib.load()
+    from vllm_omni_amd import kernels
+
+    with pytest.raises(_lib.OmniDitLibraryError):
+        kernels.attn_workspace_bytes(1, 128, 128, 1, 128) if hasattr(kernels, "attn_workspace_bytes") else _lib.load()
