@@ -388,6 +388,34 @@ def test_attention_parity(gpu, monkeypatch, variant, shape):
     _close(lse, torch.logsumexp(s, dim=-1), atol=2e-2, rtol=1e-3, what="lse")
 
 
+@pytest.mark.parametrize("variant", ["34", "38", "28"])
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("order", ["rising", "falling", "random"])
+def test_attention_peaked_logits(gpu, monkeypatch, variant, D, order):
+    """Logits with a standard deviation of about 16 and a row maximum that keeps rising (or falling) from one key
+    tile to the next: the running-maximum update, the rescaling of the accumulators that is skipped while the
+    maximum grows by less than 2^8, and probabilities that underflow to zero, against an fp64 softmax."""
+    from vllm_omni_amd import kernels
+
+    monkeypatch.setenv("ODIT_ATTN_VARIANT", variant)
+    B, Sq, Sk, H = 1, 200, 700, 2
+    q, k, v = _attn_inputs(B, Sq, Sk, H, H, D, seed=77)
+    ramp = torch.linspace(0.5, 7.5, Sk).view(1, Sk, 1, 1)
+    if order == "falling":
+        ramp = ramp.flip(1)
+    elif order == "random":
+        ramp = ramp[:, torch.randperm(Sk, generator=torch.Generator().manual_seed(5))]
+    k = (k.float() * ramp).bfloat16()
+    q = (q.float() * 4.0).bfloat16()
+    scale = 1.0 / math.sqrt(D)
+    got, lse = kernels.attn_fwd(q.to(gpu), k.to(gpu), v.to(gpu), scale, return_lse=True)
+    s = torch.einsum("bqhd,bkhd->bhqk", q.double(), k.double()) * scale
+    assert s.std() > 10 and s.max() > 80            # far outside what N(0,1) inputs reach
+    want = torch.einsum("bhqk,bkhd->bqhd", torch.softmax(s, dim=-1), v.double())
+    _close(got, want.float(), atol=2e-2, rtol=2e-2, what=f"peaked attention ({order})")
+    _close(lse, torch.logsumexp(s, dim=-1).float(), atol=2e-2, rtol=1e-3, what="lse")
+
+
 def test_attention_fp16_and_strided_views(gpu):
     from vllm_omni_amd import kernels
 
@@ -503,6 +531,15 @@ def test_attention_key_split_tail(gpu, monkeypatch, variant, shape):
         cut = Sq // 3
         head, tail = kernels.attn_fwd(qg, kg, vg, scale, split=cut)
         assert torch.equal(head, two[:, :cut]) and torch.equal(tail, two[:, cut:])
+    # peaked logits whose row maximum rises along the keys: the last key range outweighs the others by far
+    # more than 2^126, so the merge has to take weights of exactly zero without producing NaN
+    ramp = torch.linspace(0.5, 7.5, Sk).view(1, Sk, 1, 1)
+    kp, qp = (k.float() * ramp).bfloat16(), (q.float() * 4.0).bfloat16()
+    sp = torch.einsum("bqhd,bkhd->bhqk", qp.double(), kp.double().repeat_interleave(H // Hkv, dim=2)) * scale
+    wantp = torch.einsum("bhqk,bkhd->bqhd", torch.softmax(sp, dim=-1), v.double().repeat_interleave(H // Hkv, dim=2))
+    gotp, lsep = kernels.attn_fwd(qp.to(gpu), kp.to(gpu), vg, scale, return_lse=True)
+    _close(gotp, wantp.float(), atol=2e-2, rtol=2e-2, what="key-split, peaked logits")
+    _close(lsep, torch.logsumexp(sp, dim=-1).float(), atol=2e-2, rtol=1e-3, what="key-split, peaked logits, lse")
 
 
 @pytest.mark.parametrize("variant", ["34", "38", "28"])
