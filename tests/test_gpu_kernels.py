@@ -64,6 +64,39 @@ def test_adaln_modulate(gpu, dtype, B, S, C):
         assert frac_equal > 0.97, f"only {frac_equal:.3f} of elements bit-identical"
 
 
+@pytest.mark.parametrize("C", [3072, 5120, 1000])
+def test_adaln_ill_conditioned_rows(gpu, C):
+    """Rows where a one-pass variance is at risk, in float32 against a float64 LayerNorm: a mean 600 times the
+    standard deviation, constant rows (variance exactly zero: the output is the shift), one outlier channel of
+    1e4 among unit-scale values, and a row of values near 1e-3."""
+    from vllm_omni_amd import kernels
+
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(1, 6, C, generator=g)
+    x[0, 0] = 300.0 + 0.5 * x[0, 0]
+    x[0, 1] = 7.25
+    x[0, 2] = 0.0
+    x[0, 3, C // 3] = 1.0e4
+    x[0, 4] = 1.0e-3 * x[0, 4]
+    shift, scale = 0.3 * torch.randn(1, C, generator=g), 0.3 * torch.randn(1, C, generator=g)
+    want = torch.nn.functional.layer_norm(x.double(), (C,), eps=1e-6) * (1 + scale.double()[:, None]) + shift.double()[:, None]
+    got = kernels.adaln_modulate(x.to(gpu), shift.to(gpu), scale.to(gpu)).cpu()
+    assert torch.isfinite(got).all()
+    assert torch.equal(got[0, 1], shift[0]) and torch.equal(got[0, 2], shift[0])
+    for r, tol in ((0, 2e-4), (3, 1e-4), (4, 1e-4), (5, 1e-5)):
+        err = (got[0, r].double() - want[0, r]).abs().max().item()
+        assert err <= tol * max(1.0, want[0, r].abs().max().item()), (r, err)
+    # the same rows in bf16 (the mean-300 row then carries 2^-8 * 300 of input rounding: checked against the
+    # LayerNorm of the ROUNDED input)
+    xb = x.bfloat16()
+    wantb = torch.nn.functional.layer_norm(xb.double(), (C,), eps=1e-6) * (1 + scale.bfloat16().double()[:, None]) \
+        + shift.bfloat16().double()[:, None]
+    gotb = kernels.adaln_modulate(xb.to(gpu), shift.bfloat16().to(gpu), scale.bfloat16().to(gpu)).cpu()
+    assert torch.isfinite(gotb.float()).all()
+    rel = (gotb.double() - wantb).abs() / (wantb.abs() + 1.0)
+    assert rel.max().item() <= 2 ** -7, rel.max().item()
+
+
 def test_adaln_index_fp32_params_affine_and_strides(gpu):
     from vllm_omni_amd import kernels
 
