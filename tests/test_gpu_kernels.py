@@ -492,6 +492,12 @@ def test_attention_key_mask_equals_deleting_keys(gpu, monkeypatch, variant):
         got3 = kernels.attn_fwd(q2.to(gpu), k2.to(gpu), v2.to(gpu), 0.125, key_mask=m3.to(gpu))
         _close(got3, ops.sdpa(q2.float(), k2.float(), v2.float(), 0.125, key_mask=m3), atol=2e-2, rtol=2e-2,
                what=f"mask S={S2} cut={cut[:3]}")
+    # a batch row with every key excluded returns zeros (and a log-sum-exp of -inf); the other row is untouched
+    m4 = torch.ones(B, S, dtype=torch.bool)
+    m4[1] = False
+    got4, lse4 = kernels.attn_fwd(q.to(gpu), k.to(gpu), v.to(gpu), 0.125, key_mask=m4.to(gpu), return_lse=True)
+    assert torch.count_nonzero(got4[1]) == 0 and bool(torch.isneginf(lse4[1]).all())
+    assert torch.equal(got4[0].cpu(), layer(q.to(gpu), k.to(gpu), v.to(gpu))[0].cpu())
     # an all-true mask is dropped and gives the unmasked result bit for bit
     ones = AttentionMetadata(attn_mask=torch.ones(B, S, dtype=torch.bool, device=gpu))
     assert torch.equal(layer(q.to(gpu), k.to(gpu), v.to(gpu), ones).cpu(),
@@ -560,6 +566,9 @@ def test_attention_key_split_tail(gpu, monkeypatch, variant, shape):
     got_m = kernels.attn_fwd(qg, kg, vg, scale, key_mask=m.to(gpu))
     _close(got_m, ops.sdpa(q.float(), k.float(), v.float(), scale, key_mask=m), atol=2e-2, rtol=2e-2,
            what="key-split with mask")
+    none = torch.zeros(B, Sk, dtype=torch.bool, device=gpu)
+    got0, lse0 = kernels.attn_fwd(qg, kg, vg, scale, key_mask=none, return_lse=True)
+    assert torch.count_nonzero(got0) == 0 and bool(torch.isneginf(lse0).all()), "every key excluded: zeros"
     if Sq > 2:
         cut = Sq // 3
         head, tail = kernels.attn_fwd(qg, kg, vg, scale, split=cut)
