@@ -90,10 +90,16 @@ static hipDataType lin_type(int dtype) {
   return dtype == ODIT_BF16 ? HIP_R_16BF : (dtype == ODIT_F16 ? HIP_R_16F : HIP_R_32F);
 }
 
-static int lin_plan(hipblasLtHandle_t h, const LinKey& key, LinPlan** out) {
-  auto it = g_lin.plans.find(key);
-  if (it != g_lin.plans.end()) { *out = &it->second; return ODIT_OK; }
-  LinPlan p;
+static void lin_plan_release(LinPlan& p) {
+  if (p.a) hipblasLtMatrixLayoutDestroy(p.a);
+  if (p.b) hipblasLtMatrixLayoutDestroy(p.b);
+  if (p.c) hipblasLtMatrixLayoutDestroy(p.c);
+  if (p.d) hipblasLtMatrixLayoutDestroy(p.d);
+  if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
+  p = LinPlan{};
+}
+
+static int lin_plan_build(const LinKey& key, LinPlan& p) {
   const hipDataType t = lin_type(key.dtype);
   ODIT_LT(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
   const int32_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
@@ -119,6 +125,18 @@ static int lin_plan(hipblasLtHandle_t h, const LinKey& key, LinPlan** out) {
   ODIT_LT(hipblasLtMatrixLayoutCreate(&p.b, t, key.k, key.m, key.ldb));
   ODIT_LT(hipblasLtMatrixLayoutCreate(&p.c, t, key.n, key.m, key.ldc));
   ODIT_LT(hipblasLtMatrixLayoutCreate(&p.d, t, key.n, key.m, key.ldd));
+  return ODIT_OK;
+}
+
+static int lin_plan(const LinKey& key, LinPlan** out) {
+  auto it = g_lin.plans.find(key);
+  if (it != g_lin.plans.end()) { *out = &it->second; return ODIT_OK; }
+  LinPlan p;
+  const int rc = lin_plan_build(key, p);
+  if (rc != ODIT_OK) {  // nothing half-built stays behind
+    lin_plan_release(p);
+    return rc;
+  }
   auto ins = g_lin.plans.emplace(key, p);
   *out = &ins.first->second;
   return ODIT_OK;
@@ -159,7 +177,7 @@ static int lin_prepare(const LinCall& c, hipblasLtHandle_t* h, LinPlan** plan, c
   const bool has_bias = c.bias != nullptr;
   LinKey key{dev, c.M, c.N, c.K, c.epilogue * 4 + (has_bias ? 1 : 0) + (alpha_vec ? 2 : 0), c.dtype,
              c.ldw, c.ldx, gated ? c.ldr : c.ldo, c.ldo};
-  rc = lin_plan(*h, key, plan);
+  rc = lin_plan(key, plan);
   if (rc != ODIT_OK) return rc;
   const size_t gb = lin_gate_bytes(c);
   if (gb > c.ws_bytes) {
