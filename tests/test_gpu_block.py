@@ -368,6 +368,9 @@ def test_weights_loaded_after_fusing_are_used(gpu):
 def test_cfg_batched_equals_sequential(gpu):
     cfg, w, model = _build(gpu)
     lat, _, _ = _inputs(1, seed=5)
+    with pytest.raises(TypeError, match="guidance"):   # as in the reference, whose time embedding takes none
+        model(lat.to(gpu), torch.zeros(1, S_TXT, 256, device=gpu).bfloat16(), None, torch.ones(1, device=gpu),
+              [IMG_SHAPE], [S_TXT], guidance=torch.ones(1, device=gpu))
     g = torch.Generator().manual_seed(6)
     text = torch.randn(2, S_TXT, 256, generator=g).bfloat16().to(gpu)
     t = torch.tensor([0.7, 0.7]).bfloat16().to(gpu)

@@ -562,6 +562,10 @@ class QwenImageTransformer2DModel(nn.Module):
                 encoder_hidden_states_mask: torch.Tensor = None, timestep: torch.Tensor = None,
                 img_shapes=None, txt_seq_lens=None, guidance: torch.Tensor = None,
                 attention_kwargs: dict[str, Any] | None = None, additional_t_cond=None, return_dict: bool = True):
+        if guidance is not None:
+            # the reference forwards it to a time embedding whose forward has no such argument (qit.py:169,
+            # 1017-1024) and fails there; no Qwen-Image checkpoint sets guidance_embeds
+            raise TypeError("QwenImageTransformer2DModel: the timestep embedding takes no guidance; pass guidance=None")
         img, txt, temb, rotary = self.prepare(hidden_states, encoder_hidden_states, timestep, img_shapes, txt_seq_lens,
                                               additional_t_cond)
         index = self.modulate_index(img_shapes, img.device)

@@ -64,6 +64,8 @@ def extract_qwen_context(module: nn.Module, hidden_states: torch.Tensor,
         # the reference's extractor passes no per-token index to the blocks either (extractors.py:245-254):
         # an editing model under it would silently be modulated wrongly, so refuse instead
         raise NotImplementedError("TeaCache has no extractor for the zero_cond_t (editing) variant")
+    if guidance is not None:  # the reference hands it to a time embedding that takes none (extractors.py:199-203)
+        raise TypeError("extract_qwen_context: the timestep embedding takes no guidance; pass guidance=None")
     img, txt, temb, rotary = module.prepare(hidden_states, encoder_hidden_states, timestep, img_shapes, txt_seq_lens,
                                             additional_t_cond)
     block0 = module.transformer_blocks[0]
