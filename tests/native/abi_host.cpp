@@ -1,0 +1,184 @@
+// A host program with no Python and no torch in it: it links libomni_dit_hip.so through include/omni_dit.h,
+// owns its device buffers through the HIP runtime, and checks three entry points against loops written here
+// (double precision on the CPU). It is what a non-Python caller of the C ABI looks like; the GPU test
+// tests/test_gpu_native_host.py runs it as a child process and reads its exit status.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+#include "omni_dit.h"
+
+#define HIP_OK(call)                                                                          \
+  do {                                                                                        \
+    const hipError_t e__ = (call);                                                            \
+    if (e__ != hipSuccess) {                                                                  \
+      std::fprintf(stderr, "%s failed: %s\n", #call, hipGetErrorString(e__));                 \
+      return 2;                                                                               \
+    }                                                                                         \
+  } while (0)
+#define ODIT_OK_OR_FAIL(call)                                                                 \
+  do {                                                                                        \
+    const int rc__ = (call);                                                                  \
+    if (rc__ != 0) {                                                                          \
+      std::fprintf(stderr, "%s returned %d: %s\n", #call, rc__, odit_last_error());           \
+      return 3;                                                                               \
+    }                                                                                         \
+  } while (0)
+
+static uint32_t g_state = 12345u;
+static float next_uniform() {  // (-1, 1), same sequence on every run
+  g_state = g_state * 1664525u + 1013904223u;
+  return static_cast<float>(g_state >> 8) * (2.0f / 16777216.0f) - 1.0f;
+}
+static uint16_t to_bf16(float f) {  // round to nearest even
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return static_cast<uint16_t>(u >> 16);
+}
+static float from_bf16(uint16_t h) {
+  const uint32_t u = static_cast<uint32_t>(h) << 16;
+  float f;
+  std::memcpy(&f, &u, 4);
+  return f;
+}
+
+template <typename T> struct DeviceBuffer {
+  T* p = nullptr;
+  ~DeviceBuffer() { if (p) (void)hipFree(p); }
+  hipError_t alloc(size_t n) { return hipMalloc(reinterpret_cast<void**>(&p), n * sizeof(T)); }
+};
+
+static int check_rel_l1(hipStream_t st) {
+  const int B = 2;
+  const int64_t n = 5000;  // not a multiple of the vector width
+  std::vector<uint16_t> cur(B * n), prev(B * n);
+  for (auto& v : cur) v = to_bf16(next_uniform());
+  for (auto& v : prev) v = to_bf16(next_uniform());
+  DeviceBuffer<uint16_t> d_cur, d_prev;
+  DeviceBuffer<double> d_sums;
+  DeviceBuffer<char> d_ws;
+  const size_t ws = odit_rel_l1_workspace_bytes(B, n);
+  HIP_OK(d_cur.alloc(cur.size())); HIP_OK(d_prev.alloc(prev.size())); HIP_OK(d_sums.alloc(2 * B));
+  HIP_OK(d_ws.alloc(ws > 0 ? ws : 16));
+  HIP_OK(hipMemcpy(d_cur.p, cur.data(), cur.size() * 2, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_prev.p, prev.data(), prev.size() * 2, hipMemcpyHostToDevice));
+  ODIT_OK_OR_FAIL(odit_rel_l1(d_cur.p, d_prev.p, d_sums.p, d_ws.p, ws, B, n, n, n, ODIT_BF16, 0, st));
+  HIP_OK(hipStreamSynchronize(st));
+  double got[4];
+  HIP_OK(hipMemcpy(got, d_sums.p, sizeof(got), hipMemcpyDeviceToHost));
+  for (int b = 0; b < B; ++b) {
+    double sd = 0.0, sp = 0.0;
+    for (int64_t i = 0; i < n; ++i) {
+      const double c = from_bf16(cur[b * n + i]), p = from_bf16(prev[b * n + i]);
+      sd += std::fabs(c - p);
+      sp += std::fabs(p);
+    }
+    if (std::fabs(got[2 * b] - sd) > 1e-5 * sd || std::fabs(got[2 * b + 1] - sp) > 1e-5 * sp) {
+      std::fprintf(stderr, "rel_l1 row %d: got (%.9g, %.9g), want (%.9g, %.9g)\n", b, got[2 * b], got[2 * b + 1], sd, sp);
+      return 1;
+    }
+  }
+  std::printf("odit_rel_l1: ok\n");
+  return 0;
+}
+
+static int check_gated_residual(hipStream_t st) {
+  const int B = 2, S = 7, C = 40;
+  std::vector<float> h(B * S * C), y(B * S * C), gate(B * C), out(B * S * C);
+  for (auto& v : h) v = next_uniform();
+  for (auto& v : y) v = next_uniform();
+  for (auto& v : gate) v = next_uniform();
+  DeviceBuffer<float> d_h, d_y, d_g, d_o;
+  HIP_OK(d_h.alloc(h.size())); HIP_OK(d_y.alloc(y.size())); HIP_OK(d_g.alloc(gate.size())); HIP_OK(d_o.alloc(out.size()));
+  HIP_OK(hipMemcpy(d_h.p, h.data(), h.size() * 4, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_y.p, y.data(), y.size() * 4, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_g.p, gate.data(), gate.size() * 4, hipMemcpyHostToDevice));
+  const int64_t dense[2] = {static_cast<int64_t>(S) * C, C}, per_batch[2] = {C, 0};
+  ODIT_OK_OR_FAIL(odit_gated_residual(d_h.p, d_y.p, d_g.p, nullptr, d_o.p, B, S, C, dense, dense, dense, per_batch,
+                                      ODIT_F32, ODIT_F32, 0, st));
+  HIP_OK(hipStreamSynchronize(st));
+  HIP_OK(hipMemcpy(out.data(), d_o.p, out.size() * 4, hipMemcpyDeviceToHost));
+  for (int b = 0; b < B; ++b)
+    for (int s = 0; s < S; ++s)
+      for (int c = 0; c < C; ++c) {
+        const int i = (b * S + s) * C + c;
+        const double want = static_cast<double>(h[i]) + static_cast<double>(gate[b * C + c]) * y[i];
+        if (std::fabs(out[i] - want) > 1e-6) {
+          std::fprintf(stderr, "gated_residual (%d,%d,%d): got %.9g, want %.9g\n", b, s, c, out[i], want);
+          return 1;
+        }
+      }
+  std::printf("odit_gated_residual: ok\n");
+  return 0;
+}
+
+static int check_attention(hipStream_t st) {
+  const int B = 1, Sq = 70, Sk = 130, H = 2, D = 64;  // ragged in queries and keys
+  const float scale = 0.125f;
+  std::vector<uint16_t> q(B * Sq * H * D), k(B * Sk * H * D), v(B * Sk * H * D), o(B * Sq * H * D);
+  for (auto& x : q) x = to_bf16(2.0f * next_uniform());
+  for (auto& x : k) x = to_bf16(2.0f * next_uniform());
+  for (auto& x : v) x = to_bf16(next_uniform());
+  DeviceBuffer<uint16_t> d_q, d_k, d_v, d_o;
+  HIP_OK(d_q.alloc(q.size())); HIP_OK(d_k.alloc(k.size())); HIP_OK(d_v.alloc(v.size())); HIP_OK(d_o.alloc(o.size()));
+  HIP_OK(hipMemcpy(d_q.p, q.data(), q.size() * 2, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_k.p, k.data(), k.size() * 2, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_v.p, v.data(), v.size() * 2, hipMemcpyHostToDevice));
+  const int64_t qs[3] = {static_cast<int64_t>(Sq) * H * D, H * D, D}, ks[3] = {static_cast<int64_t>(Sk) * H * D, H * D, D};
+  ODIT_OK_OR_FAIL(odit_attn_fwd(d_q.p, d_k.p, d_v.p, d_o.p, nullptr, nullptr, B, Sq, Sk, H, H, D, qs, ks, ks, qs, scale,
+                                ODIT_BF16, st));
+  HIP_OK(hipStreamSynchronize(st));
+  HIP_OK(hipMemcpy(o.data(), d_o.p, o.size() * 2, hipMemcpyDeviceToHost));
+  double worst = 0.0;
+  std::vector<double> s(Sk);
+  for (int h = 0; h < H; ++h)
+    for (int i = 0; i < Sq; ++i) {
+      double m = -1e300;
+      for (int j = 0; j < Sk; ++j) {
+        double acc = 0.0;
+        for (int d = 0; d < D; ++d) acc += static_cast<double>(from_bf16(q[(i * H + h) * D + d])) * from_bf16(k[(j * H + h) * D + d]);
+        s[j] = acc * scale;
+        m = s[j] > m ? s[j] : m;
+      }
+      double l = 0.0;
+      for (int j = 0; j < Sk; ++j) { s[j] = std::exp(s[j] - m); l += s[j]; }
+      for (int d = 0; d < D; ++d) {
+        double acc = 0.0;
+        for (int j = 0; j < Sk; ++j) acc += s[j] * from_bf16(v[(j * H + h) * D + d]);
+        const double err = std::fabs(from_bf16(o[(i * H + h) * D + d]) - acc / l);
+        worst = err > worst ? err : worst;
+      }
+    }
+  if (!(worst <= 2e-2)) {  // bf16 output, probabilities rounded to bf16 inside the kernel
+    std::fprintf(stderr, "attention: max abs error %.4g\n", worst);
+    return 1;
+  }
+  // an unsupported head size must be refused before any launch, with a message
+  const int rc = odit_attn_fwd(d_q.p, d_k.p, d_v.p, d_o.p, nullptr, nullptr, B, Sq, Sk, H, H, 96, qs, ks, ks, qs, scale, ODIT_BF16, st);
+  if (rc == 0 || std::strlen(odit_last_error()) == 0) {
+    std::fprintf(stderr, "attention: head size 96 was not refused\n");
+    return 1;
+  }
+  std::printf("odit_attn_fwd: ok (max abs error %.4g; head size 96 refused: %s)\n", worst, odit_last_error());
+  return 0;
+}
+
+int main() {
+  if (odit_version() != ODIT_VERSION) {
+    std::fprintf(stderr, "library version %d, header %d\n", odit_version(), ODIT_VERSION);
+    return 1;
+  }
+  HIP_OK(hipSetDevice(0));
+  hipStream_t st;
+  HIP_OK(hipStreamCreate(&st));
+  int rc = check_rel_l1(st);
+  if (rc == 0) rc = check_gated_residual(st);
+  if (rc == 0) rc = check_attention(st);
+  (void)hipStreamDestroy(st);
+  return rc;
+}
