@@ -129,3 +129,19 @@ def test_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
 
     with pytest.raises(_lib.OmniDitLibraryError):
         kernels.attn_workspace_bytes(1, 128, 128, 1, 128) if hasattr(kernels, "attn_workspace_bytes") else _lib.load()
+
+
+def test_header_is_plain_c(tmp_path):
+    """include/omni_dit.h is a C header: it compiles as C99 with pedantic warnings as errors, alone."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc on this machine")
+    src = tmp_path / "h.c"
+    src.write_text('#include "omni_dit.h"\nint main(void) { return ODIT_VERSION == 0; }\n')
+    include = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    proc = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I" + include, "-fsyntax-only", str(src)],
+                          capture_output=True, text=True)
+    assert proc.returncode == 0, proc.stderr
