@@ -1,5 +1,5 @@
 // A host program with no Python and no torch in it: it links libomni_dit_hip.so through include/omni_dit.h,
-// owns its device buffers through the HIP runtime, and checks three entry points against loops written here
+// owns its device buffers through the HIP runtime, and checks five entry points against loops written here
 // (double precision on the CPU). It is what a non-Python caller of the C ABI looks like; the GPU test
 // tests/test_gpu_native_host.py runs it as a child process and reads its exit status.
 #include <hip/hip_runtime.h>
@@ -168,6 +168,98 @@ static int check_attention(hipStream_t st) {
   return 0;
 }
 
+static int check_adaln(hipStream_t st) {
+  const int B = 2, S = 5, C = 96;
+  const float eps = 1e-6f;
+  std::vector<float> x(B * S * C), shift(B * C), scale(B * C), out(B * S * C);
+  for (auto& v : x) v = 3.0f * next_uniform() + 0.5f;
+  for (auto& v : shift) v = 0.5f * next_uniform();
+  for (auto& v : scale) v = 0.5f * next_uniform();
+  DeviceBuffer<float> d_x, d_sh, d_sc, d_o;
+  HIP_OK(d_x.alloc(x.size())); HIP_OK(d_sh.alloc(shift.size())); HIP_OK(d_sc.alloc(scale.size())); HIP_OK(d_o.alloc(out.size()));
+  HIP_OK(hipMemcpy(d_x.p, x.data(), x.size() * 4, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_sh.p, shift.data(), shift.size() * 4, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_sc.p, scale.data(), scale.size() * 4, hipMemcpyHostToDevice));
+  const int64_t dense[2] = {static_cast<int64_t>(S) * C, C};
+  ODIT_OK_OR_FAIL(odit_adaln_modulate(d_x.p, d_o.p, d_sh.p, d_sc.p, nullptr, nullptr, nullptr, nullptr, nullptr, B, S, C,
+                                      dense, dense, C, 0, eps, ODIT_F32, ODIT_F32, 0, st));
+  HIP_OK(hipStreamSynchronize(st));
+  HIP_OK(hipMemcpy(out.data(), d_o.p, out.size() * 4, hipMemcpyDeviceToHost));
+  for (int b = 0; b < B; ++b)
+    for (int s = 0; s < S; ++s) {
+      const float* row = &x[(b * S + s) * C];
+      double mean = 0.0, var = 0.0;
+      for (int c = 0; c < C; ++c) mean += row[c];
+      mean /= C;
+      for (int c = 0; c < C; ++c) var += (row[c] - mean) * (row[c] - mean);
+      const double rstd = 1.0 / std::sqrt(var / C + eps);
+      for (int c = 0; c < C; ++c) {
+        const double want = (row[c] - mean) * rstd * (1.0 + scale[b * C + c]) + shift[b * C + c];
+        if (std::fabs(out[(b * S + s) * C + c] - want) > 1e-4) {
+          std::fprintf(stderr, "adaln (%d,%d,%d): got %.9g, want %.9g\n", b, s, c, out[(b * S + s) * C + c], want);
+          return 1;
+        }
+      }
+    }
+  std::printf("odit_adaln_modulate: ok\n");
+  return 0;
+}
+
+static int check_qknorm_rope(hipStream_t st) {
+  // q and k are two thirds of a fused [B,S,3,H,D] projection output; they land at rows off.. of joint buffers
+  const int B = 2, S = 9, H = 3, D = 64, off = 4, S_total = S + off;
+  const float eps = 1e-6f;
+  std::vector<float> qkv(B * S * 3 * H * D), wq(D), wk(D), cs(S * D / 2), sn(S * D / 2);
+  std::vector<float> jq(B * S_total * H * D, 0.f), jk(jq);
+  for (auto& v : qkv) v = 2.0f * next_uniform();
+  for (auto& v : wq) v = 1.0f + 0.2f * next_uniform();
+  for (auto& v : wk) v = 1.0f + 0.2f * next_uniform();
+  for (int i = 0; i < S * D / 2; ++i) { const float a = 3.0f * next_uniform(); cs[i] = std::cos(a); sn[i] = std::sin(a); }
+  DeviceBuffer<float> d_qkv, d_wq, d_wk, d_cs, d_sn, d_jq, d_jk;
+  HIP_OK(d_qkv.alloc(qkv.size())); HIP_OK(d_wq.alloc(D)); HIP_OK(d_wk.alloc(D)); HIP_OK(d_cs.alloc(cs.size()));
+  HIP_OK(d_sn.alloc(sn.size())); HIP_OK(d_jq.alloc(jq.size())); HIP_OK(d_jk.alloc(jk.size()));
+  HIP_OK(hipMemcpy(d_qkv.p, qkv.data(), qkv.size() * 4, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_wq.p, wq.data(), D * 4, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_wk.p, wk.data(), D * 4, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_cs.p, cs.data(), cs.size() * 4, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_sn.p, sn.data(), sn.size() * 4, hipMemcpyHostToDevice));
+  HIP_OK(hipMemset(d_jq.p, 0, jq.size() * 4));
+  HIP_OK(hipMemset(d_jk.p, 0, jk.size() * 4));
+  const int64_t in_strides[2] = {static_cast<int64_t>(S) * 3 * H * D, 3 * H * D};
+  ODIT_OK_OR_FAIL(odit_qknorm_rope(d_qkv.p, d_qkv.p + H * D, nullptr, d_jq.p, d_jk.p, nullptr, d_wq.p, d_wk.p, d_cs.p, d_sn.p,
+                                   B, S, H, D, D, in_strides, off, S_total, eps, ODIT_NORM_HEAD, ODIT_F32, ODIT_F32, 0, st));
+  HIP_OK(hipStreamSynchronize(st));
+  HIP_OK(hipMemcpy(jq.data(), d_jq.p, jq.size() * 4, hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(jk.data(), d_jk.p, jk.size() * 4, hipMemcpyDeviceToHost));
+  for (int part = 0; part < 2; ++part) {
+    const std::vector<float>& got = part == 0 ? jq : jk;
+    const std::vector<float>& w = part == 0 ? wq : wk;
+    for (int b = 0; b < B; ++b)
+      for (int s = 0; s < S_total; ++s)
+        for (int h = 0; h < H; ++h) {
+          const float* g = &got[((b * S_total + s) * H + h) * D];
+          if (s < off) {  // rows in front of the offset belong to another stream: untouched
+            for (int d = 0; d < D; ++d) if (g[d] != 0.f) { std::fprintf(stderr, "qknorm: row %d written\n", s); return 1; }
+            continue;
+          }
+          const float* in = &qkv[(((b * S + (s - off)) * 3 + part) * H + h) * D];
+          double ms = 0.0;
+          for (int d = 0; d < D; ++d) ms += static_cast<double>(in[d]) * in[d];
+          const double rstd = 1.0 / std::sqrt(ms / D + eps);
+          for (int i = 0; i < D / 2; ++i) {
+            const double x0 = in[2 * i] * rstd * w[2 * i], x1 = in[2 * i + 1] * rstd * w[2 * i + 1];
+            const double c = cs[(s - off) * (D / 2) + i], sv = sn[(s - off) * (D / 2) + i];
+            if (std::fabs(g[2 * i] - (x0 * c - x1 * sv)) > 1e-4 || std::fabs(g[2 * i + 1] - (x1 * c + x0 * sv)) > 1e-4) {
+              std::fprintf(stderr, "qknorm part %d (%d,%d,%d,%d)\n", part, b, s, h, i);
+              return 1;
+            }
+          }
+        }
+  }
+  std::printf("odit_qknorm_rope: ok\n");
+  return 0;
+}
+
 int main() {
   if (odit_version() != ODIT_VERSION) {
     std::fprintf(stderr, "library version %d, header %d\n", odit_version(), ODIT_VERSION);
@@ -178,6 +270,8 @@ int main() {
   HIP_OK(hipStreamCreate(&st));
   int rc = check_rel_l1(st);
   if (rc == 0) rc = check_gated_residual(st);
+  if (rc == 0) rc = check_adaln(st);
+  if (rc == 0) rc = check_qknorm_rope(st);
   if (rc == 0) rc = check_attention(st);
   (void)hipStreamDestroy(st);
   return rc;
