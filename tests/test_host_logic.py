@@ -125,6 +125,55 @@ def test_state_manager_contexts():
     assert sm.get_state().cnt == 0
 
 
+def test_hook_route_is_rebuilt_when_the_hook_set_changes():
+    m = _Toy()
+    reg = HookRegistry.get_or_create(m)
+    calls = []
+
+    class Skip(ModelHook):
+        def initialize_hook(self, module):
+            calls.append("init")
+            return module
+
+        def new_forward(self, module, *args, **kwargs):
+            return module._original_forward(*args, **kwargs) if args[0] else "skipped"
+
+        def reset_state(self, module):
+            calls.append("reset")
+            return module
+
+    reg.register_hook("skip", Skip())
+    assert calls == ["init"] and m(0) == "skipped" and m(2) == 5 and reg.dispatch(2) == 5
+    reg.reset_hook("skip")
+    reg.reset_hook("absent")
+    assert calls == ["init", "reset"] and isinstance(reg.get_hook("skip"), Skip) and reg.get_hook("absent") is None
+    reg.remove_hook("absent")
+    reg.remove_hook("skip")
+    assert m(0) == 1 and m._hook_registry is reg and m._original_forward(1) == 3
+
+
+def test_qwen_rotary_tables_from_integer_positions_equal_the_oracles():
+    from oracle import qwen_image as oq
+    from vllm_omni_amd.blocks.qwen_image import QwenEmbedLayer3DRope, QwenEmbedRope
+
+    cfg = oq.tiny_config()
+    cases = [(False, [(1, 4, 6)]), (False, [(1, 5, 3)]), (False, [(1, 4, 4), (1, 6, 2), (2, 3, 5)]),
+             (True, [(1, 2, 2)] * 5 + [(1, 2, 3)]), (True, [(1, 3, 3)]), (False, [(1, 64, 64)])]
+    for layer3d, shapes in cases:
+        rope = (QwenEmbedLayer3DRope if layer3d else QwenEmbedRope)(
+            theta=cfg.theta, axes_dim=list(cfg.axes_dims_rope), scale_rope=True)
+        vid, txt = rope(shapes, [3, 5], "cpu")
+        want_v, want_t = oq.qwen_rope_freqs_images(cfg, shapes, txt_len=5, layer3d=layer3d)
+        assert vid.dtype == torch.complex64 and torch.equal(vid, want_v) and torch.equal(txt, want_t)
+    # without centring rows and columns count from zero and text starts after the full extent
+    plain = QwenEmbedRope(theta=10000, axes_dim=[4, 6, 6], scale_rope=False)
+    vid, txt = plain((1, 2, 3), [2], "cpu")
+    inv = 1.0 / np.power(10000.0, np.arange(0, 6, 2) / 6)
+    np.testing.assert_allclose(vid[5, 2:5].numpy(), np.exp(1j * 1 * inv), atol=1e-6)   # token (0, 1, 2): row 1
+    np.testing.assert_allclose(vid[5, 5:8].numpy(), np.exp(1j * 2 * inv), atol=1e-6)   # column 2
+    np.testing.assert_allclose(txt[1, 5:8].numpy(), np.exp(1j * 4 * inv), atol=1e-6)   # start 3, second token
+
+
 # ----------------------------------------------------------------------------------- registry / selector
 def test_backend_registry_and_selector(monkeypatch):
     E = DiffusionAttentionBackendEnum

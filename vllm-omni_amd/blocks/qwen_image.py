@@ -124,59 +124,57 @@ def project_residual(lin: nn.Linear, x: torch.Tensor, residual: torch.Tensor, ga
 
 
 class QwenEmbedRope(nn.Module):
-    """3-axis rotary tables with centred rows/columns (``scale_rope=True``), qit.py:298-396.
-    ``forward`` returns complex64 (vid_freqs, txt_freqs) like the reference; ``cos_sin`` returns the
-    float32 [S, D/2] tables the fused kernel reads, cached per (shape, device)."""
+    """3-axis rotary tables (frame, row, column) of qit.py:298-396, built from integer token positions.
+
+    Token (f, r, c) of image number ``i`` of the list sits at frame ``i + f``; with ``scale_rope`` rows
+    and columns are centred (row r of an image with ``h`` rows sits at ``r - (h - h // 2)``), otherwise
+    they count from zero. Text token ``j`` sits at ``(p, p, p)`` with ``p = start + j`` where ``start``
+    is the largest half-extent (full extent without ``scale_rope``) over the images. A position ``x`` on
+    an axis of ``d`` channels gives the d/2 angles ``x * theta ** (-2k / d)``, evaluated in float32.
+    ``forward`` returns complex64 (vid_freqs, txt_freqs) like the reference, cached per (shapes, device)."""
 
     layer3d = False  # QwenEmbedLayer3DRope sets it
 
     def __init__(self, theta: int, axes_dim: list[int], scale_rope: bool = True):
         super().__init__()
         self.theta, self.axes_dim, self.scale_rope = theta, list(axes_dim), scale_rope
-        pos = torch.arange(4096)
-        neg = torch.arange(4096).flip(0) * -1 - 1
-        self.pos_freqs = torch.cat([self.rope_params(pos, d, theta) for d in self.axes_dim], dim=1)
-        self.neg_freqs = torch.cat([self.rope_params(neg, d, theta) for d in self.axes_dim], dim=1)
+        if any(d % 2 for d in self.axes_dim):
+            raise ValueError("every rotary axis needs an even number of channels")
+        # inverse frequencies of the three axes, side by side: [sum(d) / 2]
+        self.inv_freq = torch.cat([
+            1.0 / torch.pow(theta, torch.arange(0, d, 2).to(torch.float32).div(d)) for d in self.axes_dim])
+        self.axis_of = torch.repeat_interleave(torch.arange(len(self.axes_dim)),
+                                               torch.tensor([d // 2 for d in self.axes_dim]))
         self._tables = lru_cache(maxsize=16)(self._build)
 
-    @staticmethod
-    def rope_params(index: torch.Tensor, dim: int, theta: int = 10000) -> torch.Tensor:
-        assert dim % 2 == 0
-        inv = 1.0 / torch.pow(theta, torch.arange(0, dim, 2).to(torch.float32).div(dim))
-        ang = torch.outer(index.to(torch.float32), inv)
+    def _table(self, positions: torch.Tensor) -> torch.Tensor:
+        """positions: int64 [N, 3] -> complex64 [N, sum(d) / 2] unit phasors."""
+        ang = positions.to(torch.float32)[:, self.axis_of] * self.inv_freq
         return torch.polar(torch.ones_like(ang), ang)
 
-    def _video_freqs(self, frame: int, height: int, width: int, idx: int = 0) -> torch.Tensor:
-        """``idx`` = frame position of the image's first frame; -1 = the condition image of the layered
-        variant, which sits one frame before the origin (qit.py:278-296)."""
-        halves = [d // 2 for d in self.axes_dim]
-        fp = self.pos_freqs.split(halves, dim=1)
-        fn = self.neg_freqs.split(halves, dim=1)
-        if idx < 0:
-            if frame != 1:
-                raise ValueError("the condition image of the layered variant has one frame")
-            f_t = fn[0][-1:].view(1, 1, 1, -1).expand(frame, height, width, -1)
-        else:
-            f_t = fp[0][idx:idx + frame].view(frame, 1, 1, -1).expand(frame, height, width, -1)
-        if self.scale_rope:
-            rows = torch.cat([fn[1][-(height - height // 2):], fp[1][: height // 2]], dim=0)
-            cols = torch.cat([fn[2][-(width - width // 2):], fp[2][: width // 2]], dim=0)
-        else:
-            rows, cols = fp[1][:height], fp[2][:width]
-        f_h = rows.view(1, height, 1, -1).expand(frame, height, width, -1)
-        f_w = cols.view(1, 1, width, -1).expand(frame, height, width, -1)
-        return torch.cat([f_t, f_h, f_w], dim=-1).reshape(frame * height * width, -1).contiguous()
+    def _image_positions(self, frame: int, height: int, width: int, first_frame: int) -> torch.Tensor:
+        r0 = -(height - height // 2) if self.scale_rope else 0
+        c0 = -(width - width // 2) if self.scale_rope else 0
+        grid = torch.stack(torch.meshgrid(torch.arange(first_frame, first_frame + frame),
+                                          torch.arange(r0, r0 + height), torch.arange(c0, c0 + width),
+                                          indexing="ij"), dim=-1)
+        return grid.reshape(-1, 3)
 
     def _build(self, shapes: tuple[tuple[int, int, int], ...], txt_len: int, device: str):
-        vids, start = [], 0
-        layer_num = len(shapes) - 1
-        for idx, (f, h, w) in enumerate(shapes):
-            vids.append(self._video_freqs(f, h, w, -1 if self.layer3d and idx == layer_num else idx))
+        last = len(shapes) - 1
+        pos, start = [], 0
+        for i, (f, h, w) in enumerate(shapes):
+            first = i
+            if self.layer3d and i == last:  # the condition image: one frame before the origin (qit.py:278-296)
+                if f != 1:
+                    raise ValueError("the condition image of the layered variant has one frame")
+                first = -1
+            pos.append(self._image_positions(f, h, w, first))
             start = max(start, max(h // 2, w // 2) if self.scale_rope else max(h, w))
         if self.layer3d:
-            start = max(start, layer_num)
-        vid = torch.cat(vids, dim=0).to(device)
-        txt = self.pos_freqs[start:start + txt_len].to(device)
+            start = max(start, last)
+        vid = self._table(torch.cat(pos, dim=0)).to(device)
+        txt = self._table(torch.arange(start, start + txt_len).view(-1, 1).expand(-1, 3)).to(device)
         return vid, txt
 
     @staticmethod

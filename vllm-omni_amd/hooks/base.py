@@ -1,44 +1,65 @@
-"""Forward-interception hooks: ``HookRegistry`` wraps ``module.forward`` once and routes calls to
-registered ``ModelHook`` objects; ``StateManager`` keeps one state object per named context.
-Public surface of vllm_omni/diffusion/hooks/base.py:18-247."""
+"""Forward interception for one module, with the class and method names of
+vllm_omni/diffusion/hooks/base.py:18-247 (``BaseState``, ``StateManager``, ``ModelHook``,
+``HookRegistry``) so hooks written against the reference attach unchanged.
+
+Design of this implementation: the registry does no work per call. Every change of the hook set
+(``register_hook`` / ``remove_hook``) rebuilds ONE callable, the *route*, and ``module.forward`` is a
+thin trampoline to the current route:
+
+  * no hooks       -> the route IS the module's original bound forward;
+  * one hook       -> the route is that hook's ``new_forward`` with the module bound in (the hook owns
+                      the call and may never reach the original forward: that is how TeaCache skips);
+  * several hooks  -> a pipeline: ``pre_forward`` of every hook in ascending name order, the original
+                      forward, ``post_forward`` in descending name order.
+
+The attributes ``module._original_forward`` and ``module._hook_registry`` are part of the interface:
+hooks call the former, cache backends look up the latter.
+"""
 
 from __future__ import annotations
 
+import functools
 from collections.abc import Callable
 from typing import Any
 
 import torch.nn as nn
 
+_DEFAULT_CONTEXT = "default"
+
 
 class BaseState:
+    """State container of a hook; ``reset`` returns it to its initial condition."""
+
     def reset(self) -> None:
-        pass
+        return None
 
 
 class StateManager:
-    """Lazily creates ``state_cls()`` per context name; ``reset`` forgets them all (base.py:25-42)."""
+    """One lazily built ``state_cls()`` per context name (e.g. one per CFG branch); the current
+    context is selected with ``set_context`` and an empty name selects ``"default"``."""
 
     def __init__(self, state_cls: Callable[[], BaseState]):
-        self._state_cls = state_cls
-        self._states: dict[str, BaseState] = {}
-        self._context = "default"
+        self._factory = state_cls
+        self._by_context: dict[str, BaseState] = {}
+        self._current = _DEFAULT_CONTEXT
 
     def set_context(self, name: str) -> None:
-        self._context = name or "default"
+        self._current = name if name else _DEFAULT_CONTEXT
 
     def get_state(self) -> BaseState:
-        st = self._states.get(self._context)
-        if st is None:
-            st = self._states[self._context] = self._state_cls()
-        return st
+        try:
+            return self._by_context[self._current]
+        except KeyError:
+            state = self._by_context[self._current] = self._factory()
+            return state
 
     def reset(self) -> None:
-        self._states.clear()
+        self._by_context = {}
 
 
 class ModelHook:
-    """Override ``pre_forward`` / ``post_forward`` to edit arguments or outputs, or ``new_forward``
-    to replace the call altogether (base.py:45-122)."""
+    """A hook edits the call (``pre_forward``), its result (``post_forward``), or takes the whole call
+    over (``new_forward``, whose default is pre -> original forward -> post)."""
 
     def initialize_hook(self, module: nn.Module) -> nn.Module:
         return module
@@ -50,69 +71,82 @@ class ModelHook:
         return output
 
     def new_forward(self, module: nn.Module, *args: Any, **kwargs: Any) -> Any:
-        args, kwargs = self.pre_forward(module, *args, **kwargs)
-        return self.post_forward(module, module._original_forward(*args, **kwargs))
+        call_args, call_kwargs = self.pre_forward(module, *args, **kwargs)
+        return self.post_forward(module, module._original_forward(*call_args, **call_kwargs))
 
     def reset_state(self, module: nn.Module) -> nn.Module:
         return module
 
 
-class _WrappedForward:
-    """Callable installed as ``module.forward`` (base.py:125-135)."""
+def _pipeline(module: nn.Module, hooks: list[ModelHook]) -> Callable[..., Any]:
+    """Route for several hooks; ``hooks`` is already in ascending name order."""
+    pres = [h.pre_forward for h in hooks]
+    posts = [h.post_forward for h in hooks[::-1]]
 
-    def __init__(self, module: nn.Module):
-        self.module = module
+    def route(*args: Any, **kwargs: Any) -> Any:
+        for pre in pres:
+            args, kwargs = pre(module, *args, **kwargs)
+        result = module._original_forward(*args, **kwargs)
+        for post in posts:
+            result = post(module, result)
+        return result
 
-    def __call__(self, *args: Any, **kwargs: Any):
-        reg = getattr(self.module, "_hook_registry", None)
-        if reg is None or not reg._hooks:
-            return self.module._original_forward(*args, **kwargs)
-        return reg.dispatch(*args, **kwargs)
+    return route
 
 
 class HookRegistry:
+    """The hooks of one module, by name. Obtain it with ``HookRegistry.get_or_create(module)``."""
+
     def __init__(self, module: nn.Module):
         self.module = module
         self._hooks: dict[str, ModelHook] = {}
+        self._route: Callable[..., Any] | None = None  # None until the module's forward is captured
 
+    # -- attachment ------------------------------------------------------------------------------
     @classmethod
     def get_or_create(cls, module: nn.Module) -> "HookRegistry":
-        reg = getattr(module, "_hook_registry", None)
-        if reg is None:
-            reg = cls(module)
-            module._hook_registry = reg
-            if not hasattr(module, "_original_forward"):
-                module._original_forward = module.forward
-                module.forward = _WrappedForward(module)
-        return reg
+        existing = getattr(module, "_hook_registry", None)
+        if existing is not None:
+            return existing
+        registry = cls(module)
+        if not hasattr(module, "_original_forward"):  # capture the forward exactly once per module
+            module._original_forward = module.forward
+            module.forward = registry._trampoline
+        module._hook_registry = registry
+        registry._rebuild()
+        return registry
 
+    def _trampoline(self, *args: Any, **kwargs: Any) -> Any:
+        return self._route(*args, **kwargs)
+
+    def _rebuild(self) -> None:
+        module = self.module
+        names = sorted(self._hooks)
+        if not names:
+            self._route = module._original_forward
+        elif len(names) == 1:
+            self._route = functools.partial(self._hooks[names[0]].new_forward, module)
+        else:
+            self._route = _pipeline(module, [self._hooks[n] for n in names])
+
+    # -- hook set --------------------------------------------------------------------------------
     def register_hook(self, name: str, hook: ModelHook) -> None:
         hook.initialize_hook(self.module)
         self._hooks[name] = hook
+        self._rebuild()
 
     def remove_hook(self, name: str) -> None:
-        self._hooks.pop(name, None)
+        if self._hooks.pop(name, None) is not None:
+            self._rebuild()
 
     def get_hook(self, name: str) -> ModelHook | None:
         return self._hooks.get(name)
-
-    def dispatch(self, *args: Any, **kwargs: Any) -> Any:
-        """One hook: its ``new_forward`` owns the call. Several: all ``pre_forward`` in name order,
-        the original forward, then all ``post_forward`` in reverse (base.py:203-237)."""
-        if not self._hooks:
-            return self.module._original_forward(*args, **kwargs)
-        if len(self._hooks) == 1:
-            (hook,) = self._hooks.values()
-            return hook.new_forward(self.module, *args, **kwargs)
-        ordered = [self._hooks[k] for k in sorted(self._hooks)]
-        for h in ordered:
-            args, kwargs = h.pre_forward(self.module, *args, **kwargs)
-        out = self.module._original_forward(*args, **kwargs)
-        for h in reversed(ordered):
-            out = h.post_forward(self.module, out)
-        return out
 
     def reset_hook(self, name: str) -> None:
         hook = self._hooks.get(name)
         if hook is not None:
             hook.reset_state(self.module)
+
+    def dispatch(self, *args: Any, **kwargs: Any) -> Any:
+        """Run one call through the current route (what ``module(...)`` does)."""
+        return self._route(*args, **kwargs)
