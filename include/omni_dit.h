@@ -111,6 +111,15 @@ int odit_attn_fwd_ex(const void* q, const void* k, const void* v, const void* v_
 /* Scratch bytes odit_attn_fwd_ex can use for this shape on the current device (0 = none needed). */
 size_t odit_attn_fwd_workspace_bytes(int B, int Sq, int Sk, int H, int D);
 
+/* Which kernels odit_attn_fwd_ex launches for a problem, as text: "<kernel> units=<workgroups>" per
+ * launch, joined by "; " (the kernel names are the ones a profiler reports). k_seq_stride / v_seq_stride
+ * are the sequence strides of k and v in elements; with_workspace says whether scratch will be given.
+ * Returns the number of launches, or a negative status. Host-only: enqueues nothing. No counterpart in the
+ * reference; for tests and for benchmarks that must name the kernel they time.
+ */
+int odit_attn_fwd_plan(int B, int Sq, int Sk, int H, int D, int64_t k_seq_stride, int64_t v_seq_stride,
+                       int with_workspace, char* text, size_t text_bytes);
+
 /* ---------------------------------------------------------------------------------------------
  * K2  fused QK-RMSNorm + rotary embedding + scatter into the joint [txt;img] sequence.
  *

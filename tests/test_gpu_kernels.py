@@ -386,6 +386,34 @@ def _attn_inputs(B, Sq, Sk, H, Hkv, D, seed, dtype=torch.bfloat16):
     return q, k, v
 
 
+def _far_apart_rows(t, gpu):
+    """The same [B,S,H,D] values on the GPU as a view whose sequence stride is so large that the rows of one
+    (batch, head) span 2 GiB: the library then has to address them through 64-bit pointers (its second attention
+    kernel) instead of 32-bit buffer offsets."""
+    B, S, H, D = t.shape
+    stride = -(-(1 << 30) // (S + 64))
+    stride = max((stride + 7) // 8 * 8, H * D)
+    big = torch.empty((B, S, stride), dtype=t.dtype, device=gpu)
+    view = big[:, :, : H * D].view(B, S, H, D)
+    view.copy_(t)
+    return view
+
+
+def _kv_for_path(path, k, v, gpu):
+    from vllm_omni_amd import kernels
+
+    if path == "pointer":
+        kg, vg = _far_apart_rows(k, gpu), _far_apart_rows(v, gpu)
+    else:
+        kg, vg = k.to(gpu), v.to(gpu)
+    B, Sk, H, D = k.shape
+    plan = kernels.attn_plan(B, 64, Sk, H, D, kg.stride(1), vg.stride(1))
+    assert plan.startswith("attn_fwd_pipe_kernel" if path == "pointer" else "attn_fwd_dma_kernel"), plan
+    return kg, vg
+
+
+ATTN_PATHS = ["buffer", "pointer"]   # which of the library's two attention kernels the strides select
+
 ATTN_SHAPES = [
     # B, Sq, Sk, H, Hkv, D
     (2, 64, 64, 8, 8, 64),       # the reference's own test shape (tests/diffusion/attention/test_flash_attn.py)
@@ -397,17 +425,17 @@ ATTN_SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("variant", ["14", "18", "24", "28", "29", "38", "34"])
+@pytest.mark.parametrize("path", ATTN_PATHS)
 @pytest.mark.parametrize("shape", ATTN_SHAPES)
-def test_attention_parity(gpu, monkeypatch, variant, shape):
+def test_attention_parity(gpu, path, shape):
     from vllm_omni_amd import kernels
 
-    monkeypatch.setenv("ODIT_ATTN_VARIANT", variant)
     B, Sq, Sk, H, Hkv, D = shape
     q, k, v = _attn_inputs(B, Sq, Sk, H, Hkv, D, seed=42)
     scale = 1.0 / math.sqrt(D)
-    print(f"attn variant={variant} shape={shape}", flush=True)
-    got, lse = kernels.attn_fwd(q.to(gpu), k.to(gpu), v.to(gpu), scale, return_lse=True)
+    print(f"attn path={path} shape={shape}", flush=True)
+    kg, vg = _kv_for_path(path, k, v, gpu)
+    got, lse = kernels.attn_fwd(q.to(gpu), kg, vg, scale, return_lse=True)
     torch.cuda.synchronize()
     want = ops.sdpa(q.float(), k.float(), v.float(), scale)
     # bf16 output of values in [-~3, 3]: error budget = P rounded to bf16 inside + one output rounding
@@ -421,16 +449,15 @@ def test_attention_parity(gpu, monkeypatch, variant, shape):
     _close(lse, torch.logsumexp(s, dim=-1), atol=2e-2, rtol=1e-3, what="lse")
 
 
-@pytest.mark.parametrize("variant", ["34", "38", "28"])
+@pytest.mark.parametrize("path", ATTN_PATHS)
 @pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("order", ["rising", "falling", "random"])
-def test_attention_peaked_logits(gpu, monkeypatch, variant, D, order):
+def test_attention_peaked_logits(gpu, path, D, order):
     """Logits with a standard deviation of about 16 and a row maximum that keeps rising (or falling) from one key
     tile to the next: the running-maximum update, the rescaling of the accumulators that is skipped while the
     maximum grows by less than 2^8, and probabilities that underflow to zero, against an fp64 softmax."""
     from vllm_omni_amd import kernels
 
-    monkeypatch.setenv("ODIT_ATTN_VARIANT", variant)
     B, Sq, Sk, H = 1, 200, 700, 2
     q, k, v = _attn_inputs(B, Sq, Sk, H, H, D, seed=77)
     ramp = torch.linspace(0.5, 7.5, Sk).view(1, Sk, 1, 1)
@@ -441,7 +468,8 @@ def test_attention_peaked_logits(gpu, monkeypatch, variant, D, order):
     k = (k.float() * ramp).bfloat16()
     q = (q.float() * 4.0).bfloat16()
     scale = 1.0 / math.sqrt(D)
-    got, lse = kernels.attn_fwd(q.to(gpu), k.to(gpu), v.to(gpu), scale, return_lse=True)
+    kg, vg = _kv_for_path(path, k, v, gpu)
+    got, lse = kernels.attn_fwd(q.to(gpu), kg, vg, scale, return_lse=True)
     s = torch.einsum("bqhd,bkhd->bhqk", q.double(), k.double()) * scale
     assert s.std() > 10 and s.max() > 80            # far outside what N(0,1) inputs reach
     want = torch.einsum("bhqk,bkhd->bqhd", torch.softmax(s, dim=-1), v.double())
@@ -460,12 +488,9 @@ def test_attention_fp16_and_strided_views(gpu):
     _close(got, want, atol=3e-3, rtol=3e-3, what="fp16 strided attention")
 
 
-@pytest.mark.parametrize("variant", ["18", "24", "28", "38", "34"])
-def test_attention_key_mask_equals_deleting_keys(gpu, monkeypatch, variant):
+def test_attention_key_mask_equals_deleting_keys(gpu):
     """The reference's padding-equivalence property (test_flash_attn.py:60-147)."""
     from vllm_omni_amd import kernels
-
-    monkeypatch.setenv("ODIT_ATTN_VARIANT", variant)
     from vllm_omni_amd.attention.backends.abstract import AttentionMetadata
     from vllm_omni_amd.attention.layer import Attention
 
@@ -504,16 +529,17 @@ def test_attention_key_mask_equals_deleting_keys(gpu, monkeypatch, variant):
                        layer(q.to(gpu), k.to(gpu), v.to(gpu)).cpu())
 
 
-@pytest.mark.parametrize("variant", ["18", "28", "38", "34"])
+@pytest.mark.parametrize("path", ATTN_PATHS)
 @pytest.mark.parametrize("split", [0, 1, 37, 64, 299, 300])
-def test_attention_split_output_equals_slices(gpu, monkeypatch, variant, split):
+def test_attention_split_output_equals_slices(gpu, path, split):
     """Two dense outputs written by the kernel == slices of the single output, bit for bit."""
     from vllm_omni_amd import kernels
 
-    monkeypatch.setenv("ODIT_ATTN_VARIANT", variant)
     B, S, H, D = 2, 300, 3, 128
-    q, k, v = (t.to(gpu) for t in _attn_inputs(B, S, S, H, H, D, seed=77))
-    print(f"attn split variant={variant} split={split}", flush=True)
+    q, k, v = _attn_inputs(B, S, S, H, H, D, seed=77)
+    q = q.to(gpu)
+    k, v = _kv_for_path(path, k, v, gpu)
+    print(f"attn split path={path} split={split}", flush=True)
     whole, lse = kernels.attn_fwd(q, k, v, 0.09, return_lse=True)
     head, tail, lse2 = kernels.attn_fwd(q, k, v, 0.09, return_lse=True, split=split)
     assert head.shape == (B, split, H, D) and tail.shape == (B, S - split, H, D)
@@ -534,19 +560,19 @@ KEY_SPLIT_SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("variant", ["34", "38"])
 @pytest.mark.parametrize("shape", KEY_SPLIT_SHAPES)
-def test_attention_key_split_tail(gpu, monkeypatch, variant, shape):
+def test_attention_key_split_tail(gpu, shape):
     """The launch that cuts its last round of workgroups into key ranges and merges them must agree with
     the single-pass launch and with the oracle: plain, with a key mask, with LSE and with two outputs."""
     from vllm_omni_amd import _lib, kernels
 
-    monkeypatch.setenv("ODIT_ATTN_VARIANT", variant)
     B, Sq, Sk, H, Hkv, D = shape
     assert _lib.load().odit_attn_fwd_workspace_bytes(B, Sq, Sk, H, D) > 0, "shape does not exercise the key split"
+    assert "attn_merge_kernel" in kernels.attn_plan(B, Sq, Sk, H, D)
+    assert "attn_merge_kernel" not in kernels.attn_plan(B, Sq, Sk, H, D, use_workspace=False)
     q, k, v = _attn_inputs(B, Sq, Sk, H, Hkv, D, seed=5)
     scale = 1.0 / math.sqrt(D)
-    print(f"attn key-split variant={variant} shape={shape}", flush=True)
+    print(f"attn key-split shape={shape}", flush=True)
     qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
     one, lse1 = kernels.attn_fwd(qg, kg, vg, scale, return_lse=True, use_workspace=False)
     two, lse2 = kernels.attn_fwd(qg, kg, vg, scale, return_lse=True)
@@ -584,20 +610,18 @@ def test_attention_key_split_tail(gpu, monkeypatch, variant, shape):
     _close(lsep, torch.logsumexp(sp, dim=-1).float(), atol=2e-2, rtol=1e-3, what="key-split, peaked logits, lse")
 
 
-@pytest.mark.parametrize("variant", ["34", "38", "28"])
 @pytest.mark.parametrize("shape,cut", [((2, 300, 300, 4, 4, 128), 64), ((1, 1100, 1100, 3, 3, 64), 256),
                                        ((2, 130, 2048, 4, 2, 128), 1024), ((1, 300, 1100, 3, 3, 128), 192),
                                        ((2, 200, 200, 2, 2, 128), 70)])
-def test_attention_values_in_two_tensors(gpu, monkeypatch, variant, shape, cut):
+def test_attention_values_in_two_tensors(gpu, shape, cut):
     """Value rows of keys [0, cut) and [cut, Sk) taken from two tensors (strided views of two wider
     buffers, like the value thirds of two fused-QKV outputs) give the result of the concatenated tensor bit
     for bit: plain, masked, with two outputs, and on launches that split their last round by keys. A cut
-    that is not a multiple of 64 (last case) or a kernel variant without the feature ("28") goes through
-    a concatenation inside the wrapper."""
+    that is not a multiple of 64 (last case) goes through a concatenation inside the wrapper, which counts it."""
     from vllm_omni_amd import kernels
 
-    monkeypatch.setenv("ODIT_ATTN_VARIANT", variant)
     B, Sq, Sk, H, Hkv, D = shape
+    copies_before = kernels.HIDDEN_COPIES["attn_value_pair_concatenated"]
     q, k, v = _attn_inputs(B, Sq, Sk, H, Hkv, D, seed=11)
     scale = 1.0 / math.sqrt(D)
     qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
@@ -607,6 +631,7 @@ def test_attention_values_in_two_tensors(gpu, monkeypatch, variant, shape, cut):
     pair = (wide_a[:, :, 2], wide_b[:, :, 2])
     want = kernels.attn_fwd(qg, kg, vg, scale)
     assert torch.equal(kernels.attn_fwd(qg, kg, pair, scale), want)
+    assert kernels.HIDDEN_COPIES["attn_value_pair_concatenated"] - copies_before == (0 if cut % 64 == 0 else 1)
     m = torch.rand(B, Sk, generator=torch.Generator().manual_seed(12)) > 0.3
     m[:, -1] = True
     assert torch.equal(kernels.attn_fwd(qg, kg, pair, scale, key_mask=m.to(gpu)),

@@ -39,6 +39,10 @@ _SIGNATURES = {
          _i64p, _i64p, _i64p, _i64p, _i64p, _i64p, C.c_float, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p],
     ),
     "odit_attn_fwd_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "odit_attn_fwd_plan": (
+        C.c_int,
+        [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int, C.c_char_p, C.c_size_t],
+    ),
     "odit_qknorm_rope": (
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,

@@ -9,8 +9,6 @@ from typing import Generic, TypeVar
 
 import torch
 
-from ...platforms import current_omni_platform
-
 
 class AttentionBackend(ABC):
     """Class-level description of a backend; never instantiated (abstract.py:13-51)."""
@@ -55,7 +53,10 @@ class AttentionMetadata:
     [s, Sq) of the joint sequence, instead of one tensor the caller would slice and copy.
     ``value_tail`` (not in the reference): the ``value`` argument then holds only the rows of the first
     keys and this tensor the rest, so a caller with the values of two streams in two buffers does not
-    have to concatenate them."""
+    have to concatenate them.
+    ``attn_mask_checked`` (not in the reference): the caller vouches that ``attn_mask`` is worth applying
+    (it has already dropped an all-true mask, or accepts the masked kernel for one), so the backend skips
+    its own all-true test, which costs a device-to-host synchronisation per call."""
 
     attn_mask: torch.Tensor | None = None
     joint_attn_mask: torch.Tensor | None = None
@@ -65,13 +66,15 @@ class AttentionMetadata:
     joint_strategy: str = "front"
     output_split: int | None = None
     value_tail: torch.Tensor | None = None
+    attn_mask_checked: bool = False
 
 
 T = TypeVar("T", bound=AttentionMetadata)
 
 
 class AttentionImpl(ABC, Generic[T]):
-    """abstract.py:69-140: ``forward`` dispatches on the platform; on ROCm that is ``forward_hip``."""
+    """abstract.py:69-140. The reference's ``forward`` picks a per-platform method; with one platform
+    here it is always ``forward_hip``, which each backend implements."""
 
     @abstractmethod
     def __init__(self, num_heads: int, head_size: int, softmax_scale: float, causal: bool = False,
@@ -79,25 +82,7 @@ class AttentionImpl(ABC, Generic[T]):
 
     def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                 attn_metadata: T | None = None) -> torch.Tensor:
-        plat = current_omni_platform
-        if plat.is_rocm():
-            return self.forward_hip(query, key, value, attn_metadata)
-        if plat.is_cuda():
-            return self.forward_cuda(query, key, value, attn_metadata)
-        if plat.is_npu():
-            return self.forward_npu(query, key, value, attn_metadata)
-        if plat.is_xpu():
-            return self.forward_xpu(query, key, value, attn_metadata)
-        raise NotImplementedError(f"No forward implementation for platform: {plat}")
+        return self.forward_hip(query, key, value, attn_metadata)
 
-    def forward_cuda(self, query, key, value, attn_metadata=None):
-        raise NotImplementedError
-
-    def forward_npu(self, query, key, value, attn_metadata=None):
-        raise NotImplementedError
-
-    def forward_xpu(self, query, key, value, attn_metadata=None):
-        raise NotImplementedError
-
-    def forward_hip(self, query, key, value, attn_metadata=None):
-        return self.forward_cuda(query, key, value, attn_metadata)
+    @abstractmethod
+    def forward_hip(self, query, key, value, attn_metadata=None): ...

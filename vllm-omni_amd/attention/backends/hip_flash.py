@@ -46,21 +46,18 @@ class HipFlashAttentionImpl(AttentionImpl):
     def forward_hip(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                     attn_metadata: AttentionMetadata | None = None) -> torch.Tensor:
         """q [B,Sq,H,D], k/v [B,Sk,Hkv,D] -> [B,Sq,H,D]. A [B,Sk] ``attn_mask`` excludes keys; an
-        all-true mask is dropped like the reference does (flash_attn.py:80-84). With
+        all-true mask is dropped like the reference does (flash_attn.py:80-84) unless
+        ``attn_metadata.attn_mask_checked`` says the caller has seen to that (the test synchronises). With
         ``attn_metadata.output_split`` = s the result is the pair (out[:, :s], out[:, s:]), both dense;
         with ``attn_metadata.value_tail`` the values are [value; value_tail] along the keys, read in place."""
         mask = attn_metadata.attn_mask if attn_metadata is not None else None
         if mask is not None:
             if mask.dim() != 2:
                 raise ValueError("HipFlashAttentionImpl takes a [B,Sk] key-padding mask")
-            if bool(torch.all(mask != 0)):
+            if not attn_metadata.attn_mask_checked and bool(torch.all(mask != 0)):
                 mask = None
         split = attn_metadata.output_split if attn_metadata is not None else None
         v_tail = attn_metadata.value_tail if attn_metadata is not None else None
         if v_tail is not None:
             value = (value, v_tail)
         return kernels.attn_fwd(query, key, value, self.softmax_scale, key_mask=mask, split=split)
-
-    # the platform never routes here; kept so a direct call cannot silently pick another kernel
-    def forward_cuda(self, query, key, value, attn_metadata=None):
-        return self.forward_hip(query, key, value, attn_metadata)

@@ -50,5 +50,3 @@ class SDPAImpl(AttentionImpl):
         if split is not None:
             return out[:, :split].contiguous(), out[:, split:].contiguous()
         return out
-
-    forward_cuda = forward_hip

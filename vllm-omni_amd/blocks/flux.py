@@ -141,7 +141,7 @@ class FluxAttention(nn.Module):
         jq = torch.empty((B, S, H, D), dtype=qkv.dtype, device=qkv.device)
         jk = torch.empty_like(jq)
         # v is only moved, never changed: read in place from the two projections when the kernel can
-        v_in_place = S_c % 64 == 0 and qkv.dtype != torch.float32 and kernels.attn_reads_value_pairs() and not rr
+        v_in_place = S_c % 64 == 0 and qkv.dtype != torch.float32 and not rr
         jv = None if v_in_place else torch.empty_like(jq)
         tc = ts = ic = isn = None
         if rot is not None:

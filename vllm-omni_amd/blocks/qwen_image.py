@@ -254,7 +254,7 @@ class QwenImageCrossAttention(nn.Module):
         jk = torch.empty_like(jq)
         # q and k are rewritten by norm + rotary into the joint buffers; v is only moved, so when the
         # attention kernel can read the two value halves where the projections left them it is not copied
-        v_in_place = (S_txt % 64 == 0 and img_qkv.dtype != torch.float32 and kernels.attn_reads_value_pairs()
+        v_in_place = (S_txt % 64 == 0 and img_qkv.dtype != torch.float32
                       and not self.ref_rounding)
         jv = None if v_in_place else torch.empty_like(jq)
         rr = self.ref_rounding
@@ -273,6 +273,9 @@ class QwenImageCrossAttention(nn.Module):
             txt_m = encoder_hidden_states_mask if encoder_hidden_states_mask is not None else ones(S_txt)
             img_m = hidden_states_mask if hidden_states_mask is not None else ones(S_img)
             meta.attn_mask = torch.cat([txt_m.bool(), img_m.bool()], dim=1)
+            # the model drops an all-true mask once per forward (run_blocks); for a direct call of a block
+            # with one the masked kernel gives the same values, and testing here would synchronise per block
+            meta.attn_mask_checked = True
         txt_attn, img_attn = self.attn(jq, jk, jv, meta)
         if residuals is not None:
             img_res, img_gate, txt_res, txt_gate = residuals[:4]

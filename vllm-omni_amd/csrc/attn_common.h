@@ -80,10 +80,17 @@ __device__ __forceinline__ int xcd_remap(int bid, int total) {
 // software-pipelined kernel with direct global->LDS tile loads (attn_fwd_dma.hip); returns
 // ODIT_ENOTSUP when the tensors cannot be addressed with 32-bit buffer offsets
 // `ws` (may be null) is scratch for the key-split tail; see attn_dma_workspace_bytes.
-int launch_attn_dma(AttnParams& p, int dtype, int D, int nw, hipStream_t stream, void* ws, size_t ws_bytes);
+int launch_attn_dma(AttnParams& p, int dtype, int D, hipStream_t stream, void* ws, size_t ws_bytes);
 
 // bytes of scratch with which launch_attn_dma can split the last, partly filled round of workgroups
 // along the keys (0 when this shape gains nothing from it)
-size_t attn_dma_workspace_bytes(int B, int Sq, int Sk, int H, int D, int nw);
+size_t attn_dma_workspace_bytes(int B, int Sq, int Sk, int H, int D);
+
+
+// whether launch_attn_dma takes a problem with these key/value row strides (elements)
+bool attn_dma_addressable(int Sk, int64_t k_seq_stride, int64_t v_seq_stride);
+
+// text description of the launches launch_attn_dma makes for a shape; returns their number
+int attn_dma_plan(int B, int Sq, int Sk, int H, int D, bool with_workspace, char* text, size_t text_bytes);
 
 }  // namespace odit

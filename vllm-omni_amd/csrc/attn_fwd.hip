@@ -1,299 +1,28 @@
-// K1: non-causal joint (text+image) flash attention forward for gfx950, bf16/fp16 MFMA.
-//
-// Formulation (everything transposed so that softmax statistics stay inside a lane):
+// K1 entry points, and the pointer-addressed attention kernel used when the key/value rows of one
+// (batch, head) span 2 GiB or more and so cannot be reached through 32-bit buffer offsets (the
+// production kernel of attn_fwd_dma.hip). Both kernels share the formulation:
 //     S^T = K Q^T          v_mfma_f32_32x32x16:  A = K tile rows (from LDS), B = Q rows (registers)
 //     O^T = V^T P^T        v_mfma_f32_32x32x16:  A = V^T rows (from LDS),  B = P^T (registers)
 // In the 32x32 accumulator layout lane l owns column (l & 31) — one QUERY — and 16 rows — KEYS
 // 8g + 4(l>>5) + t, g,t in 0..3.  So a query's running max / sum need only in-lane work plus one
 // exchange between lanes l and l^32, and the P^T accumulators are, after conversion to 16-bit,
-// already in B-operand order for the second product as long as V^T is laid out in LDS with the same
+// already in B-operand order for the second product as long as V^T is read from LDS with the same
 // permutation of the summation (key) index.  P never touches LDS.
 //
-// Work decomposition: grid = B * H * ceil(Sq / BM) workgroups, BM = NW * QT * 32 queries; each of the
-// NW wavefronts owns QT tiles of 32 queries and streams all keys in tiles of BN = 64 through a
-// double-buffered LDS stage (K row-major, V transposed on the way in).  Workgroup ids are remapped so
+// Work decomposition: grid = B * H * ceil(Sq / BM) workgroups; each wavefront owns 32 queries and
+// streams all keys in tiles of 64 through a double-buffered LDS stage. Workgroup ids are remapped so
 // that the q-blocks of one (batch, head) — which share K/V — land on the same XCD and hit its L2.
 //
 // Algorithmic work: 4 * B * H * Sq * Sk * D flop; minimum traffic 2 * (2*B*Sq*H*D + 2*B*Sk*Hkv*D) bytes.
 #include "attn_common.h"
 
+#include <string.h>
+
 namespace odit {
 
-template <typename T, int D, int QT, int NW>
-__global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(const AttnParams p) {
-  using M = Mma<T>;
-  using frag = typename M::frag;
-  constexpr int BN = 64;             // keys per tile
-  constexpr int NT = NW * 64;        // threads
-  constexpr int BM = NW * QT * 32;   // queries per workgroup
-  constexpr int KS = D / 16;         // k-steps of the QK^T product
-  constexpr int DT = D / 32;         // 32-row tiles of O^T
-  constexpr int KROW = D + 8;        // K tile row pitch (elements): +16 B skews rows across banks
-  constexpr int VROW = BN + 8;       // V^T tile row pitch
-  constexpr int CPR = D / 8;         // 16-byte chunks per K/V row
-  constexpr int KCH = BN * CPR;      // chunks per K tile
-  constexpr int KPT = (KCH + NT - 1) / NT;
-  constexpr int VIT = 16 * CPR;      // (4-key group, 8-wide d chunk) items per V tile
-  constexpr int VPT = (VIT + NT - 1) / NT;
-
-  __shared__ __attribute__((aligned(16))) T Ks[2][BN * KROW];
-  __shared__ __attribute__((aligned(16))) T Vt[2][D * VROW];
-
-  const int pid = xcd_remap(blockIdx.x, p.total_blocks);
-  const int qb = pid % p.n_qblocks;
-  const int bh = pid / p.n_qblocks;
-  const int h = bh % p.H;
-  const int b = bh / p.H;
-  const int hkv = h / (p.H / p.Hkv);
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int l32 = lane & 31, hh = lane >> 5;
-  const int q0 = qb * BM + wave * (QT * 32);
-
-  const T* qbase = static_cast<const T*>(p.q) + b * p.qs_b + h * p.qs_h;
-  const T* kbase = static_cast<const T*>(p.k) + b * p.ks_b + hkv * p.ks_h;
-  const T* vbase = static_cast<const T*>(p.v) + b * p.vs_b + hkv * p.vs_h;
-
-  // ---- Q fragments stay in registers for the whole kernel ----
-  frag qf[QT][KS];
-#pragma unroll
-  for (int qt = 0; qt < QT; ++qt) {
-    int row = q0 + qt * 32 + l32;
-    row = row < p.Sq ? row : p.Sq - 1;
-    const T* qp = qbase + row * p.qs_s + hh * 8;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      qf[qt][ks] = __builtin_bit_cast(frag, *reinterpret_cast<const u32x4_v*>(qp + ks * 16));
-  }
-
-  u32x4_v kreg[KPT];
-  uint32_t vreg[VPT][4][4];  // [item][key in group][dword]: kept as scalars so it stays in registers
-
-  auto load_tile = [&](int j) {
-#pragma unroll
-    for (int i = 0; i < KPT; ++i) {
-      const int c = tid + i * NT;
-      if (KCH % NT == 0 || c < KCH) {
-        const int row = c / CPR, col = c % CPR;
-        int key = j * BN + row;
-        key = key < p.Sk ? key : p.Sk - 1;
-        kreg[i] = *reinterpret_cast<const u32x4_v*>(kbase + key * p.ks_s + col * 8);
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-      const int it = tid + i * NT;
-      if (VIT % NT == 0 || it < VIT) {
-        const int kg = it & 15, dc = it >> 4;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          int key = j * BN + kg * 4 + r;
-          key = key < p.Sk ? key : p.Sk - 1;
-          const u32x4_v t = *reinterpret_cast<const u32x4_v*>(vbase + key * p.vs_s + dc * 8);
-          vreg[i][r][0] = t.x; vreg[i][r][1] = t.y; vreg[i][r][2] = t.z; vreg[i][r][3] = t.w;
-        }
-      }
-    }
-  };
-
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < KPT; ++i) {
-      const int c = tid + i * NT;
-      if (KCH % NT == 0 || c < KCH) {
-        const int row = c / CPR, col = c % CPR;
-        *reinterpret_cast<u32x4_v*>(&Ks[buf][row * KROW + col * 8]) = kreg[i];
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-      const int it = tid + i * NT;
-      if (VIT % NT == 0 || it < VIT) {
-        const int kg = it & 15, dc = it >> 4;
-        // Position of this 4-key group inside its 16-key block: groups are stored in the order
-        // 0,2,1,3 so that the 8 keys one lane-half feeds to a k-step of the PV product are contiguous.
-        const int m = kg & 3;
-        const int pos = (kg >> 2) * 16 + (((m & 1) << 1) | (m >> 1)) * 4;
-        const uint32_t(&a0)[4] = vreg[i][0];
-        const uint32_t(&a1)[4] = vreg[i][1];
-        const uint32_t(&a2)[4] = vreg[i][2];
-        const uint32_t(&a3)[4] = vreg[i][3];
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          u32x2_v lo, hi;  // d = dc*8 + 2w (low halves) and d + 1 (high halves), keys 0..3 of the group
-          lo.x = (a0[w] & 0xffffu) | (a1[w] << 16);
-          lo.y = (a2[w] & 0xffffu) | (a3[w] << 16);
-          hi.x = (a0[w] >> 16) | (a1[w] & 0xffff0000u);
-          hi.y = (a2[w] >> 16) | (a3[w] & 0xffff0000u);
-          T* dst = &Vt[buf][(dc * 8 + 2 * w) * VROW + pos];
-          *reinterpret_cast<u32x2_v*>(dst) = lo;
-          *reinterpret_cast<u32x2_v*>(dst + VROW) = hi;
-        }
-      }
-    }
-  };
-
-  // ---- running state: one query per (lane, qt) ----
-  f32x16_v o[QT][DT];
-  float m_run[QT], l_run[QT];
-#pragma unroll
-  for (int qt = 0; qt < QT; ++qt) {
-    m_run[qt] = -INFINITY;
-    l_run[qt] = 0.f;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) o[qt][dt][e] = 0.f;
-  }
-
-  const int n_tiles = (p.Sk + BN - 1) / BN;
-  const float c = p.scale_log2;
-  const uint8_t* mrow = p.mask ? p.mask + static_cast<int64_t>(b) * p.Sk : nullptr;
-
-  load_tile(0);
-  store_tile(0);
-  __syncthreads();
-
-  for (int j = 0; j < n_tiles; ++j) {
-    const int buf = j & 1;
-    const bool more = j + 1 < n_tiles;
-    if (more) load_tile(j + 1);
-
-    // ---- S^T = K Q^T ----
-    f32x16_v s[2][QT];
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int qt = 0; qt < QT; ++qt)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) s[kt][qt][e] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt) {
-        const frag a = __builtin_bit_cast(
-            frag, *reinterpret_cast<const u32x4_v*>(&Ks[buf][(kt * 32 + l32) * KROW + ks * 16 + hh * 8]));
-#pragma unroll
-        for (int qt = 0; qt < QT; ++qt) s[kt][qt] = M::run(a, qf[qt][ks], s[kt][qt]);
-      }
-    }
-
-    // ---- exclusions: keys past Sk (last tile) and keys the padding mask removes ----
-    const bool tail = (j + 1) * BN > p.Sk;
-    if (tail || mrow != nullptr) {  // branch-free selects inside
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const int key = j * BN + kt * 32 + g * 8 + hh * 4 + t;
-            const int kc = key < p.Sk ? key : p.Sk - 1;
-            const bool live = (key < p.Sk) & (mrow == nullptr || mrow[kc] != 0);
-#pragma unroll
-            for (int qt = 0; qt < QT; ++qt) {
-              const float x = s[kt][qt][g * 4 + t];
-              s[kt][qt][g * 4 + t] = live ? x : -INFINITY;
-            }
-          }
-    }
-
-    // ---- online softmax, one query per lane per qt ----
-    uint32_t pf[QT][2][2][4];  // P^T as packed 16-bit B fragments: [qt][kt][k-step][dword]
-#pragma unroll
-    for (int qt = 0; qt < QT; ++qt) {
-      float mx = s[0][qt][0];
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[kt][qt][e]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      // Lazy rescaling: exponentials are taken against a reference maximum m_run that is only moved
-      // (and O, l rescaled) when some query of the wavefront has outgrown it by more than 2^8, so P
-      // stays below 256 and the common iteration touches neither O nor l_run's scale.
-      const float m_new = fmaxf(m_run[qt], mx);
-      if (__any((m_new - m_run[qt]) * c > 8.f)) {
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f((m_run[qt] - m_safe) * c);  // first tile: exp2(-inf) = 0
-        l_run[qt] *= alpha;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) o[qt][dt][e] *= alpha;
-        m_run[qt] = m_new;
-      }
-      const float mc = (m_run[qt] == -INFINITY) ? 0.f : m_run[qt] * c;  // -inf: every key so far excluded
-      float psum = 0.f;
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const float pv = __builtin_amdgcn_exp2f(fmaf(s[kt][qt][e], c, -mc));
-          s[kt][qt][e] = pv;
-          psum += pv;
-        }
-#pragma unroll
-        for (int g2 = 0; g2 < 2; ++g2)
-#pragma unroll
-          for (int w = 0; w < 4; ++w)
-            pf[qt][kt][g2][w] = M::pack2(s[kt][qt][g2 * 8 + 2 * w], s[kt][qt][g2 * 8 + 2 * w + 1]);
-      }
-      l_run[qt] += psum;
-    }
-
-    // ---- O^T += V^T P^T ----
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt) {
-#pragma unroll
-        for (int g2 = 0; g2 < 2; ++g2) {
-          const frag a = __builtin_bit_cast(
-              frag, *reinterpret_cast<const u32x4_v*>(
-                        &Vt[buf][(dt * 32 + l32) * VROW + kt * 32 + g2 * 16 + hh * 8]));
-#pragma unroll
-          for (int qt = 0; qt < QT; ++qt) {
-            u32x4_v pb;
-            pb.x = pf[qt][kt][g2][0]; pb.y = pf[qt][kt][g2][1];
-            pb.z = pf[qt][kt][g2][2]; pb.w = pf[qt][kt][g2][3];
-            o[qt][dt] = M::run(a, __builtin_bit_cast(frag, pb), o[qt][dt]);
-          }
-        }
-      }
-    }
-
-    if (more) store_tile(buf ^ 1);
-    __syncthreads();
-  }
-
-  // ---- epilogue: normalise and store O (and LSE) ----
-#pragma unroll
-  for (int qt = 0; qt < QT; ++qt) {
-    const float l_tot = l_run[qt] + __shfl_xor(l_run[qt], 32, 64);
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    const int row = q0 + qt * 32 + l32;
-    if (row < p.Sq) {
-      T* op = out_row_ptr<T>(p, b, h, row);
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          u32x2_v w;
-          w.x = M::pack2(o[qt][dt][g * 4 + 0] * inv, o[qt][dt][g * 4 + 1] * inv);
-          w.y = M::pack2(o[qt][dt][g * 4 + 2] * inv, o[qt][dt][g * 4 + 3] * inv);
-          *reinterpret_cast<u32x2_v*>(op + dt * 32 + g * 8 + hh * 4) = w;
-        }
-      if (p.lse != nullptr && hh == 0) {
-        const float lse = l_tot > 0.f ? m_run[qt] * p.scale + __logf(l_tot) : -INFINITY;
-        p.lse[(static_cast<int64_t>(b) * p.H + h) * p.Sq + row] = lse;
-      }
-    }
-  }
-}
-
-
 // ------------------------------------------------------------------------------------------------
-// Software-pipelined variant (one 32-query tile per wavefront).
+// Pointer-addressed, software-pipelined kernel (one 32-query tile per wavefront; tiles are staged
+// through registers with ordinary 64-bit addressed loads, so any tensor extent works).
 //
 // Per key tile j a wavefront runs two stages:
 //   A:  S(j+1)^T = K(j+1) Q^T on the matrix cores   while the vector ALU turns S(j) into P(j)
@@ -582,43 +311,7 @@ static int launch_attn_pipe(AttnParams& p, hipStream_t stream) {
   return check_launch("odit_attn_fwd");
 }
 
-template <typename T, int D, int QT, int NW>
-static int launch_attn(AttnParams& p, hipStream_t stream) {
-  constexpr int BM = NW * QT * 32;
-  p.n_qblocks = (p.Sq + BM - 1) / BM;
-  const int64_t total = static_cast<int64_t>(p.n_qblocks) * p.H * p.B;
-  if (total > 0x7fffffffll) {
-    set_error("odit_attn_fwd: grid of %lld workgroups is too large", static_cast<long long>(total));
-    return ODIT_EINVAL;
-  }
-  p.total_blocks = static_cast<int>(total);
-  hipLaunchKernelGGL((attn_fwd_kernel<T, D, QT, NW>), dim3(p.total_blocks), dim3(NW * 64), 0, stream,
-                     p);
-  return check_launch("odit_attn_fwd");
-}
-
-// Tile shape per head size; overridable for tuning runs with ODIT_ATTN_VARIANT = "<QT><NW>".
-template <typename T, int D>
-static int dispatch_attn(AttnParams& p, int variant, hipStream_t stream) {
-  switch (variant) {
-    case 14: return launch_attn<T, D, 1, 4>(p, stream);
-    case 18: return launch_attn<T, D, 1, 8>(p, stream);
-    case 24: return launch_attn<T, D, 2, 4>(p, stream);
-    case 28: return launch_attn_pipe<T, D, 8>(p, stream);
-    case 29: return launch_attn_pipe<T, D, 4>(p, stream);
-    default:
-      set_error("odit_attn_fwd: unknown tile variant %d", variant);
-      return ODIT_EINVAL;
-  }
-}
-
 }  // namespace odit
-
-static int attn_variant() {
-  int variant = 34;
-  if (const char* e = getenv("ODIT_ATTN_VARIANT")) variant = atoi(e);
-  return variant;
-}
 
 extern "C" int odit_attn_fwd_ex(const void* q, const void* k, const void* v, const void* v_tail, int k_split,
                                 void* o, void* o_tail, int q_split, const uint8_t* key_mask, float* lse,
@@ -638,10 +331,20 @@ extern "C" int odit_attn_fwd(const void* q, const void* k, const void* v, void* 
 }
 
 extern "C" size_t odit_attn_fwd_workspace_bytes(int B, int Sq, int Sk, int H, int D) {
-  const int variant = attn_variant();
-  if (variant != 34 && variant != 38) return 0;
   if (D != 64 && D != 128) return 0;
-  return odit::attn_dma_workspace_bytes(B, Sq, Sk, H, D, variant == 38 ? 8 : 4);
+  return odit::attn_dma_workspace_bytes(B, Sq, Sk, H, D);
+}
+
+extern "C" int odit_attn_fwd_plan(int B, int Sq, int Sk, int H, int D, int64_t k_seq_stride, int64_t v_seq_stride,
+                                  int with_workspace, char* text, size_t text_bytes) {
+  using namespace odit;
+  ODIT_CHECK_ARG(text != nullptr && text_bytes > 0, "odit_attn_fwd_plan: no text buffer");
+  ODIT_CHECK_ARG(B > 0 && Sq > 0 && Sk > 0 && H > 0 && (D == 64 || D == 128), "odit_attn_fwd_plan: bad shape");
+  if (attn_dma_addressable(Sk, k_seq_stride, v_seq_stride))
+    return attn_dma_plan(B, Sq, Sk, H, D, with_workspace != 0, text, text_bytes);
+  const int64_t units = static_cast<int64_t>((Sq + 255) / 256) * H * B;
+  snprintf(text, text_bytes, "attn_fwd_pipe_kernel units=%lld", static_cast<long long>(units));
+  return 1;
 }
 
 extern "C" int odit_attn_fwd_ex(const void* q, const void* k, const void* v, const void* v_tail, int k_split,
@@ -709,22 +412,17 @@ extern "C" int odit_attn_fwd_ex(const void* q, const void* k, const void* v, con
 
   p.n_full = 0; p.key_chunks = 1; p.tiles_per_chunk = 0; p.ws = nullptr;
 
-  int variant = attn_variant();
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (variant == 38 || variant == 34) {
-    const int rc = launch_attn_dma(p, dtype, D, variant == 38 ? 8 : 4, st, workspace, workspace_bytes);
-    if (rc != ODIT_ENOTSUP) return rc;
-    variant = 28;  // tensors too large for 32-bit buffer offsets: pointer-addressed kernel
-  }
+  const int rc = launch_attn_dma(p, dtype, D, st, workspace, workspace_bytes);
+  if (rc != ODIT_ENOTSUP) return rc;
+  // key/value spans of 2 GiB or more per (batch, head): the pointer-addressed kernel
   if (v_tail != nullptr) {
-    set_error("odit_attn_fwd_ex: values in two tensors need the buffer-addressed kernel (default variant, "
-              "key/value spans below 2 GiB per batch and head)");
+    set_error("odit_attn_fwd_ex: values in two tensors need key/value spans below 2 GiB per batch and head");
     return ODIT_ENOTSUP;
   }
+  constexpr int kPtrWaves = 8;
   if (dtype == ODIT_BF16) {
-    return D == 128 ? dispatch_attn<bf16_t, 128>(p, variant, st)
-                    : dispatch_attn<bf16_t, 64>(p, variant, st);
+    return D == 128 ? launch_attn_pipe<bf16_t, 128, kPtrWaves>(p, st) : launch_attn_pipe<bf16_t, 64, kPtrWaves>(p, st);
   }
-  return D == 128 ? dispatch_attn<f16_t, 128>(p, variant, st)
-                  : dispatch_attn<f16_t, 64>(p, variant, st);
+  return D == 128 ? launch_attn_pipe<f16_t, 128, kPtrWaves>(p, st) : launch_attn_pipe<f16_t, 64, kPtrWaves>(p, st);
 }

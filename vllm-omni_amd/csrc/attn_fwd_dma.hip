@@ -563,21 +563,43 @@ static int launch_dma(AttnParams& p, hipStream_t stream, void* ws, size_t ws_byt
   return check_launch("odit_attn_fwd (merge)");
 }
 
-size_t attn_dma_workspace_bytes(int B, int Sq, int Sk, int H, int D, int nw) {
+constexpr int kDmaWaves = 4;  // wavefronts per workgroup (two workgroups per compute unit)
+
+size_t attn_dma_workspace_bytes(int B, int Sq, int Sk, int H, int D) {
   if (B <= 0 || Sq <= 0 || Sk <= 0 || H <= 0) return 0;
+  constexpr int nw = kDmaWaves;
   const int bm = nw * 32;
   const int64_t units = static_cast<int64_t>((Sq + bm - 1) / bm) * H * B;
   return tail_ws_bytes(plan_tail(units, (Sk + 63) / 64, device_slots(nw)), bm, D);
 }
 
-int launch_attn_dma(AttnParams& p, int dtype, int D, int nw, hipStream_t stream, void* ws, size_t ws_bytes) {
-  // 32-bit buffer offsets: the whole key range of one (batch, head) must be addressable
-  const int64_t k_span = (static_cast<int64_t>(p.Sk) + 64) * p.ks_s * 2;
-  const int64_t v_span = (static_cast<int64_t>(p.Sk) + 64) * p.vs_s * 2;
-  if (k_span >= (1ll << 31) || v_span >= (1ll << 31) || p.ks_s < 0 || p.vs_s < 0) return ODIT_ENOTSUP;
+// 32-bit buffer offsets: the whole key range of one (batch, head) must be addressable
+bool attn_dma_addressable(int Sk, int64_t k_seq_stride, int64_t v_seq_stride) {
+  const int64_t k_span = (static_cast<int64_t>(Sk) + 64) * k_seq_stride * 2;
+  const int64_t v_span = (static_cast<int64_t>(Sk) + 64) * v_seq_stride * 2;
+  return k_span < (1ll << 31) && v_span < (1ll << 31) && k_seq_stride >= 0 && v_seq_stride >= 0;
+}
+
+int attn_dma_plan(int B, int Sq, int Sk, int H, int D, bool with_workspace, char* text, size_t text_bytes) {
+  constexpr int bm = kDmaWaves * 32;
+  const int64_t units = static_cast<int64_t>((Sq + bm - 1) / bm) * H * B;
+  TailPlan t{0, 1, 0};
+  if (with_workspace) t = plan_tail(units, (Sk + 63) / 64, device_slots(kDmaWaves));
+  if (t.rem == 0) {
+    snprintf(text, text_bytes, "attn_fwd_dma_kernel units=%lld", static_cast<long long>(units));
+    return 1;
+  }
+  snprintf(text, text_bytes, "attn_fwd_dma_kernel units=%lld; attn_fwd_dma_kernel(key ranges) units=%d x %d ranges of %d "
+           "tiles; attn_merge_kernel rows=%d", static_cast<long long>(units - t.rem), t.rem, t.key_chunks,
+           t.tiles_per_chunk, t.rem * bm);
+  return units - t.rem > 0 ? 3 : 2;
+}
+
+int launch_attn_dma(AttnParams& p, int dtype, int D, hipStream_t stream, void* ws, size_t ws_bytes) {
+  if (!attn_dma_addressable(p.Sk, p.ks_s, p.vs_s)) return ODIT_ENOTSUP;
 #define ODIT_DMA_GO(T)                                                                     \
-  if (D == 128) return nw == 8 ? launch_dma<T, 128, 8>(p, stream, ws, ws_bytes) : launch_dma<T, 128, 4>(p, stream, ws, ws_bytes); \
-  return nw == 8 ? launch_dma<T, 64, 8>(p, stream, ws, ws_bytes) : launch_dma<T, 64, 4>(p, stream, ws, ws_bytes);
+  if (D == 128) return launch_dma<T, 128, kDmaWaves>(p, stream, ws, ws_bytes);                \
+  return launch_dma<T, 64, kDmaWaves>(p, stream, ws, ws_bytes);
   if (dtype == ODIT_BF16) { ODIT_DMA_GO(bf16_t) }
   ODIT_DMA_GO(f16_t)
 #undef ODIT_DMA_GO

@@ -67,6 +67,11 @@ def _last_contig(t: torch.Tensor, name: str) -> None:
         raise ValueError(f"{name}: last dimension must be contiguous (stride {t.stride(-1)})")
 
 
+# Copies this module makes on the caller's behalf where a kernel could not take the operands as given
+# (a path whose point is having none): counted so that a model run can assert it made none.
+HIDDEN_COPIES: dict[str, int] = {"attn_value_pair_concatenated": 0, "made_contiguous": 0}
+
+
 # --------------------------------------------------------------------------------------------- K1
 def attn_fwd(
     q: torch.Tensor,
@@ -97,9 +102,9 @@ def attn_fwd(
         direct = (v.dim() == 4 and v_tail.dim() == 4 and v.shape[1] % 64 == 0 and 0 < v.shape[1] and v_tail.shape[1] > 0
                   and v.stride(1) == v_tail.stride(1) and v.dtype == v_tail.dtype
                   and all(t.stride(-1) == 1 and all(x % 8 == 0 for x in t.stride()[:3]) and t.data_ptr() % 16 == 0
-                          for t in (v, v_tail))
-                  and attn_reads_value_pairs())
+                          for t in (v, v_tail)))
         if not direct:
+            HIDDEN_COPIES["attn_value_pair_concatenated"] += 1
             v, v_tail = torch.cat([v, v_tail], dim=1), None
     _dev(q, k, v, v_tail, key_mask)
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
@@ -120,6 +125,8 @@ def attn_fwd(
 
     def _prep(t):
         ok = t.stride(-1) == 1 and all(s % 8 == 0 for s in t.stride()[:3]) and t.data_ptr() % 16 == 0
+        if not ok:
+            HIDDEN_COPIES["made_contiguous"] += 1
         return t if ok else t.contiguous()
 
     q, k = _prep(q), _prep(k)
@@ -156,6 +163,7 @@ def attn_fwd(
         float(scale), _code(q), _ptr(ws), 0 if ws is None else ws.numel(), _stream(),
     )
     if rc == -2 and v_tail is not None:  # ODIT_ENOTSUP: spans too large for the kernel that reads value pairs
+        HIDDEN_COPIES["attn_value_pair_concatenated"] += 1
         return attn_fwd(q, k, torch.cat([v, v_tail], dim=1), scale, key_mask=key_mask, return_lse=return_lse,
                         split=split, use_workspace=use_workspace)
     _lib.check(rc, "odit_attn_fwd_ex")
@@ -164,12 +172,18 @@ def attn_fwd(
     return (o, o_tail, lse) if return_lse else (o, o_tail)
 
 
-def attn_reads_value_pairs() -> bool:
-    """Whether the selected attention kernel takes the values as two tensors (the default one does; the
-    earlier variants kept for cross-checks, chosen with ODIT_ATTN_VARIANT, do not)."""
-    import os
-
-    return os.environ.get("ODIT_ATTN_VARIANT", "34") in ("34", "38")
+def attn_plan(B: int, Sq: int, Sk: int, H: int, D: int, k_seq_stride: int | None = None,
+              v_seq_stride: int | None = None, use_workspace: bool = True) -> str:
+    """The launches ``attn_fwd`` makes for a problem, as "<kernel> units=<n>" joined by "; " (kernel names as
+    a profiler reports them). Strides default to those of dense [B,S,H,D] tensors."""
+    lib = _lib.load()
+    buf = _lib.C.create_string_buffer(512)
+    dense = H * D
+    rc = lib.odit_attn_fwd_plan(B, Sq, Sk, H, D, dense if k_seq_stride is None else int(k_seq_stride),
+                                dense if v_seq_stride is None else int(v_seq_stride), int(use_workspace), buf, 512)
+    if rc < 0:
+        _lib.check(rc, "odit_attn_fwd_plan")
+    return buf.value.decode()
 
 
 _ATTN_SCRATCH: dict[tuple[int, int], torch.Tensor] = {}
@@ -408,9 +422,9 @@ def rel_l1_sums(cur: torch.Tensor, prev: torch.Tensor, *, ref_rounding: bool = T
     n = c2.shape[1]
     lib = _lib.load()
     need = int(lib.odit_rel_l1_workspace_bytes(B, n))
-    key = (cur.device.index or 0, need)
+    key = (cur.device.index or 0, _stream())  # launches on one stream are ordered and can share it
     ws = _REL_L1_SCRATCH.get(key)
-    if ws is None:
+    if ws is None or ws.numel() < need:
         ws = torch.empty(max(need, 16), dtype=torch.uint8, device=cur.device)
         _REL_L1_SCRATCH[key] = ws
     sums = torch.empty((B, 2), dtype=torch.float64, device=cur.device)

@@ -56,5 +56,3 @@ class AdaLayerNorm(CustomOp):
             nb = gate.size(0) // 2
             gate_result = torch.where(index.unsqueeze(-1) == 0, gate[:nb].unsqueeze(1), gate[nb:].unsqueeze(1))
         return (out.squeeze(0) if squeeze else out), gate_result
-
-    forward_cuda = forward_hip

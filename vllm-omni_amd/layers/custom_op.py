@@ -1,7 +1,9 @@
-"""CustomOp base: binds the platform's forward at construction, like
-vllm_omni/diffusion/layers/custom_op.py:9-53. On this package's single platform that is always
-``forward_hip``; ``forward_native`` stays an unimplemented hook (the torch restatement of every op
-lives in the test oracle, not in the product)."""
+"""CustomOp base of this package's layers. The reference's ``CustomOp``
+(vllm_omni/diffusion/layers/custom_op.py:9-53) picks one of five per-platform methods when the layer is
+constructed; this package has one platform, so the method bound at construction is always
+``forward_hip``, which every layer here implements on the gfx950 kernels. ``forward_native`` is kept as
+the hook name the reference documents for a plain-torch version, and stays unimplemented: the torch
+restatement of every op lives in the test oracle, not in the product."""
 
 from __future__ import annotations
 
@@ -10,8 +12,6 @@ from typing import Any
 
 import torch.nn as nn
 
-from ..platforms import current_omni_platform
-
 
 class CustomOp(nn.Module):
     def __init__(self) -> None:
@@ -19,31 +19,13 @@ class CustomOp(nn.Module):
         self._forward_method = self.dispatch_forward()
 
     def dispatch_forward(self) -> Callable:
-        plat = current_omni_platform
-        if plat.is_rocm():
-            return self.forward_hip
-        if plat.is_cuda():
-            return self.forward_cuda
-        if plat.is_npu():
-            return self.forward_npu
-        if plat.is_xpu():
-            return self.forward_xpu
-        return self.forward_native
+        return self.forward_hip
 
     def forward(self, *args, **kwargs) -> Any:
         return self._forward_method(*args, **kwargs)
 
+    def forward_hip(self, *args, **kwargs):
+        raise NotImplementedError(f"{type(self).__name__} does not implement forward_hip")
+
     def forward_native(self, *args, **kwargs):
         raise NotImplementedError(f"{type(self).__name__} has no torch-native path in this package")
-
-    def forward_cuda(self, *args, **kwargs):
-        raise NotImplementedError
-
-    def forward_npu(self, *args, **kwargs):
-        raise NotImplementedError
-
-    def forward_xpu(self, *args, **kwargs):
-        raise NotImplementedError
-
-    def forward_hip(self, *args, **kwargs):
-        return self.forward_cuda(*args, **kwargs)

@@ -43,5 +43,3 @@ class RMSNorm(CustomOp):
         kernels.qknorm_rope(x2, None, None, out, None, None, w, None, None, None,
                             eps=self.variance_epsilon, norm_mode=mode)
         return out.reshape(x.shape)
-
-    forward_cuda = forward_hip

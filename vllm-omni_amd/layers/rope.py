@@ -32,5 +32,3 @@ class RotaryEmbedding(CustomOp):
                             norm_mode=ODIT_NORM_NONE, neox=self.is_neox_style,
                             ref_rounding=self.ref_rounding)
         return out
-
-    forward_cuda = forward_hip

@@ -2,8 +2,7 @@
 
 Mirrors the queries the reference makes of ``current_omni_platform``
 (vllm_omni/platforms/__init__.py, platforms/rocm/platform.py:31-67). This package has exactly one
-platform: ROCm on gfx950. Every ``is_*`` query other than ``is_rocm`` is False, so ``CustomOp`` and
-``AttentionImpl`` always bind their ``forward_hip``.
+platform: ROCm on gfx950, so ``CustomOp`` and ``AttentionImpl`` always run their ``forward_hip``.
 """
 
 from __future__ import annotations
@@ -16,15 +15,6 @@ class RocmGfx950Platform:
 
     def is_rocm(self) -> bool:
         return True
-
-    def is_cuda(self) -> bool:
-        return False
-
-    def is_npu(self) -> bool:
-        return False
-
-    def is_xpu(self) -> bool:
-        return False
 
     def get_diffusion_attn_backend_cls(self, selected_backend: str | None, head_size: int) -> str:
         """Qualified class name of the attention backend (platforms/rocm/platform.py:31-67 picks

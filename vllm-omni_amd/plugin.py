@@ -34,10 +34,6 @@ class CompiledHipFlashAttentionImpl(HipFlashAttentionImpl):
     """Same kernel as ``HipFlashAttentionImpl``, reached through the traceable custom op."""
 
     forward_hip = torch_ops.attention_forward_hip
-    forward_cuda = torch_ops.attention_forward_hip
-
-    def forward(self, query, key, value, attn_metadata=None):
-        return self.forward_hip(query, key, value, attn_metadata)
 
 
 class CompiledHipFlashAttentionBackend(HipFlashAttentionBackend):
