@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define ODIT_VERSION 100 /* major*10000 + minor*100 + patch */
+#define ODIT_VERSION 101 /* major*10000 + minor*100 + patch */
 
 enum odit_dtype { ODIT_BF16 = 0, ODIT_F16 = 1, ODIT_F32 = 2 };
 
@@ -207,11 +207,18 @@ int odit_gated_residual(const void* h, const void* y, const void* gate, const fl
  *   vllm_omni/diffusion/cache/teacache/hook.py:214-221
  * ((cur-prev).abs().mean() / (prev.abs().mean() + 1e-8)); the host divides and applies the
  * polynomial. With ODIT_FLAG_REF_ROUNDING the difference is rounded to `dtype` before abs(), as
- * torch does for a bf16 subtraction. Deterministic: fixed-shape two-stage tree, fp64 final stage.
+ * torch does for a bf16 subtraction. One launch. Deterministic: every workgroup leaves an fp32 partial
+ * of a fixed slice, and the workgroup that finishes a row last adds the row's partials in fp64 in slot
+ * order, so the result does not depend on which one that is.
  *
  * cur, prev: [B, n] with row strides cur_stride / prev_stride (elements); n % 8 == 0 not required.
  * sums: double [B,2] on the device.
- * workspace: device scratch of at least odit_rel_l1_workspace_bytes(B, n) bytes, 16-byte aligned.
+ * workspace: device scratch of at least odit_rel_l1_workspace_bytes(B, n) bytes, 16-byte aligned. It
+ *   holds one ticket counter per row and the partials. THE COUNTERS MUST BE ZERO ON ENTRY: zero the
+ *   workspace once after allocating it (hipMemsetAsync, or a fill kernel under graph capture). Every call
+ *   hands the counters back at zero, so one zeroed workspace serves any number of later calls, of any
+ *   (B, n) it is large enough for. Calls that share a workspace must not overlap (same stream, or ordered
+ *   by events).
  */
 size_t odit_rel_l1_workspace_bytes(int B, int64_t n);
 int odit_rel_l1(const void* cur, const void* prev, double* sums, void* workspace,

@@ -65,12 +65,20 @@ static int check_rel_l1(hipStream_t st) {
   const size_t ws = odit_rel_l1_workspace_bytes(B, n);
   HIP_OK(d_cur.alloc(cur.size())); HIP_OK(d_prev.alloc(prev.size())); HIP_OK(d_sums.alloc(2 * B));
   HIP_OK(d_ws.alloc(ws > 0 ? ws : 16));
+  HIP_OK(hipMemset(d_ws.p, 0, ws > 0 ? ws : 16));  // the ticket counters start at zero; calls keep them there
   HIP_OK(hipMemcpy(d_cur.p, cur.data(), cur.size() * 2, hipMemcpyHostToDevice));
   HIP_OK(hipMemcpy(d_prev.p, prev.data(), prev.size() * 2, hipMemcpyHostToDevice));
-  ODIT_OK_OR_FAIL(odit_rel_l1(d_cur.p, d_prev.p, d_sums.p, d_ws.p, ws, B, n, n, n, ODIT_BF16, 0, st));
-  HIP_OK(hipStreamSynchronize(st));
-  double got[4];
-  HIP_OK(hipMemcpy(got, d_sums.p, sizeof(got), hipMemcpyDeviceToHost));
+  double got[4], first[4];
+  for (int rep = 0; rep < 2; ++rep) {  // the second call reuses the workspace as the first one left it
+    ODIT_OK_OR_FAIL(odit_rel_l1(d_cur.p, d_prev.p, d_sums.p, d_ws.p, ws, B, n, n, n, ODIT_BF16, 0, st));
+    HIP_OK(hipStreamSynchronize(st));
+    HIP_OK(hipMemcpy(got, d_sums.p, sizeof(got), hipMemcpyDeviceToHost));
+    if (rep == 0) std::memcpy(first, got, sizeof(got));
+  }
+  if (std::memcmp(first, got, sizeof(got)) != 0) {
+    std::fprintf(stderr, "rel_l1: two calls on one workspace differ\n");
+    return 1;
+  }
   for (int b = 0; b < B; ++b) {
     double sd = 0.0, sp = 0.0;
     for (int64_t i = 0; i < n; ++i) {

@@ -120,7 +120,7 @@ def test_state_manager_contexts():
     sm.set_context("teacache_negative")
     assert sm.get_state().cnt == 0
     sm.set_context("teacache_positive")
-    assert sm.get_state() is a
+    assert sm.get_state() is a and sm.current_context == "teacache_positive"
     sm.reset()
     assert sm.get_state().cnt == 0
 

@@ -71,7 +71,7 @@ class TeaCacheHook(ModelHook):
             sd, sp = sums.cpu()[0].tolist()
             rel = rel_l1_from_sums(sd, sp, modulated_inp.numel(), modulated_inp.dtype)
         compute = self._decide(state, rel)
-        self.decisions.append({"branch": self.state_manager._context, "rel": rel,
+        self.decisions.append({"branch": self.state_manager.current_context, "rel": rel,
                                "acc": state.accumulated_rel_l1_distance, "compute": compute})
         return compute
 

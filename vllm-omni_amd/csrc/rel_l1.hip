@@ -1,14 +1,29 @@
 // K5: TeaCache relative-L1 reduction. One streaming read of `cur` and `prev`
-// (algorithmic traffic 2 * B*n * sizeof(T)), per-batch-row sums, fixed reduction tree:
-//   stage 1  grid (nblk, B): every block reduces one contiguous slice of one row to two fp32 partials
-//   stage 2  grid (B): one workgroup adds the row's partials in fp64 and writes sums[b] = {sum|cur-prev|, sum|prev|}
-// The tree depends only on (B, n), never on timing, so repeated calls give bit-identical sums.
+// (algorithmic traffic 2 * B*n * sizeof(T)), per-batch-row sums, ONE launch, fixed reduction tree:
+//   grid (nblk, B): every workgroup reduces one contiguous slice of one row to two fp32 partials, stores
+//   them, and takes a ticket from the row's counter; the workgroup that draws the row's last ticket adds
+//   the row's nblk partials in fp64, in slot order, and writes sums[b] = {sum|cur-prev|, sum|prev|}.
+// Which workgroup comes last depends on timing, what it computes does not: the tree depends only on
+// (B, n), so repeated calls give bit-identical sums.
+//
+// Scratch layout: kRelL1CounterBytes of ticket counters (one uint32 per row), then the partials
+// (B * nblk float pairs). The counters must be zero when the kernel starts; the last workgroup of every
+// row puts its counter back to zero, so scratch that was zeroed once stays usable.
 #include "odit_common.h"
+
+#include <mutex>
 
 namespace odit {
 
 constexpr int kRelL1MaxBlocksPerRow = 2048;
 constexpr int kRelL1VecsPerThread = 4;
+constexpr int kRelL1MaxRows = 65535;  // grid.y limit
+// rows of the no-allocation entry point, whose scratch is a fixed array in device memory
+constexpr int kRelL1StaticRows = 64;
+
+static inline size_t rel_l1_counter_bytes(int B) {
+  return (static_cast<size_t>(B) * sizeof(uint32_t) + 255) / 256 * 256;
+}
 
 static inline int rel_l1_blocks_per_row(int64_t n) {
   // sized on bf16 vectors (8 elements); fp32 rows simply get twice the vectors per thread
@@ -20,11 +35,10 @@ static inline int rel_l1_blocks_per_row(int64_t n) {
 }
 
 template <typename T, bool REF_ROUND>
-__global__ __launch_bounds__(256) void rel_l1_stage1_kernel(const T* __restrict__ cur,
-                                                            const T* __restrict__ prev,
-                                                            float* __restrict__ partials,
-                                                            int64_t n, int64_t n_vec,
-                                                            int64_t cur_stride, int64_t prev_stride) {
+__global__ __launch_bounds__(256) void rel_l1_kernel(const T* __restrict__ cur, const T* __restrict__ prev,
+                                                     float* partials, uint32_t* counters,
+                                                     double* __restrict__ sums, int64_t n, int64_t n_vec,
+                                                     int64_t cur_stride, int64_t prev_stride) {
   constexpr int EPV = Vec16<T>::N;
   const int b = blockIdx.y;
   const int nblk = gridDim.x;
@@ -71,6 +85,7 @@ __global__ __launch_bounds__(256) void rel_l1_stage1_kernel(const T* __restrict_
   sd = wave_sum(sd);
   sp = wave_sum(sp);
   __shared__ float red[2][4];
+  __shared__ bool last_of_row;
   const int wave = threadIdx.x >> 6;
   if ((threadIdx.x & 63) == 0) { red[0][wave] = sd; red[1][wave] = sp; }
   __syncthreads();
@@ -78,36 +93,47 @@ __global__ __launch_bounds__(256) void rel_l1_stage1_kernel(const T* __restrict_
     float* out = partials + (static_cast<int64_t>(b) * nblk + blockIdx.x) * 2;
     out[0] = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
     out[1] = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+    // release the two stores to the whole device, then draw this workgroup's ticket
+    const uint32_t ticket = __hip_atomic_fetch_add(counters + b, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    last_of_row = ticket == static_cast<uint32_t>(nblk) - 1u;
   }
-}
+  __syncthreads();
+  if (!last_of_row) return;  // uniform over the workgroup
 
-__global__ __launch_bounds__(256) void rel_l1_stage2_kernel(const float* __restrict__ partials,
-                                                            double* __restrict__ sums, int nblk) {
-  const int b = blockIdx.x;
-  const float2* p = reinterpret_cast<const float2*>(partials) + static_cast<int64_t>(b) * nblk;
-  // all loads of a thread are independent; fixed assignment partial i -> thread i % 256
-  double sd = 0.0, sp = 0.0;
+  // ---- last workgroup of row b: every partial of the row is visible after this fence ----
+  __atomic_thread_fence(__ATOMIC_ACQUIRE);  // device scope; orders the loads below after thread 0's ticket
+  const float2* pr = reinterpret_cast<const float2*>(partials) + static_cast<int64_t>(b) * nblk;
+  // fixed assignment partial i -> thread i % 256, all loads of a thread independent
+  double dd = 0.0, dp = 0.0;
   for (int i = threadIdx.x; i < nblk; i += 256) {
-    const float2 v = p[i];
-    sd += v.x;
-    sp += v.y;
+    const float2 v = pr[i];
+    dd += v.x;
+    dp += v.y;
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
-    sd += __shfl_xor(sd, off, 64);
-    sp += __shfl_xor(sp, off, 64);
+    dd += __shfl_xor(dd, off, 64);
+    dp += __shfl_xor(dp, off, 64);
   }
-  __shared__ double red[2][4];
-  if ((threadIdx.x & 63) == 0) { red[0][threadIdx.x >> 6] = sd; red[1][threadIdx.x >> 6] = sp; }
+  __shared__ double red2[2][4];
+  if ((threadIdx.x & 63) == 0) { red2[0][wave] = dd; red2[1][wave] = dp; }
   __syncthreads();
   if (threadIdx.x == 0) {
-    sums[2 * b] = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
-    sums[2 * b + 1] = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+    sums[2 * b] = (red2[0][0] + red2[0][1]) + (red2[0][2] + red2[0][3]);
+    sums[2 * b + 1] = (red2[1][0] + red2[1][1]) + (red2[1][2] + red2[1][3]);
+    // hand the counter back at zero for the next call on this scratch
+    __hip_atomic_store(counters + b, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
+// Puts n ticket counters to zero (a kernel, not a memset: safe to record into a HIP graph).
+__global__ __launch_bounds__(256) void rel_l1_clear_kernel(uint32_t* counters, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) counters[i] = 0u;
+}
+
 template <typename T>
-static int launch_rel_l1(const void* cur, const void* prev, double* sums, float* partials, int B,
+static int launch_rel_l1(const void* cur, const void* prev, double* sums, void* scratch, int B,
                          int64_t n, int64_t cur_stride, int64_t prev_stride, bool ref_round,
                          hipStream_t stream) {
   constexpr int EPV = Vec16<T>::N;
@@ -115,27 +141,28 @@ static int launch_rel_l1(const void* cur, const void* prev, double* sums, float*
                       prev_stride % EPV == 0;
   const int64_t n_vec = vec_ok ? n / EPV : 0;
   const int nblk = rel_l1_blocks_per_row(n);
+  uint32_t* counters = static_cast<uint32_t*>(scratch);
+  float* partials = reinterpret_cast<float*>(static_cast<char*>(scratch) + rel_l1_counter_bytes(B));
   const dim3 grid(nblk, B);
   if (ref_round) {
-    hipLaunchKernelGGL((rel_l1_stage1_kernel<T, true>), grid, dim3(256), 0, stream,
-                       static_cast<const T*>(cur), static_cast<const T*>(prev), partials, n, n_vec,
-                       cur_stride, prev_stride);
+    hipLaunchKernelGGL((rel_l1_kernel<T, true>), grid, dim3(256), 0, stream, static_cast<const T*>(cur),
+                       static_cast<const T*>(prev), partials, counters, sums, n, n_vec, cur_stride, prev_stride);
   } else {
-    hipLaunchKernelGGL((rel_l1_stage1_kernel<T, false>), grid, dim3(256), 0, stream,
-                       static_cast<const T*>(cur), static_cast<const T*>(prev), partials, n, n_vec,
-                       cur_stride, prev_stride);
+    hipLaunchKernelGGL((rel_l1_kernel<T, false>), grid, dim3(256), 0, stream, static_cast<const T*>(cur),
+                       static_cast<const T*>(prev), partials, counters, sums, n, n_vec, cur_stride, prev_stride);
   }
-  int rc = check_launch("odit_rel_l1 (stage 1)");
-  if (rc != ODIT_OK) return rc;
-  hipLaunchKernelGGL(rel_l1_stage2_kernel, dim3(B), dim3(256), 0, stream, partials, sums, nblk);
-  return check_launch("odit_rel_l1 (stage 2)");
+  return check_launch("odit_rel_l1");
+}
+
+static size_t rel_l1_scratch_bytes(int B, int64_t n) {
+  return rel_l1_counter_bytes(B) + static_cast<size_t>(B) * rel_l1_blocks_per_row(n) * 2 * sizeof(float);
 }
 
 }  // namespace odit
 
 extern "C" size_t odit_rel_l1_workspace_bytes(int B, int64_t n) {
   if (B <= 0 || n < 0) return 0;
-  return static_cast<size_t>(B) * odit::rel_l1_blocks_per_row(n) * 2 * sizeof(float);
+  return odit::rel_l1_scratch_bytes(B, n);
 }
 
 extern "C" int odit_rel_l1(const void* cur, const void* prev, double* sums, void* workspace,
@@ -143,7 +170,7 @@ extern "C" int odit_rel_l1(const void* cur, const void* prev, double* sums, void
                            int64_t prev_stride, int dtype, unsigned flags, void* stream) {
   using namespace odit;
   ODIT_CHECK_ARG(cur && prev && sums && workspace, "odit_rel_l1: null pointer argument");
-  ODIT_CHECK_ARG(B > 0 && B <= 65535 && n >= 0, "odit_rel_l1: bad shape B=%d n=%lld", B,
+  ODIT_CHECK_ARG(B > 0 && B <= kRelL1MaxRows && n >= 0, "odit_rel_l1: bad shape B=%d n=%lld", B,
                  static_cast<long long>(n));
   ODIT_CHECK_ARG(aligned16(workspace), "odit_rel_l1: workspace must be 16-byte aligned");
   if (workspace_bytes < odit_rel_l1_workspace_bytes(B, n)) {
@@ -153,8 +180,8 @@ extern "C" int odit_rel_l1(const void* cur, const void* prev, double* sums, void
   }
   const bool rr = (flags & ODIT_FLAG_REF_ROUNDING) && dtype != ODIT_F32;
   ODIT_DISPATCH_DTYPE(dtype, T,
-                      return launch_rel_l1<T>(cur, prev, sums, static_cast<float*>(workspace), B, n,
-                                              cur_stride, prev_stride, rr,
+                      return launch_rel_l1<T>(cur, prev, sums, workspace, B, n, cur_stride, prev_stride, rr,
                                               static_cast<hipStream_t>(stream)));
   return ODIT_OK;
 }
+

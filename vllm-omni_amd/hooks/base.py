@@ -46,6 +46,10 @@ class StateManager:
     def set_context(self, name: str) -> None:
         self._current = name if name else _DEFAULT_CONTEXT
 
+    @property
+    def current_context(self) -> str:
+        return self._current
+
     def get_state(self) -> BaseState:
         try:
             return self._by_context[self._current]

@@ -425,7 +425,8 @@ def rel_l1_sums(cur: torch.Tensor, prev: torch.Tensor, *, ref_rounding: bool = T
     key = (cur.device.index or 0, _stream())  # launches on one stream are ordered and can share it
     ws = _REL_L1_SCRATCH.get(key)
     if ws is None or ws.numel() < need:
-        ws = torch.empty(max(need, 16), dtype=torch.uint8, device=cur.device)
+        # zeroed once: the kernel needs its ticket counters at zero and hands them back at zero
+        ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=cur.device)
         _REL_L1_SCRATCH[key] = ws
     sums = torch.empty((B, 2), dtype=torch.float64, device=cur.device)
     rc = lib.odit_rel_l1(
