@@ -67,6 +67,10 @@ _SIGNATURES = {
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int64,
          C.c_int64, C.c_int64, C.c_int, C.c_uint, C.c_void_p],
     ),
+    "odit_rel_l1_static": (
+        C.c_int,
+        [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_uint, C.c_void_p],
+    ),
     "odit_linear_workspace_bytes": (C.c_size_t, []),
     "odit_linear": (
         C.c_int,

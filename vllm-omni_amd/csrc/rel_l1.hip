@@ -185,3 +185,74 @@ extern "C" int odit_rel_l1(const void* cur, const void* prev, double* sums, void
   return ODIT_OK;
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same reduction for callers that cannot allocate: its scratch is a fixed array in device memory
+// (one copy per GPU the library runs on, held until the process ends).
+namespace odit {
+
+constexpr size_t kRelL1StaticBytes =
+    256 + static_cast<size_t>(kRelL1StaticRows) * kRelL1MaxBlocksPerRow * 2 * sizeof(float);  // 1 MiB + 256 B
+static_assert(kRelL1StaticRows * sizeof(uint32_t) <= 256, "the counters of the static rows fit their 256 bytes");
+
+static __device__ __align__(256) unsigned char scratch[kRelL1StaticBytes];
+
+// The array's name is only a host-side handle; its device address differs per GPU and is looked up once
+// per device, with that device current, and kept.
+static void* static_scratch_ptr(int* status) {
+  constexpr int kMaxDevices = 64;
+  static void* ptrs[kMaxDevices] = {nullptr};
+  static std::mutex mu;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("odit_rel_l1_static: cannot tell the current device (%s)", hipGetErrorString(e));
+    *status = ODIT_ELAUNCH;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (ptrs[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      set_error("odit_rel_l1_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      *status = ODIT_ELAUNCH;
+      return nullptr;
+    }
+    ptrs[dev] = p;
+  }
+  *status = ODIT_OK;
+  return ptrs[dev];
+}
+
+}  // namespace odit
+
+extern "C" int odit_rel_l1_static(const void* cur, const void* prev, double* sums, int B, int64_t n,
+                                  int64_t cur_stride, int64_t prev_stride, int dtype, unsigned flags,
+                                  void* stream) {
+  using namespace odit;
+  ODIT_CHECK_ARG(cur && prev && sums, "odit_rel_l1_static: null pointer argument");
+  ODIT_CHECK_ARG(B > 0 && n >= 0, "odit_rel_l1_static: bad shape B=%d n=%lld", B, static_cast<long long>(n));
+  if (B > kRelL1StaticRows) {
+    set_error("odit_rel_l1_static: B=%d rows exceed the %d rows the built-in scratch holds; use odit_rel_l1 with "
+              "a workspace", B, kRelL1StaticRows);
+    return ODIT_EWORKSPACE;
+  }
+  if (rel_l1_scratch_bytes(B, n) > kRelL1StaticBytes) {  // cannot happen while the row limit holds; kept as the guard
+    set_error("odit_rel_l1_static: %zu bytes of scratch needed, %zu built in", rel_l1_scratch_bytes(B, n),
+              kRelL1StaticBytes);
+    return ODIT_EWORKSPACE;
+  }
+  int rc = ODIT_OK;
+  void* ptr = static_scratch_ptr(&rc);
+  if (ptr == nullptr) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // The array keeps whatever the last call left (normally counters back at zero; not if that call's kernel never
+  // finished): clear this call's counters first. A fill kernel, not a memset, so the pair may be captured in a graph.
+  hipLaunchKernelGGL(rel_l1_clear_kernel, dim3(1), dim3(256), 0, st, static_cast<uint32_t*>(ptr), kRelL1StaticRows);
+  rc = check_launch("odit_rel_l1_static (clear)");
+  if (rc != ODIT_OK) return rc;
+  const bool rr = (flags & ODIT_FLAG_REF_ROUNDING) && dtype != ODIT_F32;
+  ODIT_DISPATCH_DTYPE(dtype, T,
+                      return launch_rel_l1<T>(cur, prev, sums, ptr, B, n, cur_stride, prev_stride, rr, st));
+  return ODIT_OK;
+}
