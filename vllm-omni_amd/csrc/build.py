@@ -21,7 +21,7 @@ PKG = CSRC.parent
 LIB_NAME = "libomni_dit_hip.so"
 LIB_PATH = PKG / LIB_NAME
 OBJ_DIR = CSRC / "build"
-HEADERS = [CSRC / "odit_common.h", CSRC / "attn_common.h", PKG.parent / "include" / "omni_dit.h"]
+HEADERS = [CSRC / "odit_common.h", CSRC / "attn_common.h", CSRC / "attn_tail.h", PKG.parent / "include" / "omni_dit.h"]
 
 # (source file, extra defines, object stem)
 UNITS: list[tuple[str, list[str], str]] = [
