@@ -332,6 +332,53 @@ def test_teacache_decisions_match_oracle_batched_cfg(gpu):
     assert err < 0.25  # bf16-vs-bf16 drift over 12 steps; decisions above are the exact check
 
 
+def test_teacache_decisions_on_the_fused_path(gpu):
+    """The model as bench.py builds it (fused GEMM epilogues, prescaled gate rows, values read in place) under the
+    hook: its decisions must equal the oracle's and those of the reference-rounding build on the same seeds. The
+    extractor rounds the decision tensor like the reference whatever the blocks do, so the only difference between
+    the two builds is the drift of the latents; rel, the accumulated distance and its distance to the threshold
+    are logged per step for both."""
+    from vllm_omni_amd.cache.teacache import TeaCacheBackend
+    from vllm_omni_amd.denoise import DenoiseInputs, diffuse
+
+    steps, thresh = 12, 0.25
+    g = torch.Generator().manual_seed(11)
+    lat0 = torch.randn(1, S_IMG, 64, generator=g).bfloat16()
+    pos = torch.randn(1, S_TXT, 256, generator=g).bfloat16()
+    neg = torch.randn(1, S_TXT, 256, generator=g).bfloat16()
+    runs = {}
+    for name, kw in (("fused", {}), ("ref_rounding", {"ref_rounding": True})):
+        cfg, w, model = _build(gpu, **kw)
+        if name == "fused":
+            model.fuse_modulation()   # as bench.py runs it: all modulation projections of a step in one GEMM
+
+        class Pipe:
+            transformer = model
+
+        backend = TeaCacheBackend({"rel_l1_thresh": thresh})
+        backend.enable(Pipe)
+        backend.refresh(Pipe, steps)
+        with torch.inference_mode():
+            lat = diffuse(model, DenoiseInputs(lat0.to(gpu), pos.to(gpu), neg.to(gpu), IMG_SHAPE), steps,
+                          true_cfg_scale=4.0, cfg_normalize=True)
+        runs[name] = (list(TeaCacheBackend.hook_of(Pipe).decisions), lat.float().cpu())
+    _, log = _oracle_teacache_run(cfg, w, lat0, pos, neg, steps, thresh, torch.bfloat16)
+    fused, rr = runs["fused"][0], runs["ref_rounding"][0]
+    print("step branch            rel(fused)  rel(ref)    acc(fused)  acc(ref)   |acc-thresh| compute", flush=True)
+    for i, (a, b) in enumerate(zip(fused, rr)):
+        if a["rel"] is not None:
+            print(f"{i // 2:4d} {a['branch']:18s} {a['rel']:.6f}  {b['rel']:.6f}  {a['acc']:.6f}  {b['acc']:.6f}  "
+                  f"{abs(a['acc'] - thresh) if a['acc'] > 0 else float('nan'):.6f}   {a['compute']}", flush=True)
+    assert [(d["branch"], d["compute"]) for d in fused] == [(d["branch"], d["compute"]) for d in rr]
+    assert [(d["branch"], d["compute"]) for d in fused] == [("teacache_" + d["branch"], d["compute"]) for d in log]
+    n_skip = sum(1 for d in fused if not d["compute"])
+    assert 0 < n_skip < len(fused)
+    drift = (runs["fused"][1] - runs["ref_rounding"][1]).abs().max().item()
+    print(f"fused vs reference-rounding latents after {steps} steps: max-abs {drift:.4f}; skipped {n_skip}/{len(fused)}",
+          flush=True)
+    assert drift < 0.25
+
+
 def test_fused_modulation_is_bit_identical(gpu):
     """Stacking the 2L modulation projections changes the schedule, not one output bit of a block
     stack fed with the same temb (per-row GEMV results do not depend on how many rows are stacked...

@@ -221,3 +221,42 @@ def test_flux_width_blocks_against_oracle(gpu):
         cos_ab = float(torch.dot(a, b) / (a.norm() * b.norm()))
         print(f"flux-width {name}: max-abs {err:.4f} cosine {cos_ab:.6f} (|x| max {mag:.2f})", flush=True)
         assert err <= 2e-2 * max(1.0, mag / 2) and cos_ab >= 0.9995
+
+
+def test_flux_teacache_decisions_on_the_fused_path(gpu):
+    """The default (fused-epilogue) Flux model under the hook against the oracle and against the reference-rounding
+    build: same 28 decisions; per-step rel / accumulated distance / distance to the threshold logged."""
+    from vllm_omni_amd.cache.teacache import TeaCacheBackend
+    from vllm_omni_amd.denoise import diffuse_flux
+
+    steps, thresh = 28, 0.25
+    runs = {}
+    for name, kw in (("fused", {}), ("ref_rounding", {"ref_rounding": True})):
+        cfg, w, model = _build(gpu, **kw)
+        if name == "fused":
+            model.fuse_modulation()   # as bench.py runs it
+        lat0, txt, pooled, _, gd, img_ids, txt_ids = _inputs(cfg, 1, seed=21)
+
+        class Pipe:
+            transformer = model
+
+        backend = TeaCacheBackend({"rel_l1_thresh": thresh})
+        backend.enable(Pipe)
+        backend.refresh(Pipe, steps)
+        with torch.inference_mode():
+            lat = diffuse_flux(model, lat0.to(gpu), txt.to(gpu), pooled.to(gpu), img_ids.to(gpu), txt_ids.to(gpu),
+                               steps, guidance_scale=3.5)
+        runs[name] = (list(TeaCacheBackend.hook_of(Pipe).decisions), lat.float().cpu())
+    _, log = _oracle_teacache_run(cfg, w, lat0, txt, pooled, gd, img_ids, txt_ids, steps, thresh)
+    fused, rr = runs["fused"][0], runs["ref_rounding"][0]
+    print("step rel(fused)  rel(ref)   rel(oracle) acc(fused) |acc-thresh| compute", flush=True)
+    for i, (a, b, o) in enumerate(zip(fused, rr, log)):
+        if a["rel"] is not None:
+            print(f"{i:4d} {a['rel']:.6f}  {b['rel']:.6f}  {o['rel']:.6f}  {a['acc']:.6f}  "
+                  f"{abs(a['acc'] - thresh) if a['acc'] > 0 else float('nan'):.6f}   {a['compute']}", flush=True)
+    assert [d["compute"] for d in fused] == [d["compute"] for d in rr] == [d["compute"] for d in log]
+    n_skip = sum(1 for d in fused if not d["compute"])
+    print(f"skip rate on the fused path: {n_skip}/{len(fused)}", flush=True)
+    assert 0 < n_skip < len(fused)
+    assert (runs["fused"][1] - runs["ref_rounding"][1]).abs().max().item() < 0.25
+

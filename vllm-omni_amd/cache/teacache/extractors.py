@@ -10,6 +10,8 @@ from typing import Any
 import torch
 import torch.nn as nn
 
+from ... import kernels
+
 
 @dataclass
 class CacheContext:
@@ -70,7 +72,11 @@ def extract_qwen_context(module: nn.Module, hidden_states: torch.Tensor,
                                             additional_t_cond)
     block0 = module.transformer_blocks[0]
     mod1 = block0.img_mod(temb).chunk(2, dim=-1)[0]
-    modulated, _ = block0.img_norm1(img, mod1)
+    shift, scale, _ = mod1.chunk(3, dim=-1)
+    # The decision tensor is always rounded where the reference's torch ops round (one 50 MB elementwise pass
+    # per step), whatever rounding the block stack itself runs with: skip/compute decisions then do not depend
+    # on whether the model was built with fused GEMM epilogues.
+    modulated = kernels.adaln_modulate(img, shift, scale, eps=block0.img_norm1.eps, ref_rounding=True)
     mask = encoder_hidden_states_mask
     return_dict = kwargs.get("return_dict", True)
 
@@ -108,7 +114,10 @@ def extract_flux_context(module: nn.Module, hidden_states: torch.Tensor,
                         f"finish stages); got {type(module).__module__}.{type(module).__name__}")
     img, txt, temb, rotary = module.prepare(hidden_states, encoder_hidden_states, pooled_projections, timestep,
                                             img_ids, txt_ids, guidance)
-    modulated = module.transformer_blocks[0].norm1(img, emb=temb)[0]
+    norm1 = module.transformer_blocks[0].norm1
+    shift, scale = norm1.linear(kernels.silu(temb)).chunk(6, dim=1)[:2]
+    # reference rounding for the decision tensor, whatever the blocks run with (see extract_qwen_context)
+    modulated = kernels.adaln_modulate(img, shift, scale, eps=norm1.eps, ref_rounding=True)
     return_dict = kwargs.get("return_dict", True)
 
     def run_rows(rows: list[int] | None):
