@@ -7,6 +7,7 @@ TFLOP/s for the other kernels on the path, and the CPU oracle timed on the host 
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--blocks N] [--no-cpu] [--no-kernels]
   python bench.py --workload flux|wan [--steps K] [--warmup W]     (the other block families, same protocol)
+  python bench.py --workload flux --teacache 0.25                  (adds the 28-step TeaCache trajectory: skip rate, steps/s)
 """
 
 from __future__ import annotations
@@ -198,6 +199,19 @@ def flux_workload(torch, layers=None):
     gemm = 2.0 * S * Cf * Cf * (n_dual * (3 + 1 + 8) + n_single * (3 + 4 + 5))
     name = (f"Flux-shape MMDiT denoise step: {n_dual} dual + {n_single} single blocks, hidden 3072, 24 heads x 128, "
             f"{s_txt} text + {side * side} image tokens, batch 1 (guidance-distilled), random weights N(0,0.02)")
+    def trajectory(steps):
+        """One whole guidance-distilled denoise trajectory of `steps` Euler steps from lat0 (what TeaCache's
+        decisions are defined on: every step compares its modulated input with the previous step's)."""
+        sg = flow_match_sigmas(steps, side * side)
+        lat = lat0
+        for i in range(steps):
+            t = torch.full((1,), float(sg[i]), device=dev, dtype=torch.bfloat16)
+            out = model(hidden_states=lat, encoder_hidden_states=text, pooled_projections=pooled, timestep=t,
+                        img_ids=img_ids, txt_ids=txt_ids, guidance=guidance, return_dict=False)[0]
+            lat = euler_step(lat, out, float(sg[i]), float(sg[i + 1]))
+        return lat
+
+    step.trajectory = trajectory
     return model, step, lat0, name, gemm, (n_dual, n_single) == (19, 38)
 
 
@@ -257,6 +271,11 @@ def run_secondary(torch, kernels, args):
     ms, flop, n = timer.dominant()
     tf = flop / ms / 1e9
     attn_total = sum(timer.flops) / args.steps
+    teacache = None
+    if args.teacache is not None:
+        if args.workload != "flux":
+            sys.exit("bench.py: --teacache is measured at the Flux shape (BASELINE.json configs[4]): use --workload flux")
+        teacache = teacache_trajectory(torch, model, step, args.teacache, args.steps / elapsed)
     print(json.dumps({
         "metric": f"DiT denoise steps/s, {args.workload} shape (1 GPU)", "value": args.steps / elapsed,
         "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -267,7 +286,40 @@ def run_secondary(torch, kernels, args):
                      "traffic": None, "launches_timed": n, "avg_ms": ms, "flop_per_launch": flop},
         "step_flop": {"gemm": gemm_flop, "attention": attn_total,
                       "achieved_TFLOP/s": (gemm_flop + attn_total) / (elapsed / args.steps) / 1e12},
+        "teacache": teacache,
     }))
+
+
+def teacache_trajectory(torch, model, step, thresh, plain_steps_per_s, steps=28):
+    """BASELINE.json configs[4]: the 28-step trajectory with the TeaCache hook on (relative-L1 threshold `thresh`
+    on the modulated first-block input, the reference's 4th-order polynomial for this model): one untimed
+    trajectory, then the same trajectory timed. Steps/s counts every denoise step, skipped or computed."""
+    from vllm_omni_amd.cache.teacache import TeaCacheBackend
+
+    class Pipe:
+        transformer = model
+
+    backend = TeaCacheBackend({"rel_l1_thresh": float(thresh)})
+    backend.enable(Pipe)
+    with torch.inference_mode():
+        backend.refresh(Pipe, steps)
+        step.trajectory(steps)
+        torch.cuda.synchronize()
+        backend.refresh(Pipe, steps)
+        t0 = time.perf_counter()
+        lat = step.trajectory(steps)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    hook = TeaCacheBackend.hook_of(Pipe)
+    decisions = [bool(d["compute"]) for d in hook.decisions]
+    margins = [abs(d["acc"] - float(thresh)) for d in hook.decisions if d["rel"] is not None and d["acc"] > 0]
+    assert len(decisions) == steps and bool(torch.isfinite(lat.float()).all())
+    skipped = decisions.count(False)
+    return {"rel_l1_thresh": float(thresh), "steps": steps, "skipped": skipped, "skip_rate": skipped / steps,
+            "steps/s": steps / elapsed, "ms_per_step": elapsed * 1e3 / steps, "steps/s_without_cache": plain_steps_per_s,
+            "speedup": steps / elapsed / plain_steps_per_s, "compute_pattern": "".join("C" if c else "s" for c in decisions),
+            "min_distance_to_threshold": min(margins) if margins else None,
+            "data": "synthetic latents, random weights: the skip pattern is this trajectory's, not a trained model's"}
 
 
 def _time_rot(torch, fns, iters=40, warmup=4):
@@ -487,6 +539,9 @@ def main():
                     help="A/B switch: GELU and gated residuals as separate kernels after plain GEMMs")
     ap.add_argument("--autotune", type=int, default=0,
                     help="time the library's kernels for each fused-epilogue GEMM in an untimed first step")
+    ap.add_argument("--teacache", type=float, default=None, metavar="THRESH",
+                    help="with --workload flux: also run the 28-step trajectory under the TeaCache hook with this "
+                         "relative-L1 threshold and report skip rate and steps/s")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
     args = ap.parse_args()
