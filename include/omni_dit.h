@@ -228,7 +228,7 @@ int odit_rel_l1(const void* cur, const void* prev, double* sums, void* workspace
 /* odit_rel_l1 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same arguments and bit-identical
  * sums, without the workspace: the ticket counters and partials live in an array built into the library's
- * device image, 1 MiB + 256 bytes per GPU the library is used on, held until the process ends. It calls no
+ * device image, 2304 bytes per GPU the library is used on, held until the process ends. It calls no
  * allocating routine. Limit: B <= 64 rows (any n); more returns ODIT_EWORKSPACE and enqueues nothing.
  * Two launches: a fill kernel puts the counters to zero (a kernel, not a memset, so the call can be captured),
  * then the reduction. Every call on a GPU shares that GPU's array: calls that may overlap on one GPU

@@ -165,6 +165,12 @@ def test_qwen_rotary_tables_from_integer_positions_equal_the_oracles():
         vid, txt = rope(shapes, [3, 5], "cpu")
         want_v, want_t = oq.qwen_rope_freqs_images(cfg, shapes, txt_len=5, layer3d=layer3d)
         assert vid.dtype == torch.complex64 and torch.equal(vid, want_v) and torch.equal(txt, want_t)
+    # built under a non-default device context (as bench.py builds the model) the tables still come from the host
+    with torch.device("meta"):
+        rope_meta = QwenEmbedRope(theta=cfg.theta, axes_dim=list(cfg.axes_dims_rope), scale_rope=True)
+    vid_m, txt_m = rope_meta([(1, 4, 6)], [5], "cpu")
+    want_v, want_t = oq.qwen_rope_freqs_images(cfg, [(1, 4, 6)], txt_len=5)
+    assert torch.equal(vid_m, want_v) and torch.equal(txt_m, want_t)
     # without centring rows and columns count from zero and text starts after the full extent
     plain = QwenEmbedRope(theta=10000, axes_dim=[4, 6, 6], scale_rope=False)
     vid, txt = plain((1, 2, 3), [2], "cpu")

@@ -141,10 +141,12 @@ class QwenEmbedRope(nn.Module):
         if any(d % 2 for d in self.axes_dim):
             raise ValueError("every rotary axis needs an even number of channels")
         # inverse frequencies of the three axes, side by side: [sum(d) / 2]
+        # table construction runs on the host whatever default device the model is built under
+        cpu = torch.device("cpu")
         self.inv_freq = torch.cat([
-            1.0 / torch.pow(theta, torch.arange(0, d, 2).to(torch.float32).div(d)) for d in self.axes_dim])
-        self.axis_of = torch.repeat_interleave(torch.arange(len(self.axes_dim)),
-                                               torch.tensor([d // 2 for d in self.axes_dim]))
+            1.0 / torch.pow(theta, torch.arange(0, d, 2, device=cpu).to(torch.float32).div(d)) for d in self.axes_dim])
+        self.axis_of = torch.repeat_interleave(torch.arange(len(self.axes_dim), device=cpu),
+                                               torch.tensor([d // 2 for d in self.axes_dim], device=cpu))
         self._tables = lru_cache(maxsize=16)(self._build)
 
     def _table(self, positions: torch.Tensor) -> torch.Tensor:
@@ -155,9 +157,10 @@ class QwenEmbedRope(nn.Module):
     def _image_positions(self, frame: int, height: int, width: int, first_frame: int) -> torch.Tensor:
         r0 = -(height - height // 2) if self.scale_rope else 0
         c0 = -(width - width // 2) if self.scale_rope else 0
-        grid = torch.stack(torch.meshgrid(torch.arange(first_frame, first_frame + frame),
-                                          torch.arange(r0, r0 + height), torch.arange(c0, c0 + width),
-                                          indexing="ij"), dim=-1)
+        cpu = torch.device("cpu")
+        grid = torch.stack(torch.meshgrid(torch.arange(first_frame, first_frame + frame, device=cpu),
+                                          torch.arange(r0, r0 + height, device=cpu),
+                                          torch.arange(c0, c0 + width, device=cpu), indexing="ij"), dim=-1)
         return grid.reshape(-1, 3)
 
     def _build(self, shapes: tuple[tuple[int, int, int], ...], txt_len: int, device: str):
@@ -174,7 +177,7 @@ class QwenEmbedRope(nn.Module):
         if self.layer3d:
             start = max(start, last)
         vid = self._table(torch.cat(pos, dim=0)).to(device)
-        txt = self._table(torch.arange(start, start + txt_len).view(-1, 1).expand(-1, 3)).to(device)
+        txt = self._table(torch.arange(start, start + txt_len, device="cpu").view(-1, 1).expand(-1, 3)).to(device)
         return vid, txt
 
     @staticmethod

@@ -15,8 +15,12 @@
 
 namespace odit {
 
-constexpr int kRelL1MaxBlocksPerRow = 2048;
+constexpr int kRelL1MaxBlocksPerRow = 256;
 constexpr int kRelL1VecsPerThread = 4;
+// Measured at B = 2, n = 12.6 M bf16 (100 MB): 256 workgroups of 1024 threads 21.9 us; 512 x 512 22.4; 1024 x 256
+// 25.9; 3072 x 256 45 us: the tickets are device-scope atomics on one address per row and serialise at ~25 ns each.
+constexpr int kRelL1Threads = 1024;     // threads per workgroup
+constexpr int kRelL1TotalBlocks = 256;  // workgroups of a launch, over all rows (when rows are long enough)
 constexpr int kRelL1MaxRows = 65535;  // grid.y limit
 // rows of the no-allocation entry point, whose scratch is a fixed array in device memory
 constexpr int kRelL1StaticRows = 64;
@@ -25,17 +29,22 @@ static inline size_t rel_l1_counter_bytes(int B) {
   return (static_cast<size_t>(B) * sizeof(uint32_t) + 255) / 256 * 256;
 }
 
-static inline int rel_l1_blocks_per_row(int64_t n) {
-  // sized on bf16 vectors (8 elements); fp32 rows simply get twice the vectors per thread
-  const int64_t per_block = 256ll * kRelL1VecsPerThread * 8;
+static inline int rel_l1_blocks_per_row(int B, int64_t n) {
+  // at least one pass of four 16-byte vectors per thread (sized on 8-element vectors; fp32 rows get twice the
+  // vectors), at most kRelL1TotalBlocks workgroups over all rows: every workgroup ends with one device-scope
+  // atomic on its row's counter, and those serialise
+  const int64_t per_block = static_cast<int64_t>(kRelL1Threads) * kRelL1VecsPerThread * 8;
   int64_t nb = (n + per_block - 1) / per_block;
+  int64_t cap = kRelL1TotalBlocks / (B > 0 ? B : 1);
+  if (cap < 1) cap = 1;
+  if (cap > kRelL1MaxBlocksPerRow) cap = kRelL1MaxBlocksPerRow;
+  if (nb > cap) nb = cap;
   if (nb < 1) nb = 1;
-  if (nb > kRelL1MaxBlocksPerRow) nb = kRelL1MaxBlocksPerRow;
   return static_cast<int>(nb);
 }
 
 template <typename T, bool REF_ROUND>
-__global__ __launch_bounds__(256) void rel_l1_kernel(const T* __restrict__ cur, const T* __restrict__ prev,
+__global__ __launch_bounds__(kRelL1Threads) void rel_l1_kernel(const T* __restrict__ cur, const T* __restrict__ prev,
                                                      float* partials, uint32_t* counters,
                                                      double* __restrict__ sums, int64_t n, int64_t n_vec,
                                                      int64_t cur_stride, int64_t prev_stride) {
@@ -62,19 +71,20 @@ __global__ __launch_bounds__(256) void rel_l1_kernel(const T* __restrict__ cur, 
   // four vector pairs (eight 16-byte loads) in flight per lane before the first use
   constexpr int U = 4;
   int64_t i = v_begin + threadIdx.x;
-  for (; i + (U - 1) * 256 < v_end; i += U * 256) {
+  constexpr int NT = kRelL1Threads;
+  for (; i + (U - 1) * NT < v_end; i += U * NT) {
     Vec16<T> cv[U], pv[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      cv[u] = load16(c + (i + u * 256) * EPV);
-      pv[u] = load16(p + (i + u * 256) * EPV);
+      cv[u] = load16(c + (i + u * NT) * EPV);
+      pv[u] = load16(p + (i + u * NT) * EPV);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) accumulate(cv[u], pv[u]);
   }
-  for (; i < v_end; i += 256) accumulate(load16(c + i * EPV), load16(p + i * EPV));
+  for (; i < v_end; i += NT) accumulate(load16(c + i * EPV), load16(p + i * EPV));
   if (blockIdx.x == 0) {  // scalar tail (also the whole row when vector loads are not possible)
-    for (int64_t i = n_vec * EPV + threadIdx.x; i < n; i += blockDim.x) {
+    for (int64_t i = n_vec * EPV + threadIdx.x; i < n; i += NT) {
       const float pf = to_float(p[i]);
       float d = to_float(c[i]) - pf;
       if (REF_ROUND) d = round_to<T>(d);
@@ -84,43 +94,52 @@ __global__ __launch_bounds__(256) void rel_l1_kernel(const T* __restrict__ cur, 
   }
   sd = wave_sum(sd);
   sp = wave_sum(sp);
-  __shared__ float red[2][4];
+  constexpr int NWAVE = kRelL1Threads / 64;
+  __shared__ float red[2][NWAVE];
   __shared__ bool last_of_row;
   const int wave = threadIdx.x >> 6;
   if ((threadIdx.x & 63) == 0) { red[0][wave] = sd; red[1][wave] = sp; }
   __syncthreads();
   if (threadIdx.x == 0) {
     float* out = partials + (static_cast<int64_t>(b) * nblk + blockIdx.x) * 2;
-    out[0] = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
-    out[1] = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
-    // release the two stores to the whole device, then draw this workgroup's ticket
-    const uint32_t ticket = __hip_atomic_fetch_add(counters + b, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+    for (int w = 0; w < NWAVE; ++w) { o0 += red[0][w]; o1 += red[1][w]; }   // fixed order
+    // The partials go out as device-scope stores (written through to memory, past the XCD-private L2), the wait
+    // lets them land, then the ticket is drawn: the last workgroup's device-scope loads below see every partial
+    // of the row. A release/acquire pair on the ticket would do the same through a write-back and an
+    // invalidation of the whole L2 per workgroup: measured 25.3 us against 21.9 us.
+    __hip_atomic_store(out, o0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(out + 1, o1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(0);
+    const uint32_t ticket = __hip_atomic_fetch_add(counters + b, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     last_of_row = ticket == static_cast<uint32_t>(nblk) - 1u;
   }
   __syncthreads();
   if (!last_of_row) return;  // uniform over the workgroup
 
-  // ---- last workgroup of row b: every partial of the row is visible after this fence ----
-  __atomic_thread_fence(__ATOMIC_ACQUIRE);  // device scope; orders the loads below after thread 0's ticket
+  // ---- last workgroup of row b: every partial of the row has landed (see above) ----
   const float2* pr = reinterpret_cast<const float2*>(partials) + static_cast<int64_t>(b) * nblk;
-  // fixed assignment partial i -> thread i % 256, all loads of a thread independent
+  // fixed assignment partial i -> thread i % NT, all loads of a thread independent
   double dd = 0.0, dp = 0.0;
-  for (int i = threadIdx.x; i < nblk; i += 256) {
-    const float2 v = pr[i];
-    dd += v.x;
-    dp += v.y;
+  for (int i = threadIdx.x; i < nblk; i += NT) {
+    dd += __hip_atomic_load(&pr[i].x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    dp += __hip_atomic_load(&pr[i].y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     dd += __shfl_xor(dd, off, 64);
     dp += __shfl_xor(dp, off, 64);
   }
-  __shared__ double red2[2][4];
+  __shared__ double red2[2][NWAVE];
   if ((threadIdx.x & 63) == 0) { red2[0][wave] = dd; red2[1][wave] = dp; }
   __syncthreads();
   if (threadIdx.x == 0) {
-    sums[2 * b] = (red2[0][0] + red2[0][1]) + (red2[0][2] + red2[0][3]);
-    sums[2 * b + 1] = (red2[1][0] + red2[1][1]) + (red2[1][2] + red2[1][3]);
+    double t0 = 0.0, t1 = 0.0;
+#pragma unroll
+    for (int w = 0; w < NWAVE; ++w) { t0 += red2[0][w]; t1 += red2[1][w]; }
+    sums[2 * b] = t0;
+    sums[2 * b + 1] = t1;
     // hand the counter back at zero for the next call on this scratch
     __hip_atomic_store(counters + b, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
@@ -140,22 +159,22 @@ static int launch_rel_l1(const void* cur, const void* prev, double* sums, void* 
   const bool vec_ok = aligned16(cur) && aligned16(prev) && cur_stride % EPV == 0 &&
                       prev_stride % EPV == 0;
   const int64_t n_vec = vec_ok ? n / EPV : 0;
-  const int nblk = rel_l1_blocks_per_row(n);
+  const int nblk = rel_l1_blocks_per_row(B, n);
   uint32_t* counters = static_cast<uint32_t*>(scratch);
   float* partials = reinterpret_cast<float*>(static_cast<char*>(scratch) + rel_l1_counter_bytes(B));
   const dim3 grid(nblk, B);
   if (ref_round) {
-    hipLaunchKernelGGL((rel_l1_kernel<T, true>), grid, dim3(256), 0, stream, static_cast<const T*>(cur),
+    hipLaunchKernelGGL((rel_l1_kernel<T, true>), grid, dim3(kRelL1Threads), 0, stream, static_cast<const T*>(cur),
                        static_cast<const T*>(prev), partials, counters, sums, n, n_vec, cur_stride, prev_stride);
   } else {
-    hipLaunchKernelGGL((rel_l1_kernel<T, false>), grid, dim3(256), 0, stream, static_cast<const T*>(cur),
+    hipLaunchKernelGGL((rel_l1_kernel<T, false>), grid, dim3(kRelL1Threads), 0, stream, static_cast<const T*>(cur),
                        static_cast<const T*>(prev), partials, counters, sums, n, n_vec, cur_stride, prev_stride);
   }
   return check_launch("odit_rel_l1");
 }
 
 static size_t rel_l1_scratch_bytes(int B, int64_t n) {
-  return rel_l1_counter_bytes(B) + static_cast<size_t>(B) * rel_l1_blocks_per_row(n) * 2 * sizeof(float);
+  return rel_l1_counter_bytes(B) + static_cast<size_t>(B) * rel_l1_blocks_per_row(B, n) * 2 * sizeof(float);
 }
 
 }  // namespace odit
@@ -190,9 +209,11 @@ extern "C" int odit_rel_l1(const void* cur, const void* prev, double* sums, void
 // (one copy per GPU the library runs on, held until the process ends).
 namespace odit {
 
-constexpr size_t kRelL1StaticBytes =
-    256 + static_cast<size_t>(kRelL1StaticRows) * kRelL1MaxBlocksPerRow * 2 * sizeof(float);  // 1 MiB + 256 B
+// 256 bytes of counters + one float pair per workgroup: a launch over at most kRelL1StaticRows rows has at most
+// kRelL1TotalBlocks workgroups (rel_l1_blocks_per_row), so 2304 bytes hold any call this entry point accepts
+constexpr size_t kRelL1StaticBytes = 256 + static_cast<size_t>(kRelL1TotalBlocks) * 2 * sizeof(float);
 static_assert(kRelL1StaticRows * sizeof(uint32_t) <= 256, "the counters of the static rows fit their 256 bytes");
+static_assert(kRelL1StaticRows <= kRelL1TotalBlocks, "one workgroup per row at least");
 
 static __device__ __align__(256) unsigned char scratch[kRelL1StaticBytes];
 
