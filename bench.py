@@ -539,6 +539,9 @@ def main():
                     help="A/B switch: GELU and gated residuals as separate kernels after plain GEMMs")
     ap.add_argument("--autotune", type=int, default=0,
                     help="time the library's kernels for each fused-epilogue GEMM in an untimed first step")
+    ap.add_argument("--linear-engine", choices=("auto", "library", "handwritten"), default="auto",
+                    help="A/B switch for the fused-epilogue projections: auto = the hand-written stream-K kernel where "
+                         "it is expected (or was tuned) to win and the library elsewhere; library = hipBLASLt always")
     ap.add_argument("--teacache", type=float, default=None, metavar="THRESH",
                     help="with --workload flux: also run the 28-step trajectory under the TeaCache hook with this "
                          "relative-L1 threshold and report skip rate and steps/s")
@@ -560,6 +563,7 @@ def main():
     from vllm_omni_amd import gemm_tuning
 
     tuned = gemm_tuning.enable()  # hipBLASLt solution ids picked offline for this model's GEMM shapes
+    kernels.set_linear_engine(args.linear_engine)
     torch.cuda.set_device(0)
     dev = torch.device("cuda:0")
     if args.traffic_probe:

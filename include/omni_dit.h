@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define ODIT_VERSION 101 /* major*10000 + minor*100 + patch */
+#define ODIT_VERSION 102 /* major*10000 + minor*100 + patch */
 
 enum odit_dtype { ODIT_BF16 = 0, ODIT_F16 = 1, ODIT_F32 = 2 };
 
@@ -264,18 +264,28 @@ int odit_silu(const void* x, void* out, int64_t n, int dtype, void* stream);
  *                                                          flux_transformer.py:30-45, wan2_2_transformer.py:92-109
  *   RowParallelLinear followed by `h + gate * y`           qwen_image_transformer.py:794-795, 801, 806,
  *                                                          flux_transformer.py:288-309, wan2_2_transformer.py:661, 673
- * The contraction runs on hipBLASLt's MFMA kernels (it is a plain dense GEMM); this entry point sets the
- * problem up so that bias, activation, gate and residual ride in that kernel's epilogue.
+ * Two engines. Problems with many rows run on hipBLASLt's MFMA kernels (a plain dense GEMM), set up so
+ * that bias, activation, gate and residual ride in that kernel's epilogue. bf16 problems with
+ * 64 <= M <= 1024 rows, K a multiple of 64, N a multiple of 8 and 16-byte aligned rows can also run on a
+ * hand-written stream-K MFMA kernel (csrc/gemm_bf16.hip) that keeps all CUs busy on few output tiles and
+ * takes one gate vector per group of rows in a single launch (odit_linear_rows); it is used where a
+ * tuning call found it faster or, untuned, where K >= 2 N.
  *
  * x [M,K] (row stride ldx), W [N,K] (row stride ldw: torch's nn.Linear weight, or a column range of
  * one), bias [N] or NULL, out [M,N] (row stride ldo). Gated form: residual [M,N] (row stride ldr; may be
  * `out` itself), gate [N] of `dtype` or float32 (gate_dtype), NULL = ones: one call per batch row when
  * the gate differs per batch row. dtype: ODIT_BF16, ODIT_F16 or ODIT_F32 (fp32 accumulation always).
- * workspace: device scratch, 256-byte aligned, for the library's split-K kernels and, in the gated
- * form, two float[N] vectors; odit_linear_workspace_bytes() is a size that suits every kernel. NULL
- * restricts the choice to kernels that need none (not allowed for the gated form).
+ * workspace: device scratch, 256-byte aligned, for the library's split-K kernels, in the gated form two
+ * float[N] vectors, and the hand-written kernel's tile counters and partial tiles;
+ * odit_linear_workspace_bytes() is a size that suits every kernel. A workspace of that size must be
+ * ZERO-FILLED ONCE before its first use and not written by the caller afterwards (the first 16 KB hold
+ * the tile counters, which every call leaves at zero); calls that share a workspace must not overlap
+ * in time (one workspace per stream). A smaller workspace goes to the library alone and rules the
+ * hand-written kernel out; NULL restricts the choice to library kernels that need none (not allowed
+ * for the gated form).
  *
- * odit_linear_tune launches every kernel the library offers for the problem on the given buffers
+ * odit_linear_tune launches every kernel the library offers for the problem, and the hand-written
+ * kernel where it takes the problem, on the given buffers
  * (`out` is overwritten; this call synchronises with the stream), keeps the fastest for later
  * odit_linear calls with the same shape, strides, epilogue and dtype FROM THE SAME HOST THREAD, and
  * reports its time. `flush` (optional device buffer, ideally larger than the last-level cache) is
@@ -301,6 +311,36 @@ int odit_linear_tune(const void* x, const void* w, const void* bias, void* out, 
                      const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int64_t ldr,
                      int epilogue, int gate_dtype, int dtype, void* workspace, size_t workspace_bytes,
                      void* stream, int iters, void* flush, size_t flush_bytes, float* best_us);
+
+/* odit_linear with one gate vector per group of rows_per_gate consecutive rows (the rows of one batch
+ * row of a [B, S, N] activation): gate vector i, gate_stride elements after vector i - 1, scales rows
+ * [i rows_per_gate, (i + 1) rows_per_gate); in the pre-scaled form `bias` is laid out the same way.
+ * rows_per_gate = 0 is odit_linear. One launch when the hand-written kernel takes the problem, one
+ * library launch per group of rows otherwise.
+ */
+int odit_linear_rows(const void* x, const void* w, const void* bias, void* out, const void* residual,
+                     const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int64_t ldr,
+                     int epilogue, int gate_dtype, int dtype, int rows_per_gate, int64_t gate_stride,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* What odit_linear_rows would do with these arguments, without launching anything: *handwritten = 1 when
+ * the hand-written kernel would run, *launches = kernel launches the call would make. */
+int odit_linear_rows_plan(const void* x, const void* w, const void* bias, void* out, const void* residual,
+                          const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int64_t ldr,
+                          int epilogue, int gate_dtype, int dtype, int rows_per_gate, int64_t gate_stride,
+                          void* workspace, size_t workspace_bytes, int* handwritten, int* launches);
+
+int odit_linear_rows_tune(const void* x, const void* w, const void* bias, void* out, const void* residual,
+                          const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int64_t ldr,
+                          int epilogue, int gate_dtype, int dtype, int rows_per_gate, int64_t gate_stride,
+                          void* workspace, size_t workspace_bytes, void* stream, int iters, void* flush,
+                          size_t flush_bytes, float* best_us);
+
+/* Which kernel odit_linear / odit_linear_rows run (process-wide; for measurements and tests):
+ * 0 = the hand-written kernel where it takes the problem and the library elsewhere (the default),
+ * 1 = the library always, 2 = the hand-written kernel always (ODIT_ENOTSUP for problems it does not take).
+ */
+int odit_linear_set_engine(int engine);
 
 /* ---------------------------------------------------------------------------------------------
  * Roofline calibration (no counterpart in the reference): launches `workgroups` workgroups of 8

@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     for name in _declared_functions():
         assert hasattr(lib, name), name
-    assert lib.odit_version() == 101
+    assert lib.odit_version() == 102
 
 
 def _strides(*v):

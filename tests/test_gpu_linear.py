@@ -116,7 +116,8 @@ def test_linear_prescaled_gate_rows_and_autotune(gpu):
     finally:
         kernels.set_linear_autotune(0)
     torch.testing.assert_close(tuned.float(), per_call.float(), atol=4e-2, rtol=2e-2)
-    assert any(k[1:4] == (S, N, K) for k in kernels.linear_tuning_report())
+    # the tuning record is keyed by the whole problem: all B * S rows, S rows per gate vector
+    assert any(k[1:4] == (B * S, N, K) and k[-1] == S for k in kernels.linear_tuning_report())
     with pytest.raises(TypeError):
         kernels.linear(xg, wg, None, residual=hg, gate=gg, prescaled=True)
 
@@ -165,3 +166,93 @@ def test_linear_argument_errors(gpu):
         kernels.linear(x.to(gpu), w.to(gpu), b.to(gpu), gate=torch.ones(16, device=gpu, dtype=torch.bfloat16))
     with pytest.raises(RuntimeError):
         kernels.linear(x, w, b)  # CPU tensors: no fallback
+
+
+# ---------------------------------------------------------------------------- hand-written stream-K kernel
+@pytest.fixture
+def handwritten(gpu):
+    from vllm_omni_amd import kernels
+
+    kernels.set_linear_engine("handwritten")
+    yield kernels
+    kernels.set_linear_engine("auto")
+
+
+def _counters_are_zero(kernels):
+    return all(int(ws[:16384].view(torch.int32).abs().max().item()) == 0 for ws in kernels._LINEAR_SCRATCH.values())
+
+
+@pytest.mark.parametrize("M,N,K", [
+    (512, 768, 1024),    # 4 row tiles x 4 feature tiles
+    (200, 392, 448),     # ragged row and feature tiles (N a multiple of 8 only)
+    (64, 192, 64),       # one tile, one step
+    (1024, 200, 4096),   # 8 row tiles, 2 feature tiles, every tile shared by 16 workgroups
+    (512, 3072, 3072),   # text-stream output projection of the headline workload
+])
+def test_streamk_gemm_matches_fp64_product(handwritten, gpu, M, N, K):
+    x, w, b = _mk(M, N, K, torch.bfloat16, seed=M + N)
+    print(f"stream-K {M}x{N}x{K}", flush=True)
+    xg, wg, bg = x.to(gpu), w.to(gpu), b.to(gpu)
+    got = handwritten.linear(xg, wg, bg)
+    torch.testing.assert_close(got.double().cpu(), _ref(x, w, b), atol=2e-2, rtol=2e-2)
+    again = handwritten.linear(xg, wg, bg)
+    assert torch.equal(got, again), "the order of the partial sums must not depend on arrival order"
+    assert _counters_are_zero(handwritten)
+    got = handwritten.linear(xg, wg, None, activation="gelu_tanh")
+    torch.testing.assert_close(got.double().cpu(), ops.gelu_tanh(_ref(x, w, None)), atol=2e-2, rtol=2e-2)
+    # agreement with the library kernel on the same operands (both accumulate in fp32)
+    handwritten.set_linear_engine("library")
+    lib = handwritten.linear(xg, wg, bg)
+    handwritten.set_linear_engine("handwritten")
+    torch.testing.assert_close(handwritten.linear(xg, wg, bg).float(), lib.float(), atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("gate_dtype", [torch.bfloat16, torch.float32])
+def test_streamk_gemm_gates_per_batch_row_in_one_launch(handwritten, gpu, gate_dtype):
+    B, S, N, K = 2, 256, 384, 1536
+    x, w, b = _mk(S, N, K, torch.bfloat16, seed=21, lead=(B,))
+    g = torch.Generator().manual_seed(22)
+    h = torch.randn(B, S, N, generator=g).bfloat16()
+    mod = torch.randn(B, 6 * N, generator=g).to(gate_dtype)   # the gate is a column range of a wider tensor
+    gate = mod[:, 2 * N:3 * N]
+    want = h.double() + gate.double()[:, None, :] * _ref(x, w, b)
+    xg, wg, bg, hg, mg = (t.to(gpu) for t in (x, w, b, h, mod))
+    got = handwritten.linear(xg, wg, bg, residual=hg, gate=mg[:, 2 * N:3 * N])
+    torch.testing.assert_close(got.double().cpu(), want, atol=4e-2, rtol=2e-2)
+    assert torch.equal(hg.cpu(), h)
+    h2 = hg.clone()
+    inplace = handwritten.linear(xg, wg, bg, residual=h2, gate=mg[:, 2 * N:3 * N], out=h2)
+    assert inplace.data_ptr() == h2.data_ptr() and torch.equal(inplace, got)
+    if gate_dtype == torch.float32:
+        g32 = mg[:, 2 * N:3 * N]
+        gb = torch.zeros_like(mg)                      # gate * bias rows with the gate's row stride
+        gb[:, 2 * N:3 * N] = g32 * bg.float()
+        pre = handwritten.linear(xg, wg, None, residual=hg, gate=g32, gate_bias=gb[:, 2 * N:3 * N], prescaled=True)
+        torch.testing.assert_close(pre.double().cpu(), want, atol=4e-2, rtol=2e-2)
+    assert _counters_are_zero(handwritten)
+
+
+def test_streamk_gemm_refuses_what_it_does_not_take(handwritten, gpu):
+    from vllm_omni_amd._lib import OmniDitKernelError
+
+    x, w, b = _mk(77, 200, 136, torch.bfloat16)      # K not a multiple of 64
+    with pytest.raises(OmniDitKernelError):
+        handwritten.linear(x.to(gpu), w.to(gpu), b.to(gpu))
+    x, w, b = _mk(4096, 256, 256, torch.bfloat16)    # too many rows: the library's large tiles win there
+    with pytest.raises(OmniDitKernelError):
+        handwritten.linear(x.to(gpu), w.to(gpu), b.to(gpu))
+    handwritten.set_linear_engine("auto")
+    got = handwritten.linear(x.to(gpu), w.to(gpu), b.to(gpu))
+    torch.testing.assert_close(got.double().cpu(), _ref(x, w, b), atol=2e-2, rtol=2e-2)
+
+
+def test_linear_tune_compares_both_engines(gpu):
+    from vllm_omni_amd import kernels
+
+    x, w, b = _mk(512, 768, 3072, torch.bfloat16, seed=31)
+    xg, wg, bg = x.to(gpu), w.to(gpu), b.to(gpu)
+    us = kernels.linear(xg, wg, bg, tune_iters=5)
+    print(f"tuned 512x768x3072: best of both engines {us:.1f} us", flush=True)
+    assert 0 < us < 1e4
+    got = kernels.linear(xg, wg, bg)
+    torch.testing.assert_close(got.double().cpu(), _ref(x, w, b), atol=2e-2, rtol=2e-2)

@@ -100,9 +100,10 @@ class FeedForward(nn.Module):
                                 fused=self.fused, ref_rounding=ref_rounding, pre=pre)
 
 
-# The gate differs per batch entry, so the fused form is one GEMM per entry: below this many rows per
-# entry (the 256-token text stream of a CFG batch: two GEMMs of 256 rows) one GEMM over all entries plus
-# the gated-residual kernel is faster (measured: 1.2 ms of a 135 ms step).
+# The gate differs per batch entry. The hand-written GEMM takes one gate vector per batch entry in one
+# launch; the library needs one GEMM per entry, and below this many rows per entry (the 256-token text
+# stream of a CFG batch: two GEMMs of 256 rows) one library GEMM over all entries plus the
+# gated-residual kernel is faster than that (measured: 1.2 ms of a 135 ms step).
 FUSE_MIN_ROWS = 1024
 
 
@@ -114,12 +115,16 @@ def project_residual(lin: nn.Linear, x: torch.Tensor, residual: torch.Tensor, ga
     gate * bias [B,N] or None) made by the caller for all blocks at once replaces ``gate`` on the fused path."""
     per_token_gate = gate is not None and gate.dim() == 3 and gate.shape[1] != 1
     few_rows = gate is not None and x.dim() == 3 and x.shape[0] > 1 and x.shape[1] < FUSE_MIN_ROWS
-    if (fused and not ref_rounding and not per_token_gate and not few_rows and x.dtype != torch.float32
+    if (fused and not ref_rounding and not per_token_gate and x.dtype != torch.float32
             and x.is_contiguous() and residual.is_contiguous()):
         if pre is not None:
-            return kernels.linear(x, lin.weight, None, residual=residual, gate=pre[0], gate_bias=pre[1],
-                                  prescaled=True, out=out)
-        return kernels.linear(x, lin.weight, lin.bias, residual=residual, gate=gate, out=out)
+            args = dict(residual=residual, gate=pre[0], gate_bias=pre[1], prescaled=True)
+            bias = None
+        else:
+            args = dict(residual=residual, gate=gate)
+            bias = lin.bias
+        if not few_rows or kernels.linear(x, lin.weight, bias, plan_only=True, **args)[0]:
+            return kernels.linear(x, lin.weight, bias, out=out, **args)
     return kernels.gated_residual(residual, lin(x), gate, out=out, ref_rounding=ref_rounding)
 
 

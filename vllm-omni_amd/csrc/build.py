@@ -21,7 +21,7 @@ PKG = CSRC.parent
 LIB_NAME = "libomni_dit_hip.so"
 LIB_PATH = PKG / LIB_NAME
 OBJ_DIR = CSRC / "build"
-HEADERS = [CSRC / "odit_common.h", CSRC / "attn_common.h", CSRC / "attn_tail.h", PKG.parent / "include" / "omni_dit.h"]
+HEADERS = [CSRC / "odit_common.h", CSRC / "attn_common.h", CSRC / "attn_tail.h", CSRC / "gemm_bf16.h", PKG.parent / "include" / "omni_dit.h"]
 
 # (source file, extra defines, object stem)
 UNITS: list[tuple[str, list[str], str]] = [
@@ -35,6 +35,7 @@ UNITS: list[tuple[str, list[str], str]] = [
     ("attn_fwd.hip", [], "attn_fwd"),
     ("attn_fwd_dma.hip", [], "attn_fwd_dma"),
     ("linear.hip", [], "linear"),
+    ("gemm_bf16.hip", [], "gemm_bf16"),
     ("probe.hip", [], "probe"),
 ]
 

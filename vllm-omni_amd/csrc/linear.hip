@@ -12,11 +12,13 @@
 // K x N (ld = ldw, transposed), B = x stored K x M (ld = ldx): the bias and the alpha vector run along
 // D's rows, i.e. along the N output features, as needed.
 #include "odit_common.h"
+#include "gemm_bf16.h"
 
 #include <hipblaslt/hipblaslt.h>
 #include <hipblaslt/hipblaslt-ext.hpp>
 
 #include <algorithm>
+#include <atomic>
 #include <unordered_map>
 #include <vector>
 
@@ -67,6 +69,9 @@ struct LinPlan {
 struct LinState {
   hipblasLtHandle_t handle[64] = {nullptr};
   std::unordered_map<LinKey, LinPlan, LinKeyHash> plans;
+  // problems for which a tuning call has compared the hand-written kernel with the library:
+  // true = the hand-written kernel won (key: the whole problem, rows_per_gate in the lda field)
+  std::unordered_map<LinKey, bool, LinKeyHash> handwritten_wins;
 };
 static thread_local LinState g_lin;
 
@@ -141,6 +146,10 @@ static int lin_plan(const LinKey& key, LinPlan** out) {
   *out = &ins.first->second;
   return ODIT_OK;
 }
+
+// 0 = the hand-written kernel where it takes the problem, else the library; 1 = library only;
+// 2 = hand-written only (problems it does not take fail with ODIT_ENOTSUP)
+static std::atomic<int> g_engine{0};
 
 struct LinCall {
   const void *x, *w, *bias, *residual, *gate;
@@ -266,53 +275,171 @@ static int lin_check(const LinCall& c) {
 
 }  // namespace odit
 
-extern "C" size_t odit_linear_workspace_bytes(void) { return static_cast<size_t>(64) << 20; }
+// Workspace split: a workspace large enough starts with the hand-written kernel's scratch (tile
+// counters that are zero between calls, partial-tile slots); the rest is the library's.
+static void lin_split_ws(void* ws, size_t bytes, void** sk, void** lib, size_t* lib_bytes) {
+  if (ws != nullptr && bytes >= odit::kGemmScratchBytes + (static_cast<size_t>(1) << 20)) {
+    *sk = ws;
+    *lib = static_cast<char*>(ws) + odit::kGemmScratchBytes;
+    *lib_bytes = bytes - odit::kGemmScratchBytes;
+  } else {
+    *sk = nullptr;
+    *lib = ws;
+    *lib_bytes = bytes;
+  }
+}
 
-extern "C" int odit_linear(const void* x, const void* w, const void* bias, void* out, const void* residual,
-                           const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
-                           int64_t ldr, int epilogue, int gate_dtype, int dtype, void* workspace,
-                           size_t workspace_bytes, void* stream) {
+static int lin_run_library(const odit::LinCall& c) {
   using namespace odit;
-  LinCall c{x, w, bias, residual, gate, out, M, N, K, ldx, ldw, ldo, ldr, epilogue, gate_dtype, dtype,
-            workspace, workspace_bytes, static_cast<hipStream_t>(stream)};
-  int rc = lin_check(c);
-  if (rc != ODIT_OK || M == 0) return rc;
   hipblasLtHandle_t h;
   LinPlan* p;
   const void *alpha, *cptr;
   void* lws;
   size_t lws_bytes;
-  rc = lin_prepare(c, &h, &p, &alpha, &cptr, &lws, &lws_bytes);
+  int rc = lin_prepare(c, &h, &p, &alpha, &cptr, &lws, &lws_bytes);
   if (rc != ODIT_OK) return rc;
   if (!p->have_algo || p->algo_ws > lws_bytes) {
     rc = lin_default_algo(h, *p, lws_bytes);
     if (rc != ODIT_OK) return rc;
   }
   const float beta = lin_is_residual(c) ? 1.f : 0.f;
-  ODIT_LT(hipblasLtMatmul(h, p->desc, alpha, w, p->a, x, p->b, &beta, cptr, p->c, out, p->d, &p->algo, lws,
+  ODIT_LT(hipblasLtMatmul(h, p->desc, alpha, c.w, p->a, c.x, p->b, &beta, cptr, p->c, c.out, p->d, &p->algo, lws,
                           lws_bytes, c.stream));
   return ODIT_OK;
 }
 
-extern "C" int odit_linear_tune(const void* x, const void* w, const void* bias, void* out, const void* residual,
+static odit::GemmCall lin_gemm_call(const odit::LinCall& c, int rows_per_gate, int64_t ldg) {
+  odit::GemmCall g;
+  g.x = c.x; g.w = c.w; g.bias = c.bias; g.residual = c.residual; g.gate = c.gate; g.out = c.out;
+  g.M = c.M; g.N = c.N; g.K = c.K;
+  g.ldx = c.ldx; g.ldw = c.ldw; g.ldo = c.ldo; g.ldr = c.ldr;
+  g.epilogue = c.epilogue;
+  g.gate_f32 = c.gate_dtype == ODIT_F32 ? 1 : 0;
+  g.rows_per_gate = rows_per_gate;
+  g.ldg = ldg;
+  return g;
+}
+
+// key of the whole problem for the record of which engine won a tuning run
+static odit::LinKey lin_engine_key(int dev, const odit::LinCall& c, int rows_per_gate) {
+  return odit::LinKey{dev, c.M, c.N, c.K, c.epilogue * 4 + (c.bias != nullptr ? 1 : 0) + (c.gate != nullptr ? 2 : 0),
+                      c.dtype, rows_per_gate, c.ldx, c.ldw, c.ldo};
+}
+
+// Without a tuning record the hand-written kernel is used where the reduction is long against the
+// number of output tiles (K >= 2 N: the library's choices split K badly there, measured 58 vs 72 us at
+// M=512, N=3072, K=12288) and the library elsewhere.
+static bool lin_prefers_handwritten(int dev, const odit::LinCall& c, int rows_per_gate) {
+  const auto it = odit::g_lin.handwritten_wins.find(lin_engine_key(dev, c, rows_per_gate));
+  if (it != odit::g_lin.handwritten_wins.end()) return it->second;
+  return c.K >= 2 * c.N;
+}
+
+extern "C" size_t odit_linear_workspace_bytes(void) {
+  return odit::kGemmScratchBytes + (static_cast<size_t>(64) << 20);
+}
+
+extern "C" int odit_linear_set_engine(int engine) {
+  if (engine < 0 || engine > 2) { odit::set_error("odit_linear_set_engine: engine must be 0, 1 or 2"); return ODIT_EINVAL; }
+  odit::g_engine.store(engine);
+  return ODIT_OK;
+}
+
+extern "C" int odit_linear_rows(const void* x, const void* w, const void* bias, void* out, const void* residual,
                                 const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
-                                int64_t ldr, int epilogue, int gate_dtype, int dtype, void* workspace,
-                                size_t workspace_bytes, void* stream, int iters, void* flush,
-                                size_t flush_bytes, float* best_us) {
+                                int64_t ldr, int epilogue, int gate_dtype, int dtype, int rows_per_gate,
+                                int64_t gate_stride, void* workspace, size_t workspace_bytes, void* stream) {
   using namespace odit;
+  void *sk, *lib;
+  size_t lib_bytes;
+  lin_split_ws(workspace, workspace_bytes, &sk, &lib, &lib_bytes);
   LinCall c{x, w, bias, residual, gate, out, M, N, K, ldx, ldw, ldo, ldr, epilogue, gate_dtype, dtype,
-            workspace, workspace_bytes, static_cast<hipStream_t>(stream)};
+            lib, lib_bytes, static_cast<hipStream_t>(stream)};
+  int rc = lin_check(c);
+  if (rc != ODIT_OK || M == 0) return rc;
+  ODIT_CHECK_ARG(rows_per_gate >= 0 && (rows_per_gate == 0 || gate_stride >= 0),
+                 "odit_linear_rows: rows_per_gate and gate_stride must not be negative");
+  const bool per_rows = lin_is_residual(c) && gate != nullptr && rows_per_gate > 0 && rows_per_gate < M;
+  const int engine = g_engine.load();
+  const GemmCall g = lin_gemm_call(c, per_rows ? rows_per_gate : 0, per_rows ? gate_stride : 0);
+  const bool takes = sk != nullptr && gemm_streamk_takes(g, dtype);
+  if (engine == 2 && !takes) {
+    set_error("odit_linear: the hand-written kernel does not take this problem (M=%d N=%d K=%d, workspace %zu bytes)",
+              M, N, K, workspace_bytes);
+    return ODIT_ENOTSUP;
+  }
+  if (takes && engine != 1) {
+    int dev = 0;
+    if (engine == 2 || (hipGetDevice(&dev) == hipSuccess && lin_prefers_handwritten(dev, c, g.rows_per_gate)))
+      return launch_gemm_streamk(g, sk, c.stream);
+  }
+  if (!per_rows) return lin_run_library(c);
+  // the library's epilogue takes one gate vector per launch: one launch per group of rows
+  const size_t esz = dtype == ODIT_F32 ? 4 : 2, gsz = gate_dtype == ODIT_F32 ? 4 : esz;
+  for (int r0 = 0; r0 < M; r0 += rows_per_gate) {
+    LinCall cg = c;
+    const int64_t grp = r0 / rows_per_gate;
+    cg.M = M - r0 < rows_per_gate ? M - r0 : rows_per_gate;
+    cg.x = static_cast<const char*>(x) + static_cast<size_t>(r0) * ldx * esz;
+    cg.out = static_cast<char*>(out) + static_cast<size_t>(r0) * ldo * esz;
+    cg.residual = static_cast<const char*>(residual) + static_cast<size_t>(r0) * ldr * esz;
+    cg.gate = static_cast<const char*>(gate) + static_cast<size_t>(grp * gate_stride) * gsz;
+    if (epilogue == ODIT_EPI_GATED_RESIDUAL_PRE && bias != nullptr)
+      cg.bias = static_cast<const char*>(bias) + static_cast<size_t>(grp * gate_stride) * 4;
+    rc = lin_run_library(cg);
+    if (rc != ODIT_OK) return rc;
+  }
+  return ODIT_OK;
+}
+
+extern "C" int odit_linear_rows_plan(const void* x, const void* w, const void* bias, void* out, const void* residual,
+                                     const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
+                                     int64_t ldr, int epilogue, int gate_dtype, int dtype, int rows_per_gate,
+                                     int64_t gate_stride, void* workspace, size_t workspace_bytes, int* handwritten,
+                                     int* launches) {
+  using namespace odit;
+  void *sk, *lib;
+  size_t lib_bytes;
+  lin_split_ws(workspace, workspace_bytes, &sk, &lib, &lib_bytes);
+  LinCall c{x, w, bias, residual, gate, out, M, N, K, ldx, ldw, ldo, ldr, epilogue, gate_dtype, dtype,
+            lib, lib_bytes, nullptr};
   int rc = lin_check(c);
   if (rc != ODIT_OK) return rc;
-  ODIT_CHECK_ARG(M > 0 && iters > 0, "odit_linear_tune: needs M > 0 and iters > 0");
+  ODIT_CHECK_ARG(handwritten != nullptr && launches != nullptr, "odit_linear_rows_plan: null result pointers");
+  const bool per_rows = lin_is_residual(c) && gate != nullptr && rows_per_gate > 0 && rows_per_gate < M;
+  const int engine = g_engine.load();
+  const GemmCall g = lin_gemm_call(c, per_rows ? rows_per_gate : 0, per_rows ? gate_stride : 0);
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  const bool takes = M > 0 && sk != nullptr && gemm_streamk_takes(g, dtype);
+  const bool own = takes && engine != 1 && (engine == 2 || lin_prefers_handwritten(dev, c, g.rows_per_gate));
+  *handwritten = own ? 1 : 0;
+  *launches = M == 0 ? 0 : (own || !per_rows ? 1 : (M + rows_per_gate - 1) / rows_per_gate);
+  if (!own && lin_needs_prep(c)) *launches *= 2;  // plus the [N]-sized gate-vector launch of the library form
+  return ODIT_OK;
+}
+
+extern "C" int odit_linear(const void* x, const void* w, const void* bias, void* out, const void* residual,
+                           const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
+                           int64_t ldr, int epilogue, int gate_dtype, int dtype, void* workspace,
+                           size_t workspace_bytes, void* stream) {
+  return odit_linear_rows(x, w, bias, out, residual, gate, M, N, K, ldx, ldw, ldo, ldr, epilogue, gate_dtype, dtype, 0,
+                          0, workspace, workspace_bytes, stream);
+}
+
+// Times the library's kernels for problem c (cold caches before every timed launch when a flush buffer
+// is given: in a model every projection has its own weights, which are never cache-resident, so
+// back-to-back launches on one weight would rank the kernels wrongly) and keeps the fastest in the plan.
+static int lin_tune_library(const odit::LinCall& c, int iters, void* flush, size_t flush_bytes, float* best_us) {
+  using namespace odit;
   hipblasLtHandle_t h;
   LinPlan* p;
   const void *alpha, *cptr;
   void* lws;
   size_t lws_bytes;
-  rc = lin_prepare(c, &h, &p, &alpha, &cptr, &lws, &lws_bytes);
+  int rc = lin_prepare(c, &h, &p, &alpha, &cptr, &lws, &lws_bytes);
   if (rc != ODIT_OK) return rc;
-  const hipDataType t = lin_type(dtype);
+  const hipDataType t = lin_type(c.dtype);
   std::vector<hipblasLtMatmulHeuristicResult_t> all;
   ODIT_LT(hipblaslt_ext::getAllAlgos(h, hipblaslt_ext::GemmType::HIPBLASLT_GEMM, HIPBLAS_OP_T, HIPBLAS_OP_N, t, t, t, t,
                                      HIPBLAS_COMPUTE_32F, all));
@@ -324,18 +451,16 @@ extern "C" int odit_linear_tune(const void* x, const void* w, const void* bias, 
   }
   float best = 1e30f;
   int n_ok = 0;
-  // Every timed launch starts from cold caches when a flush buffer is given (it is overwritten in
-  // between, outside the timed interval): in a model every projection has its own weights, which are
-  // never cache-resident, so back-to-back launches on one weight would rank the kernels wrongly.
   auto time_algo = [&](hipblasLtMatmulAlgo_t& algo, int reps) -> float {
-    if (hipblasLtMatmul(h, p->desc, alpha, w, p->a, x, p->b, &beta, cptr, p->c, out, p->d, &algo, lws, lws_bytes,
+    if (hipblasLtMatmul(h, p->desc, alpha, c.w, p->a, c.x, p->b, &beta, cptr, p->c, c.out, p->d, &algo, lws, lws_bytes,
                         c.stream) != HIPBLAS_STATUS_SUCCESS)
       return -1.f;
     float total = 0.f;
     for (int i = 0; i < reps; ++i) {
       if (flush != nullptr && flush_bytes > 0) (void)hipMemsetAsync(flush, i & 0xff, flush_bytes, c.stream);
       (void)hipEventRecord(e0, c.stream);
-      hipblasLtMatmul(h, p->desc, alpha, w, p->a, x, p->b, &beta, cptr, p->c, out, p->d, &algo, lws, lws_bytes, c.stream);
+      hipblasLtMatmul(h, p->desc, alpha, c.w, p->a, c.x, p->b, &beta, cptr, p->c, c.out, p->d, &algo, lws, lws_bytes,
+                      c.stream);
       (void)hipEventRecord(e1, c.stream);
       if (hipEventSynchronize(e1) != hipSuccess) return -1.f;
       float ms = 0.f;
@@ -375,6 +500,83 @@ extern "C" int odit_linear_tune(const void* x, const void* w, const void* bias, 
     set_error("odit_linear_tune: none of the library's %zu kernels accepts this problem", all.size());
     return ODIT_ENOTSUP;
   }
+  *best_us = best;
+  return ODIT_OK;
+}
+
+static int lin_time_handwritten(const odit::GemmCall& g, void* sk, hipStream_t stream, int iters, void* flush,
+                                size_t flush_bytes, float* us) {
+  using namespace odit;
+  hipEvent_t e0, e1;
+  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+    set_error("odit_linear_tune: hipEventCreate failed");
+    return ODIT_ELAUNCH;
+  }
+  int rc = launch_gemm_streamk(g, sk, stream);
+  float total = 0.f;
+  for (int i = 0; i < iters && rc == ODIT_OK; ++i) {
+    if (flush != nullptr && flush_bytes > 0) (void)hipMemsetAsync(flush, i & 0xff, flush_bytes, stream);
+    (void)hipEventRecord(e0, stream);
+    rc = launch_gemm_streamk(g, sk, stream);
+    (void)hipEventRecord(e1, stream);
+    if (hipEventSynchronize(e1) != hipSuccess) { set_error("odit_linear_tune: hipEventSynchronize failed"); rc = ODIT_ELAUNCH; }
+    float ms = 0.f;
+    (void)hipEventElapsedTime(&ms, e0, e1);
+    total += ms;
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  *us = total * 1e3f / iters;
+  return rc;
+}
+
+extern "C" int odit_linear_rows_tune(const void* x, const void* w, const void* bias, void* out, const void* residual,
+                                     const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
+                                     int64_t ldr, int epilogue, int gate_dtype, int dtype, int rows_per_gate,
+                                     int64_t gate_stride, void* workspace, size_t workspace_bytes, void* stream,
+                                     int iters, void* flush, size_t flush_bytes, float* best_us) {
+  using namespace odit;
+  void *sk, *lib;
+  size_t lib_bytes;
+  lin_split_ws(workspace, workspace_bytes, &sk, &lib, &lib_bytes);
+  LinCall c{x, w, bias, residual, gate, out, M, N, K, ldx, ldw, ldo, ldr, epilogue, gate_dtype, dtype,
+            lib, lib_bytes, static_cast<hipStream_t>(stream)};
+  int rc = lin_check(c);
+  if (rc != ODIT_OK) return rc;
+  ODIT_CHECK_ARG(M > 0 && iters > 0, "odit_linear_tune: needs M > 0 and iters > 0");
+  ODIT_CHECK_ARG(rows_per_gate >= 0 && gate_stride >= 0, "odit_linear_tune: rows_per_gate and gate_stride must not be negative");
+  const bool per_rows = lin_is_residual(c) && gate != nullptr && rows_per_gate > 0 && rows_per_gate < M;
+  // the library runs one launch per group of rows: tune that launch (on the first group)
+  LinCall cl = c;
+  int launches = 1;
+  if (per_rows) {
+    cl.M = rows_per_gate;
+    launches = (M + rows_per_gate - 1) / rows_per_gate;
+  }
+  float lib_us = 0.f;
+  rc = lin_tune_library(cl, iters, flush, flush_bytes, &lib_us);
+  if (rc != ODIT_OK) return rc;
+  lib_us *= static_cast<float>(launches);
+  float best = lib_us;
+  const GemmCall g = lin_gemm_call(c, per_rows ? rows_per_gate : 0, per_rows ? gate_stride : 0);
+  if (sk != nullptr && gemm_streamk_takes(g, dtype)) {
+    float own_us = 0.f;
+    rc = lin_time_handwritten(g, sk, c.stream, iters, flush, flush_bytes, &own_us);
+    if (rc != ODIT_OK) return rc;
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    g_lin.handwritten_wins[lin_engine_key(dev, c, per_rows ? rows_per_gate : 0)] = own_us < lib_us;
+    if (own_us < best) best = own_us;
+  }
   if (best_us) *best_us = best;
   return ODIT_OK;
+}
+
+extern "C" int odit_linear_tune(const void* x, const void* w, const void* bias, void* out, const void* residual,
+                                const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
+                                int64_t ldr, int epilogue, int gate_dtype, int dtype, void* workspace,
+                                size_t workspace_bytes, void* stream, int iters, void* flush,
+                                size_t flush_bytes, float* best_us) {
+  return odit_linear_rows_tune(x, w, bias, out, residual, gate, M, N, K, ldx, ldw, ldo, ldr, epilogue, gate_dtype, dtype,
+                               0, 0, workspace, workspace_bytes, stream, iters, flush, flush_bytes, best_us);
 }

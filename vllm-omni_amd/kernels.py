@@ -491,6 +491,19 @@ def set_linear_autotune(iters: int) -> None:
         _FLUSH.clear()
 
 
+_LINEAR_ENGINES = {"auto": 0, "library": 1, "handwritten": 2}
+
+
+def set_linear_engine(engine: str) -> None:
+    """Which kernel ``linear`` runs, process-wide: "auto" (the hand-written stream-K kernel where a tuning
+    run found it faster or, untuned, where K >= 2 N and it takes the problem; the library elsewhere),
+    "library" (hipBLASLt always) or "handwritten" (the stream-K kernel always; problems it does not take
+    raise). For measurements and tests."""
+    if engine not in _LINEAR_ENGINES:
+        raise ValueError(f"engine must be one of {sorted(_LINEAR_ENGINES)}")
+    _lib.check(_lib.load().odit_linear_set_engine(_LINEAR_ENGINES[engine]), "odit_linear_set_engine")
+
+
 def linear_tuning_report() -> dict[tuple, float]:
     """{problem key: best time in microseconds} of everything tuned so far in this process."""
     return dict(_LINEAR_TUNED)
@@ -500,7 +513,8 @@ def _linear_workspace(lib, device: torch.device) -> torch.Tensor:
     key = (device.index or 0, _stream())
     ws = _LINEAR_SCRATCH.get(key)
     if ws is None:
-        ws = torch.empty(int(lib.odit_linear_workspace_bytes()), dtype=torch.uint8, device=device)
+        # zero-filled: the hand-written kernel keeps tile counters at the start, zero between calls
+        ws = torch.zeros(int(lib.odit_linear_workspace_bytes()), dtype=torch.uint8, device=device)
         _LINEAR_SCRATCH[key] = ws
     return ws
 
@@ -517,16 +531,19 @@ def _rows2d(t: torch.Tensor, name: str) -> tuple[torch.Tensor, int]:
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *, activation: str | None = None,
            residual: torch.Tensor | None = None, gate: torch.Tensor | None = None, out: torch.Tensor | None = None,
-           gate_bias: torch.Tensor | None = None, prescaled: bool = False, tune_iters: int = 0):
+           gate_bias: torch.Tensor | None = None, prescaled: bool = False, tune_iters: int = 0,
+           plan_only: bool = False):
     """x W^T (+ bias) with the elementwise tail inside the GEMM's epilogue.
 
     activation="gelu_tanh": GELU(tanh) of the result. residual (same shape as the result) with optional
-    gate [B,N] / [B,1,N] / [N]: ``residual + gate * (x W^T + bias)``; one GEMM per batch row when the gate
-    differs per batch row. ``prescaled=True``: ``gate`` is float32 and ``gate_bias`` (float32, same shape, or
+    gate [B,N] / [B,1,N] / [N]: ``residual + gate * (x W^T + bias)``; gates that differ per batch row go
+    down as one call (one launch of the hand-written kernel, or one library launch per batch row). ``prescaled=True``: ``gate`` is float32 and ``gate_bias`` (float32, same shape, or
     None) already holds gate * bias — nothing is derived per call (``bias`` is then ignored).
     ``weight`` may be a column range of a Linear weight (row stride > K).
-    ``tune_iters`` > 0 first times the library's kernels for this problem (overwrites ``out``) and
-    returns the best time in microseconds instead of the result.
+    ``tune_iters`` > 0 first times the library's kernels and the hand-written kernel for this problem
+    (overwrites ``out``), keeps the faster for later calls and returns its time in microseconds instead
+    of the result. ``plan_only`` launches nothing and returns (the hand-written kernel would run, number of
+    kernel launches the call would make).
     """
     _dev(x, weight, bias, residual, gate, out)
     if weight.dim() != 2 or weight.stride(1) != 1 or x.shape[-1] != weight.shape[1]:
@@ -538,7 +555,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
     M = x2.shape[0]
     out_shape = (*x.shape[:-1], N)
     if out is None:
-        out = torch.empty(out_shape, dtype=x.dtype, device=x.device)
+        out = (residual if plan_only and residual is not None
+               else torch.empty(out_shape, dtype=x.dtype, device=x.device))
     elif tuple(out.shape) != out_shape or out.dtype != x.dtype:
         raise ValueError(f"out must be {out_shape} of {x.dtype}")
     o2, ldo = _rows2d(out, "out")
@@ -548,29 +566,37 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
     ws = _linear_workspace(lib, x.device)
     ldw = weight.stride(0) if N > 1 else K
     best = _lib.C.c_float(0.0)
+    plan = [_lib.C.c_int(0), _lib.C.c_int(0)]
 
-    def call(xp, op, rp, gp, m, epi, gate_code, bp=_ptr(bias)):
+    def call(rp, gp, epi, gate_code, bp=_ptr(bias), rows_per_gate=0, gate_stride=0, row0=0, M=M):
+        esz = x.element_size()
+        prob = (x2.data_ptr() + row0 * ldx * esz, weight.data_ptr(), bp, o2.data_ptr() + row0 * ldo * esz,
+                None if rp is None else rp + row0 * ldr * esz, gp, M, N, K, ldx, ldw, ldo, ldr, epi, gate_code,
+                _code(x), rows_per_gate, gate_stride)
+        if plan_only:
+            _lib.check(lib.odit_linear_rows_plan(*prob, ws.data_ptr(), ws.numel(), _lib.C.byref(plan[0]),
+                                                 _lib.C.byref(plan[1])), "odit_linear_rows_plan")
+            return
         if _LINEAR_AUTOTUNE_ITERS > 0 and tune_iters == 0:
-            key = (x.device.index or 0, m, N, K, epi, bp is not None, gp is not None, _code(x), ldx, ldw, ldo, ldr)
+            key = (x.device.index or 0, M, N, K, epi, bp is not None, gp is not None, _code(x), ldx, ldw, ldo, ldr,
+                   rows_per_gate)
             if key not in _LINEAR_TUNED:
                 # time the candidates on scratch output operands: tuning overwrites (and, for the residual
                 # forms, keeps accumulating into) whatever it is given
-                t_out = torch.empty((m, ldo), dtype=x.dtype, device=x.device)
-                t_res = torch.zeros((m, max(ldr, 1)), dtype=x.dtype, device=x.device) if rp is not None else None
+                t_out = torch.empty((M, ldo), dtype=x.dtype, device=x.device)
+                t_res = torch.zeros((M, max(ldr, 1)), dtype=x.dtype, device=x.device) if rp is not None else None
                 t_best = _lib.C.c_float(0.0)
-                _lib.check(lib.odit_linear_tune(xp, weight.data_ptr(), bp, t_out.data_ptr(), _ptr(t_res), gp, m, N, K,
-                                                ldx, ldw, ldo, ldr, epi, gate_code, _code(x), ws.data_ptr(),
-                                                ws.numel(), _stream(), _LINEAR_AUTOTUNE_ITERS, _flush_buffer(x.device),
-                                                _FLUSH_BYTES, _lib.C.byref(t_best)),
-                           "odit_linear_tune")
+                t_prob = prob[:3] + (t_out.data_ptr(), _ptr(t_res)) + prob[5:]
+                _lib.check(lib.odit_linear_rows_tune(*t_prob, ws.data_ptr(), ws.numel(), _stream(),
+                                                     _LINEAR_AUTOTUNE_ITERS, _flush_buffer(x.device), _FLUSH_BYTES,
+                                                     _lib.C.byref(t_best)), "odit_linear_rows_tune")
                 _LINEAR_TUNED[key] = t_best.value
-        args = (xp, weight.data_ptr(), bp, op, rp, gp, m, N, K, ldx, ldw, ldo, ldr, epi, gate_code, _code(x),
-                ws.data_ptr(), ws.numel(), _stream())
         if tune_iters > 0:
-            _lib.check(lib.odit_linear_tune(*args, int(tune_iters), _flush_buffer(x.device), _FLUSH_BYTES,
-                                            _lib.C.byref(best)), "odit_linear_tune")
+            _lib.check(lib.odit_linear_rows_tune(*prob, ws.data_ptr(), ws.numel(), _stream(), int(tune_iters),
+                                                 _flush_buffer(x.device), _FLUSH_BYTES, _lib.C.byref(best)),
+                       "odit_linear_rows_tune")
         else:
-            _lib.check(lib.odit_linear(*args), "odit_linear")
+            _lib.check(lib.odit_linear_rows(*prob, ws.data_ptr(), ws.numel(), _stream()), "odit_linear_rows")
 
     ldr = 0
     if residual is None:
@@ -582,45 +608,49 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
             epi = ODIT_EPI_BIAS_GELU_TANH if bias is not None else ODIT_EPI_GELU_TANH
         else:
             raise ValueError(f"unknown activation {activation!r}")
-        call(x2.data_ptr(), o2.data_ptr(), None, None, M, epi, _code(x))
+        call(None, None, epi, _code(x))
+        if plan_only:
+            return bool(plan[0].value), plan[1].value
         return best.value if tune_iters > 0 else out
     if activation is not None:
         raise ValueError("activation and residual cannot be combined")
     if tuple(residual.shape) != out_shape or residual.dtype != x.dtype:
         raise ValueError(f"residual must be {out_shape} of {x.dtype}")
     r2, ldr = _rows2d(residual, "residual")
-    esz = x.element_size()
     if gate is None or gate.dim() == 1:
-        groups, rows, g2 = 1, M, (None if gate is None else gate.reshape(1, N))
+        rows, g2 = 0, (None if gate is None else gate.reshape(1, N))
     else:
         B = x.shape[0]
         g2 = gate.reshape(B, N) if gate.numel() == B * N else None
         if g2 is None or x.dim() < 2:
             raise ValueError(f"gate shape {tuple(gate.shape)} does not give one row of {N} per batch row")
-        groups, rows = B, M // B
+        rows = M // B if B > 1 else 0
     if g2 is not None:
         _last_contig(g2, "gate")
         if g2.dtype not in (x.dtype, torch.float32):
             raise TypeError("gate must have x's dtype or float32")
-    gb2 = None
+    gstride = g2.stride(0) if (g2 is not None and rows > 0) else 0
     if prescaled:
         if g2 is None or g2.dtype != torch.float32:
             raise TypeError("prescaled=True needs a float32 gate")
+        gb2 = None
         if gate_bias is not None:
             gb2 = gate_bias.reshape(g2.shape)
             _last_contig(gb2, "gate_bias")
             if gb2.dtype != torch.float32:
                 raise TypeError("gate_bias must be float32")
-    for b in range(groups):
-        off = b * rows
-        xp, op, rp = (x2.data_ptr() + off * ldx * esz, o2.data_ptr() + off * ldo * esz,
-                      r2.data_ptr() + off * ldr * esz)
-        if prescaled:
-            call(xp, op, rp, g2[b].data_ptr(), rows, ODIT_EPI_GATED_RESIDUAL_PRE, ODIT_F32,
-                 None if gb2 is None else gb2[b].data_ptr())
+        if rows > 0 and gb2 is not None and gb2.stride(0) != gstride:
+            # gate and gate * bias rows laid out differently: one call per batch row
+            for b in range(g2.shape[0]):
+                call(r2.data_ptr(), g2[b].data_ptr(), ODIT_EPI_GATED_RESIDUAL_PRE, ODIT_F32, gb2[b].data_ptr(),
+                     row0=b * rows, M=rows)
+                if tune_iters > 0 or plan_only:
+                    break  # every batch row is the same problem
         else:
-            call(xp, op, rp, None if g2 is None else g2[b].data_ptr(), rows, ODIT_EPI_GATED_RESIDUAL,
-                 _code(x) if g2 is None else _code(g2))
-        if tune_iters > 0:
-            break  # every batch row is the same problem
+            call(r2.data_ptr(), g2.data_ptr(), ODIT_EPI_GATED_RESIDUAL_PRE, ODIT_F32, _ptr(gb2), rows, gstride)
+    else:
+        call(r2.data_ptr(), _ptr(g2), ODIT_EPI_GATED_RESIDUAL, _code(x) if g2 is None else _code(g2), _ptr(bias), rows,
+             gstride)
+    if plan_only:
+        return bool(plan[0].value), plan[1].value
     return best.value if tune_iters > 0 else out
