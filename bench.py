@@ -25,17 +25,9 @@ if ROOT not in sys.path:
 
 PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, vendor figure
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E, vendor figure
-# HBM bytes of one attention call at the headline shape, from rocprofv3 FETCH_SIZE / WRITE_SIZE passes
-# over `bench.py --traffic-probe`, each scaled by what the same counter reads for a 512 MiB copy
-# (FETCH_SIZE x2.0, WRITE_SIZE x1.0). One call = three launches: the full units (203.7 MB fetched + 51.9 MB
-# written), the key ranges of the last round (74.0 + 36.4 MB) and their merge (33.5 + 3.1 MB).
-ATTN_TRAFFIC_BYTES = 402.6e6
-# Matrix-pipe counters of the attention main launch at the headline shape, from a rocprofv3 SQ-counter pass over
-# `bench.py --counter-probe` (not measured live): share of the launch's cycles with the MFMA pipe busy
-# (SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE / 8 x 1024 SIMDs)) and the clock those cycles ran at
-# (GRBM_GUI_ACTIVE / 8 / duration); the nominal peak assumes 2400 MHz.
-ATTN_MFMA_BUSY_FRAC = 0.560
-ATTN_CLOCK_MHZ = 1771.0
+# HBM traffic, MFMA-busy share and in-kernel clock of the attention call come from the committed counter
+# summaries under profiles/ (vllm_omni_amd.profiling.attention_figures), which name the launches they were
+# measured on: a build that dispatches other launches for the headline shape makes bench.py stop.
 
 # Qwen-Image shape at 1024x1024 (BASELINE.json configs[2])
 LAYERS, HEADS, HEAD_DIM, MLP_RATIO = 60, 24, 128, 4
@@ -435,6 +427,12 @@ def counter_probe(torch, kernels, dev):
     b_up = torch.zeros(MLP_RATIO * C, device=dev, dtype=bf)
     w_qkv = torch.randn(3 * C, C, device=dev, dtype=bf) * 0.02
     b_qkv = torch.zeros(3 * C, device=dev, dtype=bf)
+    # text stream's MLP down-projection with its gated residual (the hand-written stream-K GEMM)
+    t_in = torch.randn(B, S_TXT, MLP_RATIO * C, device=dev, dtype=bf)
+    t_res = torch.randn(B, S_TXT, C, device=dev, dtype=bf)
+    w_dn = torch.randn(C, MLP_RATIO * C, device=dev, dtype=bf) * 0.02
+    g32 = torch.randn(B, C, device=dev)
+    assert kernels.linear(t_in, w_dn, None, residual=t_res, gate=g32, gate_bias=g32 * 0.1, prescaled=True, plan_only=True)[0]
     for _ in range(3):
         kernels.attn_fwd(q, k, v, 1.0 / math.sqrt(HEAD_DIM))
         kernels.qknorm_rope(qkv[:, :, 0], qkv[:, :, 1], None, jq, jk, None, w, w, cos, sin, out_seq_offset=S_TXT,
@@ -444,9 +442,12 @@ def counter_probe(torch, kernels, dev):
         kernels.rel_l1_sums(x, y)
         kernels.linear(x2, w_up, b_up, activation="gelu_tanh")
         torch.nn.functional.linear(x2, w_qkv, b_qkv)
+        kernels.linear(t_in, w_dn, None, residual=t_res, gate=g32, gate_bias=g32 * 0.1, prescaled=True)
     torch.cuda.synchronize()
     print(json.dumps({"probe": "attention, qknorm+rope, adaLN, gated residual, rel-L1, MLP-up GEMM (GELU epilogue), "
-                               "QKV GEMM at the Qwen-Image shape, 3 launches each",
+                               "QKV GEMM, text MLP-down GEMM (stream-K, gated residual) at the Qwen-Image shape, 3 launches each",
+                      "attention_plan": kernels.attn_plan(B, S, S, HEADS, HEAD_DIM),
+                      "text_mlp_down_flop": 2.0 * B * S_TXT * C * MLP_RATIO * C,
                       "attention_flop": 4.0 * B * HEADS * S * S * HEAD_DIM,
                       "mlp_up_flop": 2.0 * B * S_IMG * C * MLP_RATIO * C, "qkv_flop": 2.0 * B * S_IMG * C * 3 * C}))
 
@@ -577,6 +578,7 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"probe": "attention B=2 S=4352 24x128 bf16 x4, copy 512 MiB x4",
+                          "attention_plan": kernels.attn_plan(B, S, S, HEADS, HEAD_DIM),
                           "attention_min_bytes": 4 * q.numel() * 2, "copy_bytes_each_way": src.numel()}))
         return
     if args.counter_probe:
@@ -620,6 +622,13 @@ def main():
     S = S_IMG + S_TXT
     attn_flop = 4.0 * B * HEADS * S * S * HEAD_DIM
     attn_tflops = attn_flop / attn_ms / 1e9
+    from vllm_omni_amd import profiling
+
+    plan = kernels.attn_plan(B, S, S, HEADS, HEAD_DIM)
+    try:
+        prof = profiling.attention_figures(plan)
+    except (RuntimeError, ValueError, OSError) as e:
+        sys.exit(f"bench.py: {e}")
     result = {
         "metric": "DiT denoise steps/s @1024² Qwen-Image shape (1 GPU); attn % bf16 MFMA peak",
         "value": args.steps / elapsed,
@@ -637,15 +646,19 @@ def main():
                                f"{HEADS} heads x {HEAD_DIM}, MLP {MLP_RATIO * C}, {S_IMG} image + {S_TXT} text tokens, "
                                "CFG batch 2, random weights N(0,0.02)",
                    "valid": args.blocks == LAYERS, "gemm": "hipBLASLt via torch" + (" (tuned solution table)" if tuned else "") +
+                           ("" if args.linear_engine == "library" else "; text-stream MLP down-projection on the hand-written "
+                            "stream-K MFMA kernel") +
                            ("; GELU and gated residuals as separate kernels" if args.unfused_epilogues else
                             "; GELU and gated residuals in the GEMM epilogues (odit_linear)")},
-        "roofline": {"kernel": "attn_fwd_dma_kernel (joint attention, B=2, 24x128, S=4352; one call = the full units + "
-                               "the key-split last round + its merge, timed together)", "bound": "mfma",
+        "roofline": {"kernel": f"joint attention, B=2, 24x128, S=4352; one call = {plan} (timed together)", "bound": "mfma",
                      "achieved": attn_tflops, "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": attn_tflops / PEAK_MFMA_BF16_TFLOPS,
-                     "traffic": ATTN_TRAFFIC_BYTES if args.blocks == LAYERS else None,
-                     "counters": {"mfma_busy_frac_of_cycles": ATTN_MFMA_BUSY_FRAC, "clock_MHz_in_kernel": ATTN_CLOCK_MHZ,
-                                  "source": "rocprofv3 --pmc pass over bench.py --counter-probe, not live"},
+                     "traffic": prof["traffic_bytes"],
+                     "counters": {"mfma_busy_frac_of_cycles": prof["mfma_busy_frac"], "clock_MHz_in_kernel": prof["clock_MHz"],
+                                  "kernel": prof["profiled_kernel"],
+                                  "source": "profiles/" + profiling.COUNTERS_FILE + " and profiles/" + profiling.TRAFFIC_FILE +
+                                            " (rocprofv3 --pmc passes over bench.py --counter-probe / --traffic-probe, not live; "
+                                            "launch plan checked against this build)"},
                      "launches_timed": n_attn, "avg_ms": attn_ms, "flop_per_launch": attn_flop},
         "step_flop": None,
     }

@@ -653,3 +653,24 @@ def test_qwen_mixin_diffuse_feeds_the_transformer_like_the_reference():
     assert out.shape == lat.shape
     # velocity per branch: mean of the (padded) prompt = 2 and -2/5; combined -0.4 + 2 * 2.4 = 4.4; sum of dsigma = -1
     torch.testing.assert_close(out, torch.full_like(lat, -4.4))
+
+
+def test_profile_records_name_the_launches_they_were_measured_on():
+    """bench.py quotes HBM traffic and matrix-pipe counters from profiles/*.txt only for the launch plan those
+    files were measured on (vllm_omni_amd/profiling.py)."""
+    from vllm_omni_amd import profiling
+
+    traffic = profiling.read_record(profiling.TRAFFIC_FILE)
+    counters = profiling.read_record(profiling.COUNTERS_FILE)
+    plan = traffic["attention_plan"]
+    assert plan == counters["attention_plan"] and "attn_fwd_dma_kernel<T, 128, 4, false>" in plan
+    fig = profiling.attention_figures(plan)
+    assert fig["traffic_bytes"] == traffic["traffic_bytes"] > 213.9e6          # at least the algorithmic bytes
+    assert 0.3 < fig["mfma_busy_frac"] < 1.0 and 1000 < fig["clock_MHz"] < 2500
+    assert "attn_fwd_dma_kernel" in fig["profiled_kernel"]
+    with pytest.raises(RuntimeError, match="re-run the counter passes"):
+        profiling.attention_figures(plan.replace("units=1536", "units=1537"))
+    assert profiling._plan_kernels(plan) == ["attn_fwd_dma_kernel<T, 128, 4, false>", "attn_fwd_dma_kernel<T, 128, 4, true>",
+                                             "attn_merge_kernel<T, 128, 128>"]
+    assert profiling._is_kernel("attn_merge_kernel<T, 128, 128>", "void odit::attn_merge_kernel<odit::bf16_t, 128, 128>(odit::AttnParams, int)")
+    assert not profiling._is_kernel("attn_fwd_dma_kernel<T, 128, 4, true>", "void odit::attn_fwd_dma_kernel<odit::bf16_t, 128, 4, false>(odit::AttnParams)")

@@ -478,12 +478,13 @@ int attn_dma_plan(int B, int Sq, int Sk, int H, int D, bool with_workspace, char
   TailPlan t{0, 1, 0};
   if (with_workspace) t = plan_tail(units, (Sk + 63) / 64, device_slots(kDmaWaves));
   if (t.rem == 0) {
-    snprintf(text, text_bytes, "attn_fwd_dma_kernel units=%lld", static_cast<long long>(units));
+    snprintf(text, text_bytes, "attn_fwd_dma_kernel<T, %d, %d, false> units=%lld", D, kDmaWaves, static_cast<long long>(units));
     return 1;
   }
-  snprintf(text, text_bytes, "attn_fwd_dma_kernel units=%lld; attn_fwd_dma_kernel(key ranges) units=%d x %d ranges of %d "
-           "tiles; attn_merge_kernel rows=%d", static_cast<long long>(units - t.rem), t.rem, t.key_chunks,
-           t.tiles_per_chunk, t.rem * bm);
+  // kernel names as a profiler prints them, with T for the element type
+  snprintf(text, text_bytes, "attn_fwd_dma_kernel<T, %d, %d, false> units=%lld; attn_fwd_dma_kernel<T, %d, %d, true> "
+           "units=%d x %d key ranges of %d tiles; attn_merge_kernel<T, %d, %d> rows=%d", D, kDmaWaves,
+           static_cast<long long>(units - t.rem), D, kDmaWaves, t.rem, t.key_chunks, t.tiles_per_chunk, D, bm, t.rem * bm);
   return units - t.rem > 0 ? 3 : 2;
 }
 
