@@ -136,6 +136,14 @@ static int lin_plan_build(const LinKey& key, LinPlan& p) {
 static int lin_plan(const LinKey& key, LinPlan** out) {
   auto it = g_lin.plans.find(key);
   if (it != g_lin.plans.end()) { *out = &it->second; return ODIT_OK; }
+  // A process sees a few dozen distinct problems; a caller that keeps inventing new ones (changing row
+  // counts) must not grow the cache without bound: past the cap everything is rebuilt on demand.
+  constexpr size_t kMaxPlans = 512;
+  if (g_lin.plans.size() >= kMaxPlans) {
+    for (auto& kv : g_lin.plans) lin_plan_release(kv.second);
+    g_lin.plans.clear();
+    g_lin.handwritten_wins.clear();
+  }
   LinPlan p;
   const int rc = lin_plan_build(key, p);
   if (rc != ODIT_OK) {  // nothing half-built stays behind
