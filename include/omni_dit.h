@@ -152,6 +152,19 @@ int odit_qknorm_rope(const void* q_in, const void* k_in, const void* v_in, void*
                      int out_seq_offset, int S_total, float eps, int norm_mode, int w_dtype,
                      int dtype, unsigned flags, void* stream);
 
+/* Two odit_qknorm_rope problems that fill different rows of the same joint buffers, in ONE launch: the text
+ * rows and the image rows of a dual-stream block (qwen_image_transformer.py:588-606, where the reference
+ * normalises and rotates the two streams separately and concatenates them). Element i of every array belongs to
+ * problem i; in_strides = {batch0, seq0, batch1, seq1}. Both problems share B, H, D, rot, S_total, eps,
+ * norm_mode, the dtypes and the flags, and take the same optional operands (k, v, rotary tables). With
+ * ODIT_NORM_ROW, or when one problem is empty, the call makes one launch per problem. */
+int odit_qknorm_rope_pair(const void* const q_in[2], const void* const k_in[2], const void* const v_in[2],
+                          void* q_out, void* k_out, void* v_out, const void* const wq[2],
+                          const void* const wk[2], const float* const cos[2], const float* const sin[2],
+                          int B, const int S[2], int H, int D, int rot, const int64_t in_strides[4],
+                          const int out_seq_offset[2], int S_total, float eps, int norm_mode, int w_dtype,
+                          int dtype, unsigned flags, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * K3  fused LayerNorm (no affine, or fp32 affine) + adaLN shift/scale modulation:
  *        out = LN(x) * (1 + scale) + shift
@@ -180,6 +193,17 @@ int odit_adaln_modulate(const void* x, void* out, const void* shift, const void*
                         const int64_t x_strides[2], const int64_t out_strides[2],
                         int64_t mod_stride_b, int64_t mod_stride_s, float eps, int mod_dtype,
                         int dtype, unsigned flags, void* stream);
+
+/* odit_adaln_modulate for two tensors of the same batch and width in ONE launch: img_norm1 and txt_norm1
+ * (or img_norm2 and txt_norm2) of a dual-stream block, which the reference calls one after the other
+ * (qwen_image_transformer.py:770-773, 798, 804). One modulation row per batch entry (no index, no
+ * LayerNorm affine, no tables); element i of every array belongs to problem i, x_strides / out_strides =
+ * {batch0, seq0, batch1, seq1}, mod_stride_b[i] the row stride of shift[i] / scale[i]. */
+int odit_adaln_modulate_pair(const void* const x[2], void* const out[2], const void* const shift[2],
+                             const void* const scale[2], int B, const int S[2], int C,
+                             const int64_t x_strides[4], const int64_t out_strides[4],
+                             const int64_t mod_stride_b[2], float eps, int mod_dtype, int dtype,
+                             unsigned flags, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * K4  gated residual:  out = h + gate * y     (gate broadcast over the sequence, or per token)

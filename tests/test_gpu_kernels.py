@@ -253,6 +253,74 @@ def test_rel_l1_closed_forms(gpu):
 
 
 # ========================================================================================= K2
+# ---- two problems in one launch (the image and the text stream of a dual-stream block) ----------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("C,S0,S1", [(3072, 70, 9), (256, 5, 33), (37, 4, 6)])
+@pytest.mark.parametrize("ref_rounding", [False, True])
+def test_adaln_modulate_pair_equals_two_calls(gpu, dtype, C, S0, S1, ref_rounding):
+    """odit_adaln_modulate_pair against odit_adaln_modulate, bit for bit (C = 37 takes the any-width kernel),
+    with strided inputs and modulation rows that are views of one [B, 6C] tensor, and against the oracle."""
+    from vllm_omni_amd import kernels
+
+    B = 2
+    xs = [_rand(B, S, 2 * C, seed=3 + i, dtype=dtype, scale=2.0).to(gpu)[:, :, C:] if C % 8 == 0
+          else _rand(B, S, C, seed=3 + i, dtype=dtype, scale=2.0).to(gpu) for i, S in enumerate((S0, S1))]
+    mods = [(_rand(B, 6 * C, seed=7 + i, dtype=dtype) * 0.3).to(gpu) for i in range(2)]
+    probs = [(x, m[:, :C], m[:, C:2 * C]) for x, m in zip(xs, mods)]
+    got = kernels.adaln_modulate_pair(probs[0], probs[1], eps=1e-6, ref_rounding=ref_rounding)
+    for (x, shift, scale), m, g in zip(probs, mods, got):
+        one = kernels.adaln_modulate(x, shift, scale, eps=1e-6, ref_rounding=ref_rounding)
+        assert torch.equal(g, one), "pair launch differs from the single call"
+        want = ops.ada_layer_norm(x.float().cpu(), m[:, :3 * C].float().cpu(), eps=1e-6)[0]
+        tol = {torch.bfloat16: 2e-2, torch.float16: 3e-3, torch.float32: 2e-5}[dtype]
+        _close(g, want, atol=tol, rtol=tol, what="adaln pair vs oracle")
+    # an empty problem leaves the other one
+    empty = (xs[1][:, :0], probs[1][1], probs[1][2])
+    g0, g1 = kernels.adaln_modulate_pair(probs[0], empty, eps=1e-6, ref_rounding=ref_rounding)
+    assert torch.equal(g0, got[0]) and g1.shape[1] == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("with_v", [False, True])
+@pytest.mark.parametrize("ref_rounding", [False, True])
+def test_qknorm_rope_pair_equals_two_calls(gpu, dtype, with_v, ref_rounding):
+    """odit_qknorm_rope_pair against two odit_qknorm_rope calls into the same joint buffers, bit for bit:
+    different lengths, weights, tables and row offsets per problem; also with whole-row statistics (one launch
+    per problem inside the call) and without rotary tables."""
+    from vllm_omni_amd import kernels
+    from vllm_omni_amd._lib import ODIT_NORM_HEAD, ODIT_NORM_NONE, ODIT_NORM_ROW
+
+    B, H, D, S_txt, S_img = 2, 4, 64, 11, 150
+    S = S_txt + S_img
+    qkv = [_rand(B, n, 3, H, D, seed=30 + i, dtype=dtype).to(gpu) for i, n in enumerate((S_txt, S_img))]
+    tabs = [tuple(t.to(gpu) for t in _cos_sin(n, D // 2, seed=40 + i)) for i, n in enumerate((S_txt, S_img))]
+    for mode, wn in ((ODIT_NORM_HEAD, D), (ODIT_NORM_ROW, H * D), (ODIT_NORM_NONE, D)):
+        ws = [((_rand(wn, seed=50 + i, dtype=torch.float32) * 0.2 + 1).to(dtype).to(gpu),
+               (_rand(wn, seed=60 + i, dtype=torch.float32) * 0.2 + 1).to(dtype).to(gpu)) for i in range(2)]
+        for rotary in (True, False):
+            outs = []
+            for paired in (False, True):
+                jq = torch.zeros(B, S, H, D, dtype=dtype, device=gpu)
+                jk = torch.zeros_like(jq)
+                jv = torch.zeros_like(jq) if with_v else None
+                probs = []
+                for i, off in enumerate((0, S_txt)):
+                    t = qkv[i]
+                    cs = tabs[i] if rotary else (None, None)
+                    probs.append((t[:, :, 0], t[:, :, 1], t[:, :, 2] if with_v else None, ws[i][0], ws[i][1],
+                                  cs[0], cs[1], off))
+                if paired:
+                    kernels.qknorm_rope_pair(probs[0], probs[1], jq, jk, jv, eps=1e-6, norm_mode=mode,
+                                             ref_rounding=ref_rounding)
+                else:
+                    for (q, k, v, wq, wk, c, s_, off) in probs:
+                        kernels.qknorm_rope(q, k, v, jq, jk, jv, wq, wk, c, s_, eps=1e-6, out_seq_offset=off,
+                                            norm_mode=mode, ref_rounding=ref_rounding)
+                outs.append((jq, jk, jv))
+            for a, b in zip(*outs):
+                assert (a is None and b is None) or torch.equal(a, b), f"pair launch differs (mode {mode}, rotary {rotary})"
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("H,D", [(24, 128), (4, 64)])
 def test_qknorm_rope_joint(gpu, dtype, H, D):

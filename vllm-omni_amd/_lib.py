@@ -23,6 +23,8 @@ ODIT_EPI_GATED_RESIDUAL_PRE = 5
 
 # every symbol include/omni_dit.h declares: (name, restype, argtypes)
 _i64p = C.POINTER(C.c_int64)
+_intp = C.POINTER(C.c_int)
+_vpp = C.POINTER(C.c_void_p)
 _SIGNATURES = {
     "odit_version": (C.c_int, []),
     "odit_last_error": (C.c_char_p, []),
@@ -49,6 +51,17 @@ _SIGNATURES = {
          C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
          C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _i64p, C.c_int, C.c_int, C.c_float,
          C.c_int, C.c_int, C.c_int, C.c_uint, C.c_void_p],
+    ),
+    "odit_qknorm_rope_pair": (
+        C.c_int,
+        [_vpp, _vpp, _vpp, C.c_void_p, C.c_void_p, C.c_void_p, _vpp, _vpp, _vpp, _vpp,
+         C.c_int, _intp, C.c_int, C.c_int, C.c_int, _i64p, _intp, C.c_int, C.c_float,
+         C.c_int, C.c_int, C.c_int, C.c_uint, C.c_void_p],
+    ),
+    "odit_adaln_modulate_pair": (
+        C.c_int,
+        [_vpp, _vpp, _vpp, _vpp, C.c_int, _intp, C.c_int, _i64p, _i64p, _i64p, C.c_float, C.c_int, C.c_int,
+         C.c_uint, C.c_void_p],
     ),
     "odit_adaln_modulate": (
         C.c_int,
@@ -163,3 +176,13 @@ def check(status: int, what: str) -> None:
 def i64_array(values) -> C.Array:
     vals = [int(v) for v in values]
     return (C.c_int64 * len(vals))(*vals)
+
+
+def int_array(values) -> C.Array:
+    vals = [int(v) for v in values]
+    return (C.c_int * len(vals))(*vals)
+
+
+def ptr_array(values) -> C.Array:
+    """Array of device addresses (None = null)."""
+    return (C.c_void_p * len(values))(*[None if not v else int(v) for v in values])

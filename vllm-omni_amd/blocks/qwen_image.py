@@ -26,7 +26,7 @@ from .. import kernels
 from .._lib import ODIT_NORM_HEAD
 from ..attention.backends.abstract import AttentionMetadata
 from ..attention.layer import Attention
-from ..layers.adalayernorm import AdaLayerNorm
+from ..layers.adalayernorm import AdaLayerNorm, adaln_pair
 from ..layers.rmsnorm import RMSNorm
 from ..layers.rope import RotaryEmbedding
 
@@ -266,12 +266,13 @@ class QwenImageCrossAttention(nn.Module):
                       and not self.ref_rounding)
         jv = None if v_in_place else torch.empty_like(jq)
         rr = self.ref_rounding
-        kernels.qknorm_rope(txt_qkv[:, :, 0], txt_qkv[:, :, 1], None if v_in_place else txt_qkv[:, :, 2], jq, jk, jv,
-                            self.norm_added_q.weight, self.norm_added_k.weight, tables.txt_cos, tables.txt_sin,
-                            eps=self.eps, out_seq_offset=0, norm_mode=ODIT_NORM_HEAD, ref_rounding=rr)
-        kernels.qknorm_rope(img_qkv[:, :, 0], img_qkv[:, :, 1], None if v_in_place else img_qkv[:, :, 2], jq, jk, jv,
-                            self.norm_q.weight, self.norm_k.weight, tables.img_cos, tables.img_sin,
-                            eps=self.eps, out_seq_offset=S_txt, norm_mode=ODIT_NORM_HEAD, ref_rounding=rr)
+        # text rows [0, S_txt) and image rows [S_txt, S) of the joint buffers, one launch for both streams
+        kernels.qknorm_rope_pair(
+            (txt_qkv[:, :, 0], txt_qkv[:, :, 1], None if v_in_place else txt_qkv[:, :, 2],
+             self.norm_added_q.weight, self.norm_added_k.weight, tables.txt_cos, tables.txt_sin, 0),
+            (img_qkv[:, :, 0], img_qkv[:, :, 1], None if v_in_place else img_qkv[:, :, 2],
+             self.norm_q.weight, self.norm_k.weight, tables.img_cos, tables.img_sin, S_txt),
+            jq, jk, jv, eps=self.eps, norm_mode=ODIT_NORM_HEAD, ref_rounding=rr)
         # the backend writes the text and image rows of the output to two dense tensors
         meta = AttentionMetadata(output_split=S_txt)
         if v_in_place:
@@ -345,8 +346,13 @@ class QwenImageTransformerBlock(nn.Module):
         img_mod1, img_mod2 = img_mod_params.chunk(2, dim=-1)
         txt_mod1, txt_mod2 = txt_mod_params.chunk(2, dim=-1)
 
-        img_modulated, img_gate1 = self.img_norm1(hidden_states, img_mod1, modulate_index)
-        txt_modulated, txt_gate1 = self.txt_norm1(encoder_hidden_states, txt_mod1)
+        # without a per-token index the two streams' norms are one launch
+        if modulate_index is None:
+            (img_modulated, img_gate1), (txt_modulated, txt_gate1) = adaln_pair(
+                self.img_norm1, hidden_states, img_mod1, self.txt_norm1, encoder_hidden_states, txt_mod1)
+        else:
+            img_modulated, img_gate1 = self.img_norm1(hidden_states, img_mod1, modulate_index)
+            txt_modulated, txt_gate1 = self.txt_norm1(encoder_hidden_states, txt_mod1)
         tables = image_rotary_emb if isinstance(image_rotary_emb, RotaryTables) else RotaryTables(*image_rotary_emb)
         # the block's inputs are never written (callers such as TeaCache keep them to form residuals):
         # the attention residuals land in new tensors, the MLP residuals then update those in place
@@ -355,10 +361,14 @@ class QwenImageTransformerBlock(nn.Module):
             encoder_hidden_states_mask=encoder_hidden_states_mask,
             residuals=(hidden_states, img_gate1, encoder_hidden_states, txt_gate1, pre[0][0], pre[1][0]))
 
-        img_modulated2, img_gate2 = self.img_norm2(hidden_states, img_mod2, modulate_index)
+        if modulate_index is None:
+            (img_modulated2, img_gate2), (txt_modulated2, txt_gate2) = adaln_pair(
+                self.img_norm2, hidden_states, img_mod2, self.txt_norm2, encoder_hidden_states, txt_mod2)
+        else:
+            img_modulated2, img_gate2 = self.img_norm2(hidden_states, img_mod2, modulate_index)
+            txt_modulated2, txt_gate2 = self.txt_norm2(encoder_hidden_states, txt_mod2)
         hidden_states = self.img_mlp.forward_residual(img_modulated2, hidden_states, img_gate2, out=hidden_states,
                                                       ref_rounding=rr, pre=pre[0][1])
-        txt_modulated2, txt_gate2 = self.txt_norm2(encoder_hidden_states, txt_mod2)
         encoder_hidden_states = self.txt_mlp.forward_residual(txt_modulated2, encoder_hidden_states, txt_gate2,
                                                               out=encoder_hidden_states, ref_rounding=rr, pre=pre[1][1])
         if encoder_hidden_states.dtype == torch.float16:

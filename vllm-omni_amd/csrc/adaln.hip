@@ -41,17 +41,37 @@ __device__ __forceinline__ void load_params(const TP* p, float fill, float (&dst
 // PLAIN = the per-block call of the DiT step (shift and scale given, no per-token index, no LayerNorm
 // affine): the optional operands cost registers and address arithmetic even when absent, and this
 // pass lives on how many rows a CU keeps in flight.
+//
+// One launch can carry TWO problems of the same width (the image rows and the text rows of a dual-stream
+// block): workgroups [0, rows0) belong to the first, the rest to the second; the choice is
+// workgroup-uniform (scalar selects). A single problem is rows0 = gridDim.x.
+template <typename T, typename TM> struct AdalnProblem {
+  const T* x;
+  T* out;
+  const TM *shift, *scale;
+  int S;
+  int64_t xs_b, xs_s, os_b, os_s, mod_stride_b;
+};
+
 template <typename T, typename TM, int W, int NVL, bool REF_ROUND, bool PLAIN>
 __global__ __launch_bounds__(W * 64) void adaln_rows_kernel(
-    const T* __restrict__ x, T* __restrict__ out, const TM* __restrict__ shift,
-    const TM* __restrict__ scale, const int32_t* __restrict__ index,
+    const AdalnProblem<T, TM> p0, const AdalnProblem<T, TM> p1, unsigned rows0,
+    const int32_t* __restrict__ index,
     const float* __restrict__ ln_w, const float* __restrict__ ln_b,
-    const float* __restrict__ shift_bias, const float* __restrict__ scale_bias, int B, int S, int C,
-    int64_t xs_b, int64_t xs_s, int64_t os_b, int64_t os_s, int64_t mod_stride_b,
+    const float* __restrict__ shift_bias, const float* __restrict__ scale_bias, int B, int C,
     int64_t mod_stride_s, float eps) {
   constexpr int EPV = Vec16<T>::N;
   const int tid = threadIdx.x;
-  const unsigned row = blockIdx.x;  // the launcher keeps B*S below 2^31
+  const bool second = blockIdx.x >= rows0;  // workgroup-uniform
+  const T* __restrict__ x = second ? p1.x : p0.x;
+  T* __restrict__ out = second ? p1.out : p0.out;
+  const TM* __restrict__ shift = second ? p1.shift : p0.shift;
+  const TM* __restrict__ scale = second ? p1.scale : p0.scale;
+  const int S = second ? p1.S : p0.S;
+  const int64_t xs_b = second ? p1.xs_b : p0.xs_b, xs_s = second ? p1.xs_s : p0.xs_s;
+  const int64_t os_b = second ? p1.os_b : p0.os_b, os_s = second ? p1.os_s : p0.os_s;
+  const int64_t mod_stride_b = second ? p1.mod_stride_b : p0.mod_stride_b;
+  const unsigned row = blockIdx.x - (second ? rows0 : 0u);  // the launcher keeps B*S below 2^31
   const int b = static_cast<int>(row / static_cast<unsigned>(S));
   const int s = static_cast<int>(row - static_cast<unsigned>(b) * static_cast<unsigned>(S));
   const T* xr = x + b * xs_b + s * xs_s;
@@ -184,30 +204,48 @@ __global__ __launch_bounds__(256) void adaln_rows_generic_kernel(
   }
 }
 
+// One problem's row operands as the launcher takes them (second = nullptr: one problem).
+struct AdalnRows {
+  const void *x; void* out; const void *shift, *scale;
+  int S;
+  const int64_t *xs, *os;
+  int64_t mod_stride_b;
+};
+
 template <typename T, typename TM, bool REF_ROUND>
-static int launch_adaln(const void* x, void* out, const void* shift, const void* scale,
+static int launch_adaln(const AdalnRows& r0, const AdalnRows* r1,
                         const int32_t* index, const float* ln_w, const float* ln_b,
-                        const float* shift_bias, const float* scale_bias, int B, int S, int C,
-                        const int64_t* xs, const int64_t* os, int64_t mod_stride_b,
+                        const float* shift_bias, const float* scale_bias, int B, int C,
                         int64_t mod_stride_s, float eps, hipStream_t stream) {
   constexpr int EPV = Vec16<T>::N;
   constexpr int EPM = Vec16<TM>::N;
-  const int64_t rows = static_cast<int64_t>(B) * S;
+  auto fill = [](const AdalnRows& r) {
+    AdalnProblem<T, TM> p;
+    p.x = static_cast<const T*>(r.x); p.out = static_cast<T*>(r.out);
+    p.shift = static_cast<const TM*>(r.shift); p.scale = static_cast<const TM*>(r.scale);
+    p.S = r.S; p.xs_b = r.xs[0]; p.xs_s = r.xs[1]; p.os_b = r.os[0]; p.os_s = r.os[1];
+    p.mod_stride_b = r.mod_stride_b;
+    return p;
+  };
   // EPV >= EPM always (TM is T or float), so C % EPV == 0 keeps parameter runs vector-aligned too.
-  const bool vec_ok = (C % EPV == 0) && aligned16(x) && aligned16(out) && xs[0] % EPV == 0 &&
-                      xs[1] % EPV == 0 && os[0] % EPV == 0 && os[1] % EPV == 0 &&
-                      aligned16(shift) && aligned16(scale) && mod_stride_b % EPM == 0 &&
+  auto rows_vec_ok = [&](const AdalnRows& r) {
+    return aligned16(r.x) && aligned16(r.out) && r.xs[0] % EPV == 0 && r.xs[1] % EPV == 0 && r.os[0] % EPV == 0 &&
+           r.os[1] % EPV == 0 && aligned16(r.shift) && aligned16(r.scale) && r.mod_stride_b % EPM == 0;
+  };
+  const AdalnProblem<T, TM> p0 = fill(r0), p1 = r1 ? fill(*r1) : p0;
+  const int64_t rows0 = static_cast<int64_t>(B) * r0.S, rows1 = r1 ? static_cast<int64_t>(B) * r1->S : 0;
+  const int64_t rows = rows0 + rows1;
+  const bool vec_ok = (C % EPV == 0) && rows_vec_ok(r0) && (!r1 || rows_vec_ok(*r1)) &&
                       mod_stride_s % EPM == 0 && aligned16(ln_w) && aligned16(ln_b) &&
                       aligned16(shift_bias) && aligned16(scale_bias);
   const int nvec = (C + EPV - 1) / EPV;  // 16-byte vectors per row
-  const bool plain = shift && scale && !index && !ln_w && !ln_b && !shift_bias && !scale_bias &&
-                     mod_stride_s == 0;
+  const bool plain = r0.shift && r0.scale && (!r1 || (r1->shift && r1->scale)) && !index && !ln_w && !ln_b &&
+                     !shift_bias && !scale_bias && mod_stride_s == 0;
 #define ODIT_ADALN_LAUNCH(WW, NVLL, PL)                                                            \
   hipLaunchKernelGGL((adaln_rows_kernel<T, TM, WW, NVLL, REF_ROUND, PL>),                          \
-                     dim3(static_cast<unsigned>(rows)), dim3(WW * 64), 0, stream,                  \
-                     static_cast<const T*>(x), static_cast<T*>(out), static_cast<const TM*>(shift), \
-                     static_cast<const TM*>(scale), index, ln_w, ln_b, shift_bias, scale_bias, B,  \
-                     S, C, xs[0], xs[1], os[0], os[1], mod_stride_b, mod_stride_s, eps)
+                     dim3(static_cast<unsigned>(rows)), dim3(WW * 64), 0, stream, p0, p1,          \
+                     static_cast<unsigned>(rows0), index, ln_w, ln_b, shift_bias, scale_bias, B,   \
+                     C, mod_stride_s, eps)
 #define ODIT_ADALN_CASE(WW, NVLL)                                                                  \
   do { if (plain) ODIT_ADALN_LAUNCH(WW, NVLL, true); else ODIT_ADALN_LAUNCH(WW, NVLL, false); } while (0)
   if (vec_ok && nvec <= 8 * 64 * 2 && rows <= 0x7fffffffll) {
@@ -219,12 +257,17 @@ static int launch_adaln(const void* x, void* out, const void* shift, const void*
     else if (nvec <= 768) ODIT_ADALN_CASE(6, 2);
     else ODIT_ADALN_CASE(8, 2);
   } else {
-    const dim3 grid(static_cast<unsigned>((rows + 3) / 4));
-    hipLaunchKernelGGL((adaln_rows_generic_kernel<T, TM, REF_ROUND>), grid, dim3(256), 0, stream,
-                       static_cast<const T*>(x), static_cast<T*>(out),
-                       static_cast<const TM*>(shift), static_cast<const TM*>(scale), index, ln_w,
-                       ln_b, shift_bias, scale_bias, B, S, C, xs[0], xs[1], os[0], os[1],
-                       mod_stride_b, mod_stride_s, eps);
+    // any width: one launch per problem
+    for (const AdalnRows* r : {&r0, r1}) {
+      if (r == nullptr) continue;
+      const int64_t n = static_cast<int64_t>(B) * r->S;
+      const dim3 grid(static_cast<unsigned>((n + 3) / 4));
+      hipLaunchKernelGGL((adaln_rows_generic_kernel<T, TM, REF_ROUND>), grid, dim3(256), 0, stream,
+                         static_cast<const T*>(r->x), static_cast<T*>(r->out),
+                         static_cast<const TM*>(r->shift), static_cast<const TM*>(r->scale), index, ln_w,
+                         ln_b, shift_bias, scale_bias, B, r->S, C, r->xs[0], r->xs[1], r->os[0], r->os[1],
+                         r->mod_stride_b, mod_stride_s, eps);
+    }
   }
 #undef ODIT_ADALN_CASE
 #undef ODIT_ADALN_LAUNCH
@@ -254,18 +297,54 @@ extern "C" int odit_adaln_modulate(const void* x, void* out, const void* shift, 
   if (B == 0 || S == 0) return ODIT_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool rr = (flags & ODIT_FLAG_REF_ROUNDING) && mod_dtype == dtype && dtype != ODIT_F32;
+  const AdalnRows r0{x, out, shift, scale, S, x_strides, out_strides, mod_stride_b};
 #define ODIT_ADALN_GO(T, TM)                                                                     \
-  return rr ? launch_adaln<T, TM, true>(x, out, shift, scale, index, ln_weight, ln_bias,           \
-                                        shift_bias, scale_bias, B, S, C, x_strides, out_strides,  \
-                                        mod_stride_b, mod_stride_s, eps, st)                      \
-            : launch_adaln<T, TM, false>(x, out, shift, scale, index, ln_weight, ln_bias,          \
-                                         shift_bias, scale_bias, B, S, C, x_strides, out_strides, \
-                                         mod_stride_b, mod_stride_s, eps, st)
+  return rr ? launch_adaln<T, TM, true>(r0, nullptr, index, ln_weight, ln_bias, shift_bias,       \
+                                        scale_bias, B, C, mod_stride_s, eps, st)                  \
+            : launch_adaln<T, TM, false>(r0, nullptr, index, ln_weight, ln_bias, shift_bias,      \
+                                         scale_bias, B, C, mod_stride_s, eps, st)
   if (mod_dtype == dtype) {
     ODIT_DISPATCH_DTYPE(dtype, T, ODIT_ADALN_GO(T, T));
   } else {
     ODIT_DISPATCH_DTYPE(dtype, T, ODIT_ADALN_GO(T, float));
   }
 #undef ODIT_ADALN_GO
+  return ODIT_OK;
+}
+
+extern "C" int odit_adaln_modulate_pair(const void* const x[2], void* const out[2], const void* const shift[2],
+                                        const void* const scale[2], int B, const int S[2], int C,
+                                        const int64_t x_strides[4], const int64_t out_strides[4],
+                                        const int64_t mod_stride_b[2], float eps, int mod_dtype, int dtype,
+                                        unsigned flags, void* stream) {
+  using namespace odit;
+  ODIT_CHECK_ARG(x && out && shift && scale && S && x_strides && out_strides && mod_stride_b,
+                 "odit_adaln_modulate_pair: null argument array");
+  for (int i = 0; i < 2; ++i) {
+    ODIT_CHECK_ARG(S[i] <= 0 || (x[i] && out[i]), "odit_adaln_modulate_pair: x/out must not be null");
+    ODIT_CHECK_ARG(S[i] >= 0 && mod_stride_b[i] >= 0, "odit_adaln_modulate_pair: bad S or modulation stride");
+  }
+  ODIT_CHECK_ARG(B >= 0 && C > 0, "odit_adaln_modulate_pair: bad shape B=%d C=%d", B, C);
+  ODIT_CHECK_ARG(mod_dtype == dtype || mod_dtype == ODIT_F32,
+                 "odit_adaln_modulate_pair: mod_dtype must equal dtype or be ODIT_F32 (got %d vs %d)", mod_dtype, dtype);
+  ODIT_CHECK_ARG(static_cast<int64_t>(B) * (static_cast<int64_t>(S[0]) + S[1]) < (1ll << 31),
+                 "odit_adaln_modulate_pair: too many rows");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool rr = (flags & ODIT_FLAG_REF_ROUNDING) && mod_dtype == dtype && dtype != ODIT_F32;
+  const AdalnRows r0{x[0], out[0], shift[0], scale[0], S[0], x_strides, out_strides, mod_stride_b[0]};
+  const AdalnRows r1{x[1], out[1], shift[1], scale[1], S[1], x_strides + 2, out_strides + 2, mod_stride_b[1]};
+  if (B == 0 || (S[0] == 0 && S[1] == 0)) return ODIT_OK;
+  // an empty problem leaves a single one
+  const AdalnRows& first = S[0] > 0 ? r0 : r1;
+  const AdalnRows* second = (S[0] > 0 && S[1] > 0) ? &r1 : nullptr;
+#define ODIT_ADALN_GO2(T, TM)                                                                        \
+  return rr ? launch_adaln<T, TM, true>(first, second, nullptr, nullptr, nullptr, nullptr, nullptr, B, C, 0, eps, st) \
+            : launch_adaln<T, TM, false>(first, second, nullptr, nullptr, nullptr, nullptr, nullptr, B, C, 0, eps, st)
+  if (mod_dtype == dtype) {
+    ODIT_DISPATCH_DTYPE(dtype, T, ODIT_ADALN_GO2(T, T));
+  } else {
+    ODIT_DISPATCH_DTYPE(dtype, T, ODIT_ADALN_GO2(T, float));
+  }
+#undef ODIT_ADALN_GO2
   return ODIT_OK;
 }

@@ -141,20 +141,43 @@ struct FastDiv {
 // IDX32: vector numbers, token numbers and element offsets fit 31 bits: the two divisions per lane (by
 // vectors per row, by tokens per batch row) become a multiply-high and a shift each and the addresses are a
 // base pointer plus a 32-bit offset.
+// One launch can carry TWO problems that write into the same joint buffers (the text rows and the image rows
+// of a dual-stream block: different inputs, weights, tables, lengths and row offsets): workgroups
+// [0, blocks0) belong to the first, the rest to the second. The choice is workgroup-uniform, so it costs a
+// handful of scalar selects; a single problem is blocks0 = gridDim.x.
+template <typename T, typename TW> struct QkFlatProblem {
+  const T *q_in, *k_in, *v_in;
+  const TW *wq, *wk;
+  const float *cos_t, *sin_t;
+  int S, out_seq_offset;
+  int64_t is_b, is_s, total_vec;
+  FastDiv by_s;
+};
+
 template <typename T, typename TW, int NORM_MODE, bool GENERAL, bool IDX32>
 __global__ __launch_bounds__(256) void qknorm_flat_kernel(
-    const T* __restrict__ q_in, const T* __restrict__ k_in, const T* __restrict__ v_in,
-    T* __restrict__ q_out, T* __restrict__ k_out, T* __restrict__ v_out,
-    const TW* __restrict__ wq, const TW* __restrict__ wk, const float* __restrict__ cos_t,
-    const float* __restrict__ sin_t, int S, int HD, int D, int rot, int64_t is_b, int64_t is_s,
-    int out_seq_offset, int S_total, float eps, int vec_per_row, int64_t total_vec, bool neox,
-    bool ref_round, FastDiv by_vpr, FastDiv by_s, float inv_d) {
+    const QkFlatProblem<T, TW> p0, const QkFlatProblem<T, TW> p1, unsigned blocks0,
+    T* __restrict__ q_out, T* __restrict__ k_out, T* __restrict__ v_out, int HD, int D, int rot,
+    int S_total, float eps, int vec_per_row, bool neox, bool ref_round, FastDiv by_vpr, float inv_d) {
   constexpr int EPV = Vec16<T>::N;
   const int lane = threadIdx.x & 63;
+  const bool second = blockIdx.x >= blocks0;  // workgroup-uniform
+  const T* __restrict__ q_in = second ? p1.q_in : p0.q_in;
+  const T* __restrict__ k_in = second ? p1.k_in : p0.k_in;
+  const T* __restrict__ v_in = second ? p1.v_in : p0.v_in;
+  const TW* __restrict__ wq = second ? p1.wq : p0.wq;
+  const TW* __restrict__ wk = second ? p1.wk : p0.wk;
+  const float* __restrict__ cos_t = second ? p1.cos_t : p0.cos_t;
+  const float* __restrict__ sin_t = second ? p1.sin_t : p0.sin_t;
+  const int S = second ? p1.S : p0.S;
+  const int out_seq_offset = second ? p1.out_seq_offset : p0.out_seq_offset;
+  const int64_t is_b = second ? p1.is_b : p0.is_b, is_s = second ? p1.is_s : p0.is_s;
+  const int64_t total_vec = second ? p1.total_vec : p0.total_vec;
+  const FastDiv by_s = {second ? p1.by_s.mul : p0.by_s.mul, second ? p1.by_s.shift : p0.by_s.shift};
   // grid.y: 0 = q together with k (when there is one), 1 = the copy of v. A lane takes the SAME vector
   // position of q and of k: one index computation, one pair of cos/sin loads, two loads in flight.
   const bool copy_v = blockIdx.y != 0;
-  const int64_t i_raw = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  const int64_t i_raw = static_cast<int64_t>(blockIdx.x - (second ? blocks0 : 0u)) * 256 + threadIdx.x;
   const bool valid = i_raw < total_vec;
   const int64_t i = valid ? i_raw : total_vec - 1;  // clamped lanes compute, never store
   int e0, b, s;
@@ -302,6 +325,13 @@ struct QkArgs {
   bool w_is_f32, neox, ref_round;
   int nv;
   hipStream_t stream;
+  // optional second problem of the same launch (per-head or no statistics only): same outputs, head
+  // layout, rotary width, weights' type and flags; its own inputs, weights, tables, length and row offset
+  bool pair = false;
+  const void *q_in2 = nullptr, *k_in2 = nullptr, *v_in2 = nullptr, *wq2 = nullptr, *wk2 = nullptr;
+  const float *cos2 = nullptr, *sin2 = nullptr;
+  int S2 = 0, out_seq_offset2 = 0;
+  int64_t is_b2 = 0, is_s2 = 0;
 };
 
 int qknorm_rope_bf16(const QkArgs& a);
@@ -311,21 +341,35 @@ int qknorm_rope_f32(const QkArgs& a);
 template <typename T, typename TW, int NORM_MODE, bool GENERAL> static int qk_flat(const QkArgs& a) {
   constexpr int EPV = Vec16<T>::N;
   const int vpr = a.HD / EPV;
-  const int64_t total = static_cast<int64_t>(a.B) * a.S * vpr;
+  QkFlatProblem<T, TW> p0, p1;
+  p0.q_in = static_cast<const T*>(a.q_in); p0.k_in = static_cast<const T*>(a.k_in); p0.v_in = static_cast<const T*>(a.v_in);
+  p0.wq = static_cast<const TW*>(a.wq); p0.wk = static_cast<const TW*>(a.wk);
+  p0.cos_t = a.cos; p0.sin_t = a.sin; p0.S = a.S; p0.out_seq_offset = a.out_seq_offset;
+  p0.is_b = a.is_b; p0.is_s = a.is_s; p0.total_vec = static_cast<int64_t>(a.B) * a.S * vpr;
+  p0.by_s = FastDiv::make(static_cast<uint32_t>(a.S));
+  p1 = p0;
+  if (a.pair) {
+    p1.q_in = static_cast<const T*>(a.q_in2); p1.k_in = static_cast<const T*>(a.k_in2); p1.v_in = static_cast<const T*>(a.v_in2);
+    p1.wq = static_cast<const TW*>(a.wq2); p1.wk = static_cast<const TW*>(a.wk2);
+    p1.cos_t = a.cos2; p1.sin_t = a.sin2; p1.S = a.S2; p1.out_seq_offset = a.out_seq_offset2;
+    p1.is_b = a.is_b2; p1.is_s = a.is_s2; p1.total_vec = static_cast<int64_t>(a.B) * a.S2 * vpr;
+    p1.by_s = FastDiv::make(static_cast<uint32_t>(a.S2));
+  }
+  const int64_t blocks0 = (p0.total_vec + 255) / 256, blocks1 = a.pair ? (p1.total_vec + 255) / 256 : 0;
   const int nparts = 1 + (a.v_in != nullptr);  // q (with k) | v
-  const dim3 grid(static_cast<unsigned>((total + 255) / 256), nparts);
+  const dim3 grid(static_cast<unsigned>(blocks0 + blocks1), nparts);
 #define ODIT_QK_FLAT(I32)                                                                          \
   hipLaunchKernelGGL((qknorm_flat_kernel<T, TW, NORM_MODE, GENERAL, I32>), grid, dim3(256), 0, a.stream, \
-                     static_cast<const T*>(a.q_in), static_cast<const T*>(a.k_in),                  \
-                     static_cast<const T*>(a.v_in), static_cast<T*>(a.q_out), static_cast<T*>(a.k_out), \
-                     static_cast<T*>(a.v_out), static_cast<const TW*>(a.wq), static_cast<const TW*>(a.wk), \
-                     a.cos, a.sin, a.S, a.HD, a.D, a.rot, a.is_b, a.is_s, a.out_seq_offset, a.S_total, \
-                     a.eps, vpr, total, a.neox, a.ref_round, FastDiv::make(static_cast<uint32_t>(vpr)), \
-                     FastDiv::make(static_cast<uint32_t>(a.S)), 1.f / static_cast<float>(a.D))
+                     p0, p1, static_cast<unsigned>(blocks0), static_cast<T*>(a.q_out), static_cast<T*>(a.k_out), \
+                     static_cast<T*>(a.v_out), a.HD, a.D, a.rot, a.S_total, a.eps, vpr, a.neox, a.ref_round, \
+                     FastDiv::make(static_cast<uint32_t>(vpr)), 1.f / static_cast<float>(a.D))
   // 32-bit indexing: vector numbers and every element offset of the inputs and of the joint outputs below 2^31
   const int64_t in_span = (a.B - 1) * a.is_b + (a.S - 1) * a.is_s + a.HD;
+  const int64_t in_span2 = a.pair ? (a.B - 1) * a.is_b2 + (a.S2 - 1) * a.is_s2 + a.HD : 0;
   const int64_t out_span = static_cast<int64_t>(a.B) * a.S_total * a.HD;
-  const bool idx32 = total < (1ll << 31) && in_span < (1ll << 31) && out_span < (1ll << 31) && a.is_b >= 0 && a.is_s >= 0;
+  const bool idx32 = p0.total_vec < (1ll << 31) && p1.total_vec < (1ll << 31) && blocks0 + blocks1 < (1ll << 31) &&
+                     in_span < (1ll << 31) && in_span2 < (1ll << 31) && out_span < (1ll << 31) &&
+                     a.is_b >= 0 && a.is_s >= 0 && a.is_b2 >= 0 && a.is_s2 >= 0;
   if (idx32) ODIT_QK_FLAT(true); else ODIT_QK_FLAT(false);
 #undef ODIT_QK_FLAT
   return check_launch("odit_qknorm_rope");
@@ -377,13 +421,13 @@ int qknorm_rope_f32(const QkArgs& a) { return qk_go<float, float>(a); }
 }  // namespace odit
 
 #if ODIT_QK_TU == 0
-extern "C" int odit_qknorm_rope(const void* q_in, const void* k_in, const void* v_in, void* q_out,
-                                void* k_out, void* v_out, const void* wq, const void* wk,
-                                const float* cos, const float* sin, int B, int S, int H, int D,
-                                int rot, const int64_t in_strides[2], int out_seq_offset,
-                                int S_total, float eps, int norm_mode, int w_dtype, int dtype,
-                                unsigned flags, void* stream) {
-  using namespace odit;
+namespace odit {
+
+// argument checks of one problem and its launch arguments; *empty is set when there is nothing to do
+static int qk_fill(const void* q_in, const void* k_in, const void* v_in, void* q_out, void* k_out, void* v_out,
+                   const void* wq, const void* wk, const float* cos, const float* sin, int B, int S, int H, int D,
+                   int rot, const int64_t* in_strides, int out_seq_offset, int S_total, float eps, int norm_mode,
+                   int w_dtype, int dtype, unsigned flags, void* stream, QkArgs& a, bool* empty) {
   ODIT_CHECK_ARG(dtype == ODIT_BF16 || dtype == ODIT_F16 || dtype == ODIT_F32,
                  "odit_qknorm_rope: unknown dtype code %d", dtype);
   ODIT_CHECK_ARG(q_in && q_out, "odit_qknorm_rope: q_in/q_out must not be null");
@@ -424,9 +468,8 @@ extern "C" int odit_qknorm_rope(const void* q_in, const void* k_in, const void* 
               static_cast<long long>(HD), 16 * 64 * epv);
     return ODIT_ENOTSUP;
   }
-  if (B == 0 || S == 0) return ODIT_OK;
+  *empty = B == 0 || S == 0;
   ODIT_CHECK_ARG(static_cast<int64_t>(B) * S <= 0x7fffffffll, "odit_qknorm_rope: B*S exceeds 2^31 - 1 rows");
-  QkArgs a;
   a.q_in = q_in; a.k_in = k_in; a.v_in = v_in;
   a.q_out = q_out; a.k_out = k_out; a.v_out = v_out;
   a.wq = wq; a.wk = wk; a.cos = cos; a.sin = sin;
@@ -439,10 +482,69 @@ extern "C" int odit_qknorm_rope(const void* q_in, const void* k_in, const void* 
   a.ref_round = (flags & ODIT_FLAG_REF_ROUNDING) && dtype != ODIT_F32;
   a.nv = nv;
   a.stream = static_cast<hipStream_t>(stream);
+  return ODIT_OK;
+}
+
+static int qk_dispatch(const QkArgs& a, int dtype) {
   switch (dtype) {
     case ODIT_BF16: return qknorm_rope_bf16(a);
     case ODIT_F16: return qknorm_rope_f16(a);
     default: return qknorm_rope_f32(a);
   }
+}
+
+}  // namespace odit
+
+extern "C" int odit_qknorm_rope(const void* q_in, const void* k_in, const void* v_in, void* q_out,
+                                void* k_out, void* v_out, const void* wq, const void* wk,
+                                const float* cos, const float* sin, int B, int S, int H, int D,
+                                int rot, const int64_t in_strides[2], int out_seq_offset,
+                                int S_total, float eps, int norm_mode, int w_dtype, int dtype,
+                                unsigned flags, void* stream) {
+  using namespace odit;
+  QkArgs a;
+  bool empty = false;
+  const int rc = qk_fill(q_in, k_in, v_in, q_out, k_out, v_out, wq, wk, cos, sin, B, S, H, D, rot, in_strides,
+                         out_seq_offset, S_total, eps, norm_mode, w_dtype, dtype, flags, stream, a, &empty);
+  if (rc != ODIT_OK || empty) return rc;
+  return qk_dispatch(a, dtype);
+}
+
+extern "C" int odit_qknorm_rope_pair(const void* const q_in[2], const void* const k_in[2],
+                                     const void* const v_in[2], void* q_out, void* k_out, void* v_out,
+                                     const void* const wq[2], const void* const wk[2],
+                                     const float* const cos[2], const float* const sin[2], int B,
+                                     const int S[2], int H, int D, int rot, const int64_t in_strides[4],
+                                     const int out_seq_offset[2], int S_total, float eps, int norm_mode,
+                                     int w_dtype, int dtype, unsigned flags, void* stream) {
+  using namespace odit;
+  ODIT_CHECK_ARG(q_in && k_in && v_in && wq && wk && cos && sin && S && in_strides && out_seq_offset,
+                 "odit_qknorm_rope_pair: null argument array");
+  ODIT_CHECK_ARG((k_in[0] == nullptr) == (k_in[1] == nullptr) && (v_in[0] == nullptr) == (v_in[1] == nullptr) &&
+                     (cos[0] == nullptr) == (cos[1] == nullptr),
+                 "odit_qknorm_rope_pair: both problems take the same optional operands (k, v, rotary tables)");
+  QkArgs a[2];
+  bool empty[2] = {false, false};
+  for (int i = 0; i < 2; ++i) {
+    const int rc = qk_fill(q_in[i], k_in[i], v_in[i], q_out, k_in[i] ? k_out : nullptr, v_in[i] ? v_out : nullptr,
+                           wq[i], wk[i], cos[i], sin[i], B, S[i], H, D, rot, in_strides + 2 * i, out_seq_offset[i],
+                           S_total, eps, norm_mode, w_dtype, dtype, flags, stream, a[i], &empty[i]);
+    if (rc != ODIT_OK) return rc;
+  }
+  // one launch when the flat kernel takes both; whole-row statistics, or an empty problem: one call each
+  if (norm_mode == ODIT_NORM_ROW || empty[0] || empty[1]) {
+    for (int i = 0; i < 2; ++i) {
+      if (empty[i]) continue;
+      const int rc = qk_dispatch(a[i], dtype);
+      if (rc != ODIT_OK) return rc;
+    }
+    return ODIT_OK;
+  }
+  QkArgs m = a[0];
+  m.pair = true;
+  m.q_in2 = a[1].q_in; m.k_in2 = a[1].k_in; m.v_in2 = a[1].v_in; m.wq2 = a[1].wq; m.wk2 = a[1].wk;
+  m.cos2 = a[1].cos; m.sin2 = a[1].sin; m.S2 = a[1].S; m.out_seq_offset2 = a[1].out_seq_offset;
+  m.is_b2 = a[1].is_b; m.is_s2 = a[1].is_s;
+  return qk_dispatch(m, dtype);
 }
 #endif

@@ -228,6 +228,20 @@ def qknorm_rope(
     a fused-QKV projection). *_out: dense [B,S_total,H,D]; input row s goes to row out_seq_offset+s.
     cos/sin: float32 [S, rot/2] or None.
     """
+    B, S, H, D, S_total, rot, w_dtype, cos, sin = _qk_problem(q, k, v, q_out, k_out, v_out, wq, wk, cos, sin, norm_mode)
+    flags = (ODIT_FLAG_NEOX if neox else 0) | (ODIT_FLAG_REF_ROUNDING if ref_rounding else 0)
+    lib = _lib.load()
+    rc = lib.odit_qknorm_rope(
+        q.data_ptr(), _ptr(k), _ptr(v), q_out.data_ptr(), _ptr(k_out), _ptr(v_out),
+        _ptr(wq), _ptr(wk), _ptr(cos), _ptr(sin),
+        B, S, H, D, rot, _lib.i64_array(q.stride()[:2]), int(out_seq_offset), int(S_total),
+        float(eps), int(norm_mode), w_dtype, _code(q), flags, _stream(),
+    )
+    _lib.check(rc, "odit_qknorm_rope")
+
+
+def _qk_problem(q, k, v, q_out, k_out, v_out, wq, wk, cos, sin, norm_mode):
+    """Checks of one qknorm_rope problem; returns (B, S, H, D, S_total, rot, w_dtype, cos, sin)."""
     _dev(q, k, v, q_out, k_out, v_out, wq, wk, cos, sin)
     if q.dim() != 4:
         raise ValueError("qknorm_rope expects [B,S,H,D] inputs")
@@ -270,15 +284,43 @@ def qknorm_rope(
             if any(w.dtype != ws[0].dtype for w in ws):
                 raise TypeError("wq and wk must share a dtype")
             w_dtype = _code(ws[0])
+    return B, S, H, D, S_total, rot, w_dtype, cos, sin
+
+
+def qknorm_rope_pair(first: tuple, second: tuple, q_out: torch.Tensor, k_out: torch.Tensor | None,
+                     v_out: torch.Tensor | None, *, eps: float = 1e-6, norm_mode: int = ODIT_NORM_HEAD,
+                     neox: bool = False, ref_rounding: bool = False) -> None:
+    """Two ``qknorm_rope`` problems that fill different rows of the same joint buffers (the text rows and
+    the image rows of a dual-stream block) in ONE launch. Each problem is
+    (q, k, v, wq, wk, cos, sin, out_seq_offset) with the meaning of ``qknorm_rope``'s arguments; both take the
+    same optional operands, head layout, rotary width and dtypes."""
+    probs = []
+    for (q, k, v, wq, wk, cos, sin, off) in (first, second):
+        probs.append((q, k, v, wq, wk, int(off)) +
+                     _qk_problem(q, k, v, q_out, k_out if k is not None else None, v_out if v is not None else None,
+                                 wq, wk, cos, sin, norm_mode))
+    a, b = probs
+    # (B, H, D, S_total, rot, w_dtype) shared
+    if (a[6], a[8], a[9], a[10], a[11], a[12]) != (b[6], b[8], b[9], b[10], b[11], b[12]) or a[0].dtype != b[0].dtype:
+        raise ValueError("qknorm_rope_pair: the two problems must share batch, heads, rotary width and dtypes")
+    for i in (1, 2):
+        if (a[i] is None) != (b[i] is None):
+            raise ValueError("qknorm_rope_pair: both problems take the same optional operands")
+    if (a[13] is None) != (b[13] is None):
+        raise ValueError("qknorm_rope_pair: both problems take rotary tables or neither does")
+    vp, fp = _lib.ptr_array, _lib.ptr_array
     flags = (ODIT_FLAG_NEOX if neox else 0) | (ODIT_FLAG_REF_ROUNDING if ref_rounding else 0)
     lib = _lib.load()
-    rc = lib.odit_qknorm_rope(
-        q.data_ptr(), _ptr(k), _ptr(v), q_out.data_ptr(), _ptr(k_out), _ptr(v_out),
-        _ptr(wq), _ptr(wk), _ptr(cos), _ptr(sin),
-        B, S, H, D, rot, _lib.i64_array(q.stride()[:2]), int(out_seq_offset), int(S_total),
-        float(eps), int(norm_mode), w_dtype, _code(q), flags, _stream(),
+    rc = lib.odit_qknorm_rope_pair(
+        vp([_ptr(a[0]), _ptr(b[0])]), vp([_ptr(a[1]), _ptr(b[1])]), vp([_ptr(a[2]), _ptr(b[2])]),
+        q_out.data_ptr(), _ptr(k_out), _ptr(v_out),
+        vp([_ptr(a[3]), _ptr(b[3])]), vp([_ptr(a[4]), _ptr(b[4])]),
+        fp([_ptr(a[13]), _ptr(b[13])]), fp([_ptr(a[14]), _ptr(b[14])]),
+        a[6], _lib.int_array([a[7], b[7]]), a[8], a[9], a[11],
+        _lib.i64_array(tuple(a[0].stride()[:2]) + tuple(b[0].stride()[:2])), _lib.int_array([a[5], b[5]]),
+        int(a[10]), float(eps), int(norm_mode), a[12], _code(a[0]), flags, _stream(),
     )
-    _lib.check(rc, "odit_qknorm_rope")
+    _lib.check(rc, "odit_qknorm_rope_pair")
 
 
 # --------------------------------------------------------------------------------------------- K3
@@ -354,6 +396,44 @@ def adaln_modulate(
     )
     _lib.check(rc, "odit_adaln_modulate")
     return out
+
+
+def adaln_modulate_pair(first: tuple, second: tuple, *, eps: float = 1e-6,
+                        ref_rounding: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
+    """``adaln_modulate`` for two tensors of the same width and batch (the image and the text stream of a
+    dual-stream block) in ONE launch. Each problem is (x [B,S,C], shift [B,C], scale [B,C]): one modulation row per
+    batch entry; returns the two results."""
+    outs, rows = [], []
+    for (x, shift, scale) in (first, second):
+        _dev(x, shift, scale)
+        if x.dim() != 3:
+            raise ValueError("adaln_modulate_pair expects x [B,S,C]")
+        B, S, Cdim = x.shape
+        _last_contig(x, "x")
+        for name, t in (("shift", shift), ("scale", scale)):
+            if t is None or t.dim() != 2 or tuple(t.shape) != (B, Cdim):
+                raise ValueError(f"{name}: expected [{B},{Cdim}]")
+            _last_contig(t, name)
+        if shift.dtype != scale.dtype or shift.stride(0) != scale.stride(0):
+            raise ValueError("shift and scale must share dtype and strides")
+        out = torch.empty((B, S, Cdim), dtype=x.dtype, device=x.device)
+        outs.append(out)
+        rows.append((x, out, shift, scale, B, S, Cdim, shift.stride(0) if B > 1 else 0))
+    a, b = rows
+    if (a[4], a[6]) != (b[4], b[6]) or a[0].dtype != b[0].dtype or a[2].dtype != b[2].dtype:
+        raise ValueError("adaln_modulate_pair: the two problems must share batch, width and dtypes")
+    lib = _lib.load()
+    rc = lib.odit_adaln_modulate_pair(
+        _lib.ptr_array([a[0].data_ptr(), b[0].data_ptr()]), _lib.ptr_array([a[1].data_ptr(), b[1].data_ptr()]),
+        _lib.ptr_array([a[2].data_ptr(), b[2].data_ptr()]), _lib.ptr_array([a[3].data_ptr(), b[3].data_ptr()]),
+        a[4], _lib.int_array([a[5], b[5]]), a[6],
+        _lib.i64_array(tuple(a[0].stride()[:2]) + tuple(b[0].stride()[:2])),
+        _lib.i64_array(tuple(a[1].stride()[:2]) + tuple(b[1].stride()[:2])),
+        _lib.i64_array([a[7], b[7]]), float(eps), _code(a[2]), _code(a[0]),
+        ODIT_FLAG_REF_ROUNDING if ref_rounding else 0, _stream(),
+    )
+    _lib.check(rc, "odit_adaln_modulate_pair")
+    return outs[0], outs[1]
 
 
 # --------------------------------------------------------------------------------------------- K4

@@ -56,3 +56,17 @@ class AdaLayerNorm(CustomOp):
             nb = gate.size(0) // 2
             gate_result = torch.where(index.unsqueeze(-1) == 0, gate[:nb].unsqueeze(1), gate[nb:].unsqueeze(1))
         return (out.squeeze(0) if squeeze else out), gate_result
+
+
+def adaln_pair(norm_a: AdaLayerNorm, x_a: torch.Tensor, mod_a: torch.Tensor,
+               norm_b: AdaLayerNorm, x_b: torch.Tensor, mod_b: torch.Tensor):
+    """``norm_a(x_a, mod_a)`` and ``norm_b(x_b, mod_b)`` (no index, no LayerNorm affine) in ONE launch: the
+    two streams of a dual-stream block. Returns ((out_a, gate_a), (out_b, gate_b))."""
+    if (norm_a.elementwise_affine or norm_b.elementwise_affine or norm_a.eps != norm_b.eps
+            or norm_a.ref_rounding != norm_b.ref_rounding or x_a.dim() != 3 or x_b.dim() != 3):
+        return norm_a(x_a, mod_a), norm_b(x_b, mod_b)
+    shift_a, scale_a, gate_a = mod_a.chunk(3, dim=-1)
+    shift_b, scale_b, gate_b = mod_b.chunk(3, dim=-1)
+    out_a, out_b = kernels.adaln_modulate_pair((x_a, shift_a, scale_a), (x_b, shift_b, scale_b), eps=norm_a.eps,
+                                               ref_rounding=norm_a.ref_rounding)
+    return (out_a, gate_a.unsqueeze(1)), (out_b, gate_b.unsqueeze(1))
