@@ -146,12 +146,13 @@ class FluxAttention(nn.Module):
         tc = ts = ic = isn = None
         if rot is not None:
             tc, ts, ic, isn = rot.cos32[:S_c], rot.sin32[:S_c], rot.cos32[S_c:], rot.sin32[S_c:]
-        kernels.qknorm_rope(cqkv[:, :, 0], cqkv[:, :, 1], None if v_in_place else cqkv[:, :, 2], jq, jk, jv,
-                            self.norm_added_q.weight, self.norm_added_k.weight, tc, ts, eps=self.eps,
-                            out_seq_offset=0, norm_mode=ODIT_NORM_HEAD, ref_rounding=rr)
-        kernels.qknorm_rope(qkv[:, :, 0], qkv[:, :, 1], None if v_in_place else qkv[:, :, 2], jq, jk, jv,
-                            self.norm_q.weight, self.norm_k.weight, ic, isn, eps=self.eps, out_seq_offset=S_c,
-                            norm_mode=ODIT_NORM_HEAD, ref_rounding=rr)
+        # context rows [0, S_c) and image rows [S_c, S) of the joint buffers, one launch for both streams
+        kernels.qknorm_rope_pair(
+            (cqkv[:, :, 0], cqkv[:, :, 1], None if v_in_place else cqkv[:, :, 2],
+             self.norm_added_q.weight, self.norm_added_k.weight, tc, ts, 0),
+            (qkv[:, :, 0], qkv[:, :, 1], None if v_in_place else qkv[:, :, 2],
+             self.norm_q.weight, self.norm_k.weight, ic, isn, S_c),
+            jq, jk, jv, eps=self.eps, norm_mode=ODIT_NORM_HEAD, ref_rounding=rr)
         meta = AttentionMetadata(output_split=S_c)
         if v_in_place:
             jv, meta.value_tail = cqkv[:, :, 2], qkv[:, :, 2]
@@ -195,20 +196,27 @@ class FluxTransformerBlock(nn.Module):
         if gate_rows is not None:
             pre = [[(gate_rows[0][:, s, j], gate_rows[1][:, s, j]) for j in range(2)] for s in range(2)]
         m_x, m_c = mod_params if mod_params is not None else (None, None)
-        n_x, gate_msa, shift_mlp, scale_mlp, gate_mlp = self.norm1(hidden_states, emb=temb, mod=m_x)
-        n_c, c_gate_msa, c_shift_mlp, c_scale_mlp, c_gate_mlp = self.norm1_context(encoder_hidden_states,
-                                                                                   emb=temb, mod=m_c)
+        # the two streams' norms are one launch each time (norm1 / norm1_context, norm2 / norm2_context)
+        if m_x is None:
+            m_x = self.norm1.linear(kernels.silu(temb))
+        if m_c is None:
+            m_c = self.norm1_context.linear(kernels.silu(temb))
+        shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = m_x.chunk(6, dim=1)
+        c_shift_msa, c_scale_msa, c_gate_msa, c_shift_mlp, c_scale_mlp, c_gate_mlp = m_c.chunk(6, dim=1)
+        n_x, n_c = kernels.adaln_modulate_pair((hidden_states, shift_msa, scale_msa),
+                                               (encoder_hidden_states, c_shift_msa, c_scale_msa),
+                                               eps=self.norm1.eps, ref_rounding=rr)
         # inputs are never written (callers such as TeaCache keep them to form residuals): the attention
         # residuals land in new tensors, the feed-forward residuals then update those in place
         hidden_states, encoder_hidden_states = self.attn(
             hidden_states=n_x, encoder_hidden_states=n_c, image_rotary_emb=image_rotary_emb,
             residuals=(hidden_states, gate_msa, encoder_hidden_states, c_gate_msa, pre[0][0], pre[1][0]),
             **(joint_attention_kwargs or {}))
-        n2 = kernels.adaln_modulate(hidden_states, shift_mlp, scale_mlp, eps=self.norm2.eps, ref_rounding=rr)
+        n2, c2 = kernels.adaln_modulate_pair((hidden_states, shift_mlp, scale_mlp),
+                                             (encoder_hidden_states, c_shift_mlp, c_scale_mlp),
+                                             eps=self.norm2.eps, ref_rounding=rr)
         hidden_states = self.ff.forward_residual(n2, hidden_states, gate_mlp, out=hidden_states, ref_rounding=rr,
                                                  pre=pre[0][1])
-        c2 = kernels.adaln_modulate(encoder_hidden_states, c_shift_mlp, c_scale_mlp, eps=self.norm2_context.eps,
-                                    ref_rounding=rr)
         encoder_hidden_states = self.ff_context.forward_residual(c2, encoder_hidden_states, c_gate_mlp,
                                                                  out=encoder_hidden_states, ref_rounding=rr,
                                                                  pre=pre[1][1])
