@@ -253,6 +253,29 @@ def test_rel_l1_closed_forms(gpu):
 
 
 # ========================================================================================= K2
+@pytest.mark.parametrize("C", [3072, 2048, 1536, 1160])
+def test_adaln_many_rows_two_per_wavefront(gpu, C):
+    """From 6144 rows on the per-block form puts two rows on a wavefront: an odd row count (the last wavefront
+    has one row), 3, 4, 5 and 6 vectors per lane, alone and as a pair whose second problem starts in the middle of
+    the first wavefronts' second rows; against the oracle and, bit for bit, against calls of few rows each."""
+    from vllm_omni_amd import kernels
+
+    B, S = 1, 6145
+    x = _rand(B, S, C, seed=11, dtype=torch.bfloat16, scale=1.5).to(gpu)
+    mod = (_rand(B, 3 * C, seed=12, dtype=torch.bfloat16) * 0.3).to(gpu)
+    got = kernels.adaln_modulate(x, mod[:, :C], mod[:, C:2 * C], eps=1e-6)
+    want = ops.ada_layer_norm(x.float().cpu(), mod.float().cpu(), eps=1e-6)[0]
+    _close(got, want, atol=2e-2, rtol=2e-2, what="adaln, two rows per wavefront")
+    few = torch.cat([kernels.adaln_modulate(x[:, i:i + 1000], mod[:, :C], mod[:, C:2 * C], eps=1e-6)
+                     for i in range(0, S, 1000)], dim=1)
+    assert torch.equal(got, few), "a row's result depends on how many rows the call has"
+    x2 = _rand(B, 77, C, seed=13, dtype=torch.bfloat16).to(gpu)
+    mod2 = (_rand(B, 3 * C, seed=14, dtype=torch.bfloat16) * 0.3).to(gpu)
+    a, b = kernels.adaln_modulate_pair((x, mod[:, :C], mod[:, C:2 * C]), (x2, mod2[:, :C], mod2[:, C:2 * C]), eps=1e-6)
+    assert torch.equal(a, got)
+    assert torch.equal(b, kernels.adaln_modulate(x2, mod2[:, :C], mod2[:, C:2 * C], eps=1e-6))
+
+
 # ---- two problems in one launch (the image and the text stream of a dual-stream block) ----------
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("C,S0,S1", [(3072, 70, 9), (256, 5, 33), (37, 4, 6)])
