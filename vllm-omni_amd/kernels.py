@@ -296,29 +296,30 @@ def qknorm_rope_pair(first: tuple, second: tuple, q_out: torch.Tensor, k_out: to
     same optional operands, head layout, rotary width and dtypes."""
     probs = []
     for (q, k, v, wq, wk, cos, sin, off) in (first, second):
-        probs.append((q, k, v, wq, wk, int(off)) +
-                     _qk_problem(q, k, v, q_out, k_out if k is not None else None, v_out if v is not None else None,
-                                 wq, wk, cos, sin, norm_mode))
+        B, S, H, D, S_total, rot, w_dtype, cos, sin = _qk_problem(
+            q, k, v, q_out, k_out if k is not None else None, v_out if v is not None else None, wq, wk, cos, sin,
+            norm_mode)
+        probs.append(dict(q=q, k=k, v=v, wq=wq, wk=wk, cos=cos, sin=sin, off=int(off), S=S,
+                          shared=(B, H, D, S_total, rot, w_dtype, q.dtype)))
     a, b = probs
-    # (B, H, D, S_total, rot, w_dtype) shared
-    if (a[6], a[8], a[9], a[10], a[11], a[12]) != (b[6], b[8], b[9], b[10], b[11], b[12]) or a[0].dtype != b[0].dtype:
+    if a["shared"] != b["shared"]:
         raise ValueError("qknorm_rope_pair: the two problems must share batch, heads, rotary width and dtypes")
-    for i in (1, 2):
-        if (a[i] is None) != (b[i] is None):
-            raise ValueError("qknorm_rope_pair: both problems take the same optional operands")
-    if (a[13] is None) != (b[13] is None):
-        raise ValueError("qknorm_rope_pair: both problems take rotary tables or neither does")
-    vp, fp = _lib.ptr_array, _lib.ptr_array
+    for name in ("k", "v", "cos"):
+        if (a[name] is None) != (b[name] is None):
+            raise ValueError(f"qknorm_rope_pair: both problems take {name} or neither does")
+    B, H, D, S_total, rot, w_dtype, _ = a["shared"]
+
+    def both(name):  # the two problems' device addresses of one operand
+        return _lib.ptr_array([_ptr(a[name]), _ptr(b[name])])
+
     flags = (ODIT_FLAG_NEOX if neox else 0) | (ODIT_FLAG_REF_ROUNDING if ref_rounding else 0)
     lib = _lib.load()
     rc = lib.odit_qknorm_rope_pair(
-        vp([_ptr(a[0]), _ptr(b[0])]), vp([_ptr(a[1]), _ptr(b[1])]), vp([_ptr(a[2]), _ptr(b[2])]),
-        q_out.data_ptr(), _ptr(k_out), _ptr(v_out),
-        vp([_ptr(a[3]), _ptr(b[3])]), vp([_ptr(a[4]), _ptr(b[4])]),
-        fp([_ptr(a[13]), _ptr(b[13])]), fp([_ptr(a[14]), _ptr(b[14])]),
-        a[6], _lib.int_array([a[7], b[7]]), a[8], a[9], a[11],
-        _lib.i64_array(tuple(a[0].stride()[:2]) + tuple(b[0].stride()[:2])), _lib.int_array([a[5], b[5]]),
-        int(a[10]), float(eps), int(norm_mode), a[12], _code(a[0]), flags, _stream(),
+        both("q"), both("k"), both("v"), q_out.data_ptr(), _ptr(k_out), _ptr(v_out),
+        both("wq"), both("wk"), both("cos"), both("sin"),
+        B, _lib.int_array([a["S"], b["S"]]), H, D, rot,
+        _lib.i64_array(tuple(a["q"].stride()[:2]) + tuple(b["q"].stride()[:2])), _lib.int_array([a["off"], b["off"]]),
+        int(S_total), float(eps), int(norm_mode), w_dtype, _code(a["q"]), flags, _stream(),
     )
     _lib.check(rc, "odit_qknorm_rope_pair")
 
@@ -403,7 +404,7 @@ def adaln_modulate_pair(first: tuple, second: tuple, *, eps: float = 1e-6,
     """``adaln_modulate`` for two tensors of the same width and batch (the image and the text stream of a
     dual-stream block) in ONE launch. Each problem is (x [B,S,C], shift [B,C], scale [B,C]): one modulation row per
     batch entry; returns the two results."""
-    outs, rows = [], []
+    probs = []
     for (x, shift, scale) in (first, second):
         _dev(x, shift, scale)
         if x.dim() != 3:
@@ -416,24 +417,27 @@ def adaln_modulate_pair(first: tuple, second: tuple, *, eps: float = 1e-6,
             _last_contig(t, name)
         if shift.dtype != scale.dtype or shift.stride(0) != scale.stride(0):
             raise ValueError("shift and scale must share dtype and strides")
-        out = torch.empty((B, S, Cdim), dtype=x.dtype, device=x.device)
-        outs.append(out)
-        rows.append((x, out, shift, scale, B, S, Cdim, shift.stride(0) if B > 1 else 0))
-    a, b = rows
-    if (a[4], a[6]) != (b[4], b[6]) or a[0].dtype != b[0].dtype or a[2].dtype != b[2].dtype:
+        probs.append(dict(x=x, out=torch.empty((B, S, Cdim), dtype=x.dtype, device=x.device), shift=shift, scale=scale,
+                          S=S, mod_stride=shift.stride(0) if B > 1 else 0, shared=(B, Cdim, x.dtype, shift.dtype)))
+    a, b = probs
+    if a["shared"] != b["shared"]:
         raise ValueError("adaln_modulate_pair: the two problems must share batch, width and dtypes")
+    B, Cdim = a["shared"][:2]
+
+    def both(name):
+        return _lib.ptr_array([a[name].data_ptr(), b[name].data_ptr()])
+
+    def strides(name):  # (batch, seq) strides of both problems, side by side
+        return _lib.i64_array(tuple(a[name].stride()[:2]) + tuple(b[name].stride()[:2]))
+
     lib = _lib.load()
     rc = lib.odit_adaln_modulate_pair(
-        _lib.ptr_array([a[0].data_ptr(), b[0].data_ptr()]), _lib.ptr_array([a[1].data_ptr(), b[1].data_ptr()]),
-        _lib.ptr_array([a[2].data_ptr(), b[2].data_ptr()]), _lib.ptr_array([a[3].data_ptr(), b[3].data_ptr()]),
-        a[4], _lib.int_array([a[5], b[5]]), a[6],
-        _lib.i64_array(tuple(a[0].stride()[:2]) + tuple(b[0].stride()[:2])),
-        _lib.i64_array(tuple(a[1].stride()[:2]) + tuple(b[1].stride()[:2])),
-        _lib.i64_array([a[7], b[7]]), float(eps), _code(a[2]), _code(a[0]),
-        ODIT_FLAG_REF_ROUNDING if ref_rounding else 0, _stream(),
+        both("x"), both("out"), both("shift"), both("scale"), B, _lib.int_array([a["S"], b["S"]]), Cdim,
+        strides("x"), strides("out"), _lib.i64_array([a["mod_stride"], b["mod_stride"]]), float(eps),
+        _code(a["shift"]), _code(a["x"]), ODIT_FLAG_REF_ROUNDING if ref_rounding else 0, _stream(),
     )
     _lib.check(rc, "odit_adaln_modulate_pair")
-    return outs[0], outs[1]
+    return a["out"], b["out"]
 
 
 # --------------------------------------------------------------------------------------------- K4
