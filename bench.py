@@ -403,6 +403,24 @@ def kernel_rooflines(torch):
     fl = 2.0 * xm.shape[0] * C * MLP_RATIO * C
     out["gemm_mlp_up(hipBLASLt)"] = {"ms": ms, "TFLOP/s": fl / ms / 1e9,
                                      "frac_mfma": fl / ms / 1e9 / PEAK_MFMA_BF16_TFLOPS}
+    # the text stream's MLP down-projection with its gated residual (M = B * S_TXT rows, one gate vector per
+    # batch row) on the hand-written stream-K kernel and on the library, weights rotating so each call reads cold ones
+    del xm, wm, bm
+    n_w = 8
+    xt = torch.randn(B, S_TXT, MLP_RATIO * C, device=dev, dtype=bf)
+    wts = [torch.randn(C, MLP_RATIO * C, device=dev, dtype=bf) * 0.02 for _ in range(n_w)]
+    bt = torch.zeros(C, device=dev, dtype=bf)
+    res, gt = torch.randn(B, S_TXT, C, device=dev, dtype=bf), torch.randn(B, C, device=dev, dtype=bf)
+    ot = torch.empty_like(res)
+    fl = 2.0 * B * S_TXT * C * MLP_RATIO * C
+    for engine, label in (("handwritten", "gemm_text_mlp_down(stream-K, hand-written)"),
+                          ("library", "gemm_text_mlp_down(hipBLASLt, one launch per batch row)")):
+        kernels.set_linear_engine(engine)
+        try:
+            ms = _time_rot(torch, [lambda w=w: kernels.linear(xt, w, bt, residual=res, gate=gt, out=ot) for w in wts])
+            out[label] = {"ms": ms, "TFLOP/s": fl / ms / 1e9, "frac_mfma": fl / ms / 1e9 / PEAK_MFMA_BF16_TFLOPS}
+        finally:
+            kernels.set_linear_engine("auto")
     return out
 
 
