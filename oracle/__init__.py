@@ -22,6 +22,14 @@ Parity status of arithmetic that lives in third-party wheels absent from the ref
   * Flux: ``AdaLayerNormZero`` / ``AdaLayerNormZeroSingle`` chunk orders, the combined
     timestep/guidance/pooled-text embedding, ``get_1d_rotary_pos_embed``; Wan: ``FP32LayerNorm``,
     ``PixArtAlphaTextProjection`` (diffusers>=0.36.0; see ``oracle/flux.py``, ``oracle/wan.py``).
+The reference tree itself restates three of these conventions in code of other models, which is what the
+oracle's choice is checked against (``tests/test_oracle_heads.py``):
+  * vllm_omni/model_executor/models/qwen3_tts/modeling_qwen3_tts.py:584-598 (``Qwen3TTSRMSNorm``):
+    fp32 normalise, cast to the input dtype, THEN multiply by the weight — the cast order of ``rms_norm_head``;
+  * .../qwen3_tts/tokenizer_25hz/modeling_qwen3_tts_tokenizer_v1.py:473-488 (``AdaLayerNormZero``):
+    chunk(6) = shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp, LN(x)(1 + scale_msa) + shift_msa;
+  * same file :492-507 (``AdaLayerNormZero_Final``): chunk(2) = scale, shift, LN(x)(1 + scale) + shift — the
+    order of ``ada_layer_norm_continuous``.
 Everything else (attention, interleaved/NeoX rotary, AdaLayerNorm, gated residual, rel-L1, TeaCache
 decision logic, Qwen rope tables, block wiring, CFG combine) follows code present in the reference.
 """

@@ -16,7 +16,8 @@ def rms_norm_head(x: torch.Tensor, weight: torch.Tensor | None, eps: float = 1e-
     """Per-last-axis RMSNorm in vLLM's order: fp32 normalise, cast to x.dtype, then multiply by weight.
 
     Call sites: models/qwen_image/qwen_image_transformer.py:505-506, 543-544, 588-591 (third-party
-    vllm RMSNorm; cast order adopted from upstream — parity unpinned at that boundary).
+    vllm RMSNorm; cast order adopted from upstream — parity unpinned at that boundary; the same order is
+    written out in the reference tree at model_executor/models/qwen3_tts/modeling_qwen3_tts.py:590-598).
     """
     xf = x.float()
     var = xf.pow(2).mean(dim=-1, keepdim=True)
@@ -110,7 +111,8 @@ def ada_layer_norm_continuous(x: torch.Tensor, cond: torch.Tensor, weight: torch
                               bias: torch.Tensor | None, eps: float = 1e-6) -> torch.Tensor:
     """diffusers AdaLayerNormContinuous(elementwise_affine=False): emb = Linear(SiLU(cond));
     scale, shift = emb.chunk(2); LN(x) * (1 + scale) + shift. Call site
-    models/qwen_image/qwen_image_transformer.py:936, 1065 (third-party; chunk order from upstream)."""
+    models/qwen_image/qwen_image_transformer.py:936, 1065 (third-party; chunk order from upstream, written out
+    in the reference tree at model_executor/models/qwen3_tts/tokenizer_25hz/modeling_qwen3_tts_tokenizer_v1.py:492-507)."""
     emb = F.linear(F.silu(cond).to(x.dtype), weight, bias)
     scale, shift = emb.chunk(2, dim=1)
     normed = F.layer_norm(x, (x.shape[-1],), None, None, eps)

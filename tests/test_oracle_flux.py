@@ -138,3 +138,37 @@ def test_split_projection_equals_projection_of_concatenation():
     want = torch.nn.functional.linear(torch.cat([a, m], dim=-1), W, b)
     got = torch.nn.functional.linear(m, W[:, 16:], b) + a @ W[:, :16].t()
     torch.testing.assert_close(got, want, atol=1e-12, rtol=0)
+
+
+def test_shift_and_scale_chunks_sit_where_the_reference_tree_writes_them():
+    """The remaining four of AdaLayerNormZero's six chunks. The reference tree writes the layer out at
+    model_executor/models/qwen3_tts/tokenizer_25hz/modeling_qwen3_tts_tokenizer_v1.py:473-488:
+    chunk(6) = shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp with
+    x = LN(x) * (1 + scale_msa) + shift_msa. Bias-only modulation, one chunk at a time:
+    chunk 0 must SHIFT the attention input (seen in the TeaCache decision tensor), chunk 1 must SCALE it;
+    with gate_mlp open, chunk 3 must shift and chunk 4 scale the feed-forward input."""
+    cfg, w, lat, txt, pooled, t, gd, img_ids, txt_ids = _setup(seed=6)
+    C = cfg.dim
+    img, enc, temb = ofx.stem(w, cfg, lat, txt, pooled, t, gd)
+    cos, sin = ofx.flux_pos_embed(cfg, torch.cat((txt_ids, img_ids), dim=0))
+    ln = torch.nn.functional.layer_norm(img, (C,), eps=1e-6)
+    val = torch.linspace(0.25, 0.75, C, dtype=img.dtype)
+
+    def weights(chunks: dict):
+        ww = dict(w)
+        for name in ("norm1", "norm1_context"):
+            ww[f"transformer_blocks.0.{name}.linear.weight"] = torch.zeros(6 * C, C, dtype=img.dtype)
+            b = torch.zeros(6 * C, dtype=img.dtype)
+            if name == "norm1":
+                for ch, v in chunks.items():
+                    b[ch * C:(ch + 1) * C] = v
+            ww[f"transformer_blocks.0.{name}.linear.bias"] = b
+        return ww
+
+    torch.testing.assert_close(ofx.modulated_input(weights({0: val}), cfg, img, temb), ln + val, atol=1e-12, rtol=0)
+    torch.testing.assert_close(ofx.modulated_input(weights({1: val}), cfg, img, temb), ln * (1 + val), atol=1e-12, rtol=0)
+    ff = lambda x: ofx.feed_forward(w, "transformer_blocks.0.ff.", x)  # noqa: E731
+    _, h = ofx.dual_block_forward(weights({5: 1.0, 3: val}), 0, cfg, img, enc, temb, cos, sin)
+    torch.testing.assert_close(h, img + ff(ln + val), atol=1e-10, rtol=0)
+    _, h = ofx.dual_block_forward(weights({5: 1.0, 4: val}), 0, cfg, img, enc, temb, cos, sin)
+    torch.testing.assert_close(h, img + ff(ln * (1 + val)), atol=1e-10, rtol=0)

@@ -287,3 +287,20 @@ def test_wan_head_shift_then_scale_of_table_plus_temb():
     # per-token temb [B,S,C] with every token equal reduces to the per-batch form
     torch.testing.assert_close(ow.head(w, cfg, x, temb[:, None].expand(B, S, C).contiguous(), grid, B),
                                ow.head(w, cfg, x, temb, grid, B), rtol=1e-12, atol=1e-12)
+
+
+def test_rms_norm_head_cast_order_is_the_one_the_reference_tree_writes_out():
+    """vLLM's RMSNorm is absent from the reference tree, but the tree writes the same layer out for another
+    model (model_executor/models/qwen3_tts/modeling_qwen3_tts.py:590-598): normalise in float32, cast to the
+    input dtype, THEN multiply by the weight. Wan's DistributedRMSNorm (wan2_2_transformer.py:70-89) multiplies
+    in float32 and casts last; on bf16 inputs the two orders round differently, and the per-head norm must be
+    the first, the whole-row norm the second."""
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(4, 7, 128, generator=g).to(torch.bfloat16)
+    w = (1 + 0.3 * torch.randn(128, generator=g)).to(torch.bfloat16)
+    normed = x.float() * torch.rsqrt(x.float().pow(2).mean(-1, keepdim=True) + 1e-6)
+    cast_then_weight = w * normed.to(torch.bfloat16)
+    weight_then_cast = (normed * w.float()).to(torch.bfloat16)
+    assert not torch.equal(cast_then_weight, weight_then_cast), "the input does not tell the two orders apart"
+    assert torch.equal(ops.rms_norm_head(x, w), cast_then_weight)
+    assert torch.equal(ops.rms_norm_row_fp32(x, w.float()).to(torch.bfloat16), weight_then_cast)
