@@ -5,7 +5,7 @@ CFG combine and the Euler update, on synthetic inputs already resident in HBM. P
 steps/s, the attention kernel's live-measured roofline fraction (bf16 MFMA), per-kernel GB/s and
 TFLOP/s for the other kernels on the path, and the CPU oracle timed on the host cores.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--blocks N] [--no-cpu] [--no-kernels]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--blocks N] [--no-cpu] [--no-kernels] [--no-in-step] [--no-teacache]
   python bench.py --workload flux|wan [--steps K] [--warmup W]     (the other block families, same protocol)
   python bench.py --workload flux --teacache 0.25                  (adds the 28-step TeaCache trajectory: skip rate, steps/s)
 """
@@ -92,6 +92,91 @@ class AttnTimer:
         top = max(self.flops)
         ms = [s.elapsed_time(e) for (s, e), f in zip(self.pairs, self.flops) if f == top]
         return sum(ms) / len(ms), top, len(ms)
+
+
+class StepKernelTimer:
+    """HIP-event brackets around the hand-written kernels and the GEMMs of whole denoise steps run AFTER the timed
+    region (same process, chip in the state the timed steps left it in): what each kernel achieves on the data
+    the step hands it, as opposed to the rotating-buffer microbenchmarks of ``kernel_rooflines``. The brackets
+    cost a few microseconds each, which is why they stay out of the timed steps."""
+
+    def __init__(self, torch, kernels):
+        self.torch, self.kernels = torch, kernels
+        self.records = {}   # label -> [events..., work, unit]
+        self.saved = []
+
+    def _bracket(self, label, work, unit, fn, a, kw):
+        s, e = _events(self.torch)
+        s.record()
+        out = fn(*a, **kw)
+        e.record()
+        rec = self.records.setdefault(label, {"pairs": [], "work": work, "unit": unit})
+        rec["pairs"].append((s, e))
+        return out
+
+    def __enter__(self):
+        k, F = self.kernels, self.torch.nn.functional
+        esz = lambda t: t.element_size()  # noqa: E731
+
+        def adaln_pair(first, second, **kw):
+            byt = sum(2 * p[0].numel() * esz(p[0]) for p in (first, second))
+            return self._bracket("adaln_modulate_pair(img+txt)", byt, "B", orig["adaln_modulate_pair"], (first, second), kw)
+
+        def qknorm_pair(first, second, q_out, k_out, v_out, **kw):
+            byt = sum(2 * (p[0].numel() + (p[1].numel() if p[1] is not None else 0) +
+                           (p[2].numel() if p[2] is not None else 0)) * esz(p[0]) for p in (first, second))
+            return self._bracket("qknorm_rope_pair(img+txt)", byt, "B", orig["qknorm_rope_pair"],
+                                 (first, second, q_out, k_out, v_out), kw)
+
+        def linear(x, weight, bias=None, **kw):
+            if kw.get("plan_only") or kw.get("tune_iters"):
+                return orig["linear"](x, weight, bias, **kw)
+            M, (N, K) = x.numel() // x.shape[-1], weight.shape
+            plan_kw = {a: b for a, b in kw.items() if a != "out"}
+            own = orig["linear"](x, weight, bias, plan_only=True, **plan_kw)[0]
+            tail = "gelu" if kw.get("activation") else ("gated_residual" if kw.get("residual") is not None else "bias")
+            label = f"linear {M}x{N}x{K} {tail} [{'hand-written' if own else 'hipBLASLt'}]"
+            return self._bracket(label, 2.0 * M * N * K, "FLOP", orig["linear"], (x, weight, bias), kw)
+
+        def f_linear(x, weight, bias=None):
+            M, (N, K) = x.numel() // x.shape[-1], weight.shape
+            if M * N * K < 1 << 30:
+                return orig["F.linear"](x, weight, bias)
+            return self._bracket(f"torch linear {M}x{N}x{K} [hipBLASLt]", 2.0 * M * N * K, "FLOP", orig["F.linear"],
+                                 (x, weight, bias), {})
+
+        def attn(*a, **kw):
+            q, kk = a[0], a[1]
+            fl = 4.0 * q.shape[0] * q.shape[2] * q.shape[1] * kk.shape[1] * q.shape[3]
+            return self._bracket(f"attn_fwd B={q.shape[0]} S={q.shape[1]}x{kk.shape[1]} {q.shape[2]}x{q.shape[3]}", fl, "FLOP",
+                                 orig["attn_fwd"], a, kw)
+
+        orig = {"adaln_modulate_pair": k.adaln_modulate_pair, "qknorm_rope_pair": k.qknorm_rope_pair,
+                "linear": k.linear, "attn_fwd": k.attn_fwd, "F.linear": F.linear}
+        self.saved = [(k, "adaln_modulate_pair", k.adaln_modulate_pair), (k, "qknorm_rope_pair", k.qknorm_rope_pair),
+                      (k, "linear", k.linear), (k, "attn_fwd", k.attn_fwd), (F, "linear", F.linear)]
+        k.adaln_modulate_pair, k.qknorm_rope_pair, k.linear, k.attn_fwd, F.linear = adaln_pair, qknorm_pair, linear, attn, f_linear
+        return self
+
+    def __exit__(self, *exc):
+        for mod, name, fn in self.saved:
+            setattr(mod, name, fn)
+
+    def report(self, steps):
+        out = {}
+        for label, rec in self.records.items():
+            us = [s.elapsed_time(e) * 1e3 for s, e in rec["pairs"]]
+            mean = sum(us) / len(us)
+            row = {"calls_per_step": len(us) / steps, "avg_us": mean, "ms_per_step": sum(us) / steps / 1e3}
+            if rec["unit"] == "B":
+                row["GB/s"] = rec["work"] / mean / 1e3
+                row["frac_hbm"] = row["GB/s"] / PEAK_HBM_GBS
+                row["algorithmic_bytes"] = rec["work"]
+            else:
+                row["TFLOP/s"] = rec["work"] / mean / 1e6
+                row["frac_mfma"] = row["TFLOP/s"] / PEAK_MFMA_BF16_TFLOPS
+            out[label] = row
+        return dict(sorted(out.items(), key=lambda kv: -kv[1]["ms_per_step"]))
 
 
 def max_engine_clock_mhz():
@@ -282,7 +367,7 @@ def run_secondary(torch, kernels, args):
     }))
 
 
-def teacache_trajectory(torch, model, step, thresh, plain_steps_per_s, steps=28):
+def teacache_trajectory(torch, model, step, thresh, plain_steps_per_s, steps=28, first_trajectory_decisions=None):
     """BASELINE.json configs[4]: the 28-step trajectory with the TeaCache hook on (relative-L1 threshold `thresh`
     on the modulated first-block input, the reference's 4th-order polynomial for this model): one untimed
     trajectory, then the same trajectory timed. Steps/s counts every denoise step, skipped or computed."""
@@ -297,6 +382,8 @@ def teacache_trajectory(torch, model, step, thresh, plain_steps_per_s, steps=28)
         backend.refresh(Pipe, steps)
         step.trajectory(steps)
         torch.cuda.synchronize()
+        if first_trajectory_decisions is not None:
+            first_trajectory_decisions.extend(dict(d) for d in TeaCacheBackend.hook_of(Pipe).decisions)
         backend.refresh(Pipe, steps)
         t0 = time.perf_counter()
         lat = step.trajectory(steps)
@@ -312,6 +399,52 @@ def teacache_trajectory(torch, model, step, thresh, plain_steps_per_s, steps=28)
             "speedup": steps / elapsed / plain_steps_per_s, "compute_pattern": "".join("C" if c else "s" for c in decisions),
             "min_distance_to_threshold": min(margins) if margins else None,
             "data": "synthetic latents, random weights: the skip pattern is this trajectory's, not a trained model's"}
+
+
+def teacache_flux(torch, kernels):
+    """BASELINE.json configs[4] inside the default run: the Flux-shape model (19 dual + 38 single blocks, 512 text +
+    4096 image tokens, bf16), 28 Euler steps under the TeaCache hook at threshold 0.25, next to the uncached rate.
+    During the untimed first trajectory the operands of the first three relative-L1 reductions are copied to the
+    host, and the scalar the hook thresholded is checked, bit for bit, against the reference's own expression
+    (vllm_omni/diffusion/cache/teacache/hook.py:214-221) evaluated by torch on the host in the tensors' dtype,
+    outside every timed region."""
+    model, step, lat0, name, _gemm, valid = flux_workload(torch)
+    captured = []
+    orig = kernels.rel_l1_sums
+
+    def capturing(cur, prev, **kw):
+        if len(captured) < 3:
+            captured.append((cur.detach().cpu(), prev.detach().cpu()))
+        return orig(cur, prev, **kw)
+
+    with torch.inference_mode():
+        lat = lat0
+        for i in range(2):
+            lat = step(i, lat)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        n_plain = 4
+        for i in range(2, 2 + n_plain):
+            lat = step(i, lat)
+        torch.cuda.synchronize()
+        plain = n_plain / (time.perf_counter() - t0)
+    kernels.rel_l1_sums = capturing
+    try:
+        out = teacache_trajectory(torch, model, step, 0.25, plain, first_trajectory_decisions=(first := []))
+    finally:
+        kernels.rel_l1_sums = orig
+    rels = [d["rel"] for d in first if d["rel"] is not None][:len(captured)]
+    checks = []
+    for (cur, prev), got in zip(captured, rels):
+        want = ((cur - prev).abs().mean() / (prev.abs().mean() + 1e-8)).item()
+        checks.append({"hook": got, "host": want, "equal": got == want})
+    assert checks and all(c["equal"] for c in checks), f"relative-L1 scalars differ from the host expression's: {checks}"
+    out["workload"] = name
+    out["valid"] = valid
+    out["rel_l1_checked_against_host_expression"] = {"decisions": len(checks), "bit_identical": True,
+                                                     "values": [c["hook"] for c in checks]}
+    del model
+    return out
 
 
 def _time_rot(torch, fns, iters=40, warmup=4):
@@ -415,12 +548,22 @@ def kernel_rooflines(torch):
     fl = 2.0 * B * S_TXT * C * MLP_RATIO * C
     for engine, label in (("handwritten", "gemm_text_mlp_down(stream-K, hand-written)"),
                           ("library", "gemm_text_mlp_down(hipBLASLt, one launch per batch row)")):
-        kernels.set_linear_engine(engine)
-        try:
-            ms = _time_rot(torch, [lambda w=w: kernels.linear(xt, w, bt, residual=res, gate=gt, out=ot) for w in wts])
-            out[label] = {"ms": ms, "TFLOP/s": fl / ms / 1e9, "frac_mfma": fl / ms / 1e9 / PEAK_MFMA_BF16_TFLOPS}
-        finally:
-            kernels.set_linear_engine("auto")
+        ms = _time_rot(torch, [lambda w=w: kernels.linear(xt, w, bt, residual=res, gate=gt, out=ot, engine=engine)
+                               for w in wts])
+        out[label] = {"ms": ms, "TFLOP/s": fl / ms / 1e9, "frac_mfma": fl / ms / 1e9 / PEAK_MFMA_BF16_TFLOPS}
+    del xt, wts, res, ot
+    # the image stream's MLP up-projection with its GELU epilogue, hand-written tile kernel against the library,
+    # weights rotating (four 75 MB weights and the 201 MB output exceed the last-level cache)
+    xm = torch.randn(B * S_IMG, C, device=dev, dtype=bf)
+    wms = [torch.randn(MLP_RATIO * C, C, device=dev, dtype=bf) * 0.02 for _ in range(4)]
+    bm = torch.zeros(MLP_RATIO * C, device=dev, dtype=bf)
+    om = torch.empty(B * S_IMG, MLP_RATIO * C, device=dev, dtype=bf)
+    fl = 2.0 * B * S_IMG * C * MLP_RATIO * C
+    for engine, label in (("handwritten", "gemm_img_mlp_up_gelu(tile kernel, hand-written)"),
+                          ("library", "gemm_img_mlp_up_gelu(hipBLASLt)")):
+        ms = _time_rot(torch, [lambda w=w: kernels.linear(xm, w, bm, activation="gelu_tanh", out=om, engine=engine)
+                               for w in wms], iters=16)
+        out[label] = {"ms": ms, "TFLOP/s": fl / ms / 1e9, "frac_mfma": fl / ms / 1e9 / PEAK_MFMA_BF16_TFLOPS}
     return out
 
 
@@ -477,20 +620,25 @@ def mfma_ceiling(torch):
 
     from vllm_omni_amd import _lib
 
-    lib = _lib.load()
+    path = _lib.LIB_PATH.with_name("libomni_dit_probe.so")   # a measurement aid, kept out of the product library
+    if not path.exists():
+        return {"error": f"{path.name} not built"}
+    lib = C.CDLL(os.fspath(path))
+    lib.odit_probe_mfma.restype = C.c_int
+    lib.odit_probe_mfma.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double), C.c_void_p]
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     sink = torch.empty(cus * 512, device="cuda", dtype=torch.float32)
     st = torch.cuda.current_stream().cuda_stream
     out = {}
     for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
         flop = C.c_double(0.0)
-        _lib.check(lib.odit_probe_mfma(rnd, 2000, cus, sink.data_ptr(), C.byref(flop), st), "odit_probe_mfma")
+        assert lib.odit_probe_mfma(rnd, 2000, cus, sink.data_ptr(), C.byref(flop), st) == 0
         torch.cuda.synchronize()
         best = 0.0
         for _ in range(3):
             a, b = _events(torch)
             a.record()
-            _lib.check(lib.odit_probe_mfma(rnd, 20000, cus, sink.data_ptr(), C.byref(flop), st), "odit_probe_mfma")
+            assert lib.odit_probe_mfma(rnd, 20000, cus, sink.data_ptr(), C.byref(flop), st) == 0
             b.record()
             torch.cuda.synchronize()
             best = max(best, flop.value / a.elapsed_time(b) / 1e9)
@@ -566,6 +714,10 @@ def main():
                          "relative-L1 threshold and report skip rate and steps/s")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
+    ap.add_argument("--no-in-step", action="store_true",
+                    help="skip the two extra, untimed steps whose kernels are bracketed one by one (kernels_in_step)")
+    ap.add_argument("--no-teacache", action="store_true",
+                    help="skip the Flux-shape TeaCache trajectory (BASELINE.json configs[4]) that follows the headline measurement")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build runs the DiT step on ONE GPU (CFG branches are batched on it; "
@@ -636,6 +788,15 @@ def main():
         attn_ms = timer.mean_ms()
         n_attn = len(timer.pairs)
     assert bool(torch.isfinite(lat.float()).all()), "non-finite latents"
+    in_step = None
+    if not args.no_in_step:
+        # two more steps, outside the timed region, every hand-written kernel and GEMM between its own events
+        n_extra = 2
+        with torch.inference_mode(), StepKernelTimer(torch, kernels) as kt:
+            for i in range(n_extra):
+                lat = step(i, lat)
+            torch.cuda.synchronize()
+        in_step = kt.report(n_extra)
     ms_per_step = elapsed * 1e3 / args.steps
     S = S_IMG + S_TXT
     attn_flop = 4.0 * B * HEADS * S * S * HEAD_DIM
@@ -683,6 +844,11 @@ def main():
     gemm_flop = 2.0 * (B * S_IMG + B * S_TXT) * (3 * C * C + C * C + 2 * MLP_RATIO * C * C) * args.blocks
     result["step_flop"] = {"gemm": gemm_flop, "attention": attn_flop * args.blocks,
                            "achieved_TFLOP/s": (gemm_flop + attn_flop * args.blocks) / elapsed * args.steps / 1e12}
+    if in_step is not None:
+        result["kernels_in_step"] = {
+            "what": "per-kernel averages over two extra steps run right after the timed region, each call between its "
+                    "own HIP events (not part of `value`): the rate on the data the step hands the kernel",
+            "kernels": in_step}
     if not args.no_kernels:
         with torch.inference_mode():
             result["kernels"] = kernel_rooflines(torch)
@@ -700,6 +866,9 @@ def main():
     }
     del model
     torch.cuda.empty_cache()
+    if not args.no_teacache and args.blocks == LAYERS:
+        result["teacache_flux"] = teacache_flux(torch, kernels)
+        torch.cuda.empty_cache()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch)
         result["gpu_over_cpu"] = result["value"] / result["cpu_baseline"]["value"]

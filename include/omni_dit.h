@@ -13,9 +13,10 @@
  *   - Return value: 0 on success, a negative ODIT_E* code on failure; odit_last_error() then returns a
  *     thread-local, NUL-terminated description. Argument errors are detected on the host BEFORE any
  *     launch, so a failing call enqueues nothing.
- *   - Re-entrant; the only state kept between calls is thread-local: the error string, and in
- *     odit_linear the library handle with the matmul descriptors of the problems seen so far
- *     (plus a process-wide, write-once table of each device's compute-unit count).
+ *   - Re-entrant; the state kept between calls is thread-local (the error string, and in odit_linear the
+ *     library handle with the matmul descriptors of the problems seen so far) or process-wide behind a
+ *     lock or an atomic (each device's compute-unit count, the record of which engine a tuning call found
+ *     faster for a problem, the launch counter that ticket words in caller scratch are stamped with).
  *
  * The reference (Flink-ddd/vllm-omni) is pure Python and has no FFI of its own for this path; each
  * entry point below replaces the third-party kernel call(s) made at the cited reference lines.
@@ -30,7 +31,7 @@
 extern "C" {
 #endif
 
-#define ODIT_VERSION 102 /* major*10000 + minor*100 + patch */
+#define ODIT_VERSION 200 /* major*10000 + minor*100 + patch */
 
 enum odit_dtype { ODIT_BF16 = 0, ODIT_F16 = 1, ODIT_F32 = 2 };
 
@@ -237,12 +238,15 @@ int odit_gated_residual(const void* h, const void* y, const void* gate, const fl
  *
  * cur, prev: [B, n] with row strides cur_stride / prev_stride (elements); n % 8 == 0 not required.
  * sums: double [B,2] on the device.
- * workspace: device scratch of at least odit_rel_l1_workspace_bytes(B, n) bytes, 16-byte aligned. It
- *   holds one ticket counter per row and the partials. THE COUNTERS MUST BE ZERO ON ENTRY: zero the
- *   workspace once after allocating it (hipMemsetAsync, or a fill kernel under graph capture). Every call
- *   hands the counters back at zero, so one zeroed workspace serves any number of later calls, of any
- *   (B, n) it is large enough for. Calls that share a workspace must not overlap (same stream, or ordered
- *   by events).
+ * workspace: device scratch of at least odit_rel_l1_workspace_bytes(B, n) bytes, 16-byte aligned: a
+ *   region of fixed size (512 KiB, whatever B is) with one 64-bit ticket word per row, then the partials.
+ *   ZERO-FILL IT ONCE after allocating it (hipMemsetAsync, or a fill kernel under graph capture) and do
+ *   not write it afterwards. A ticket word is (launch number << 16 | tickets drawn); every launch first
+ *   raises its rows' words to its own number, which is larger than any earlier launch's, and the last
+ *   workgroup of a row puts the word back to zero. One zeroed workspace therefore serves any number of
+ *   later calls of any (B, n) it is large enough for, also after a launch that did not finish (its stale
+ *   words are overridden), and a call recorded into a HIP graph can be replayed. Calls that share a
+ *   workspace must not overlap (same stream, or ordered by events).
  */
 size_t odit_rel_l1_workspace_bytes(int B, int64_t n);
 int odit_rel_l1(const void* cur, const void* prev, double* sums, void* workspace,
@@ -251,17 +255,24 @@ int odit_rel_l1(const void* cur, const void* prev, double* sums, void* workspace
 
 /* odit_rel_l1 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same arguments and bit-identical
- * sums, without the workspace: the ticket counters and partials live in an array built into the library's
- * device image, 2304 bytes per GPU the library is used on, held until the process ends. It calls no
+ * sums, without the workspace: the ticket words and partials live in an array built into the library's
+ * device image, 2560 bytes per GPU the library is used on, held until the process ends. It calls no
  * allocating routine. Limit: B <= 64 rows (any n); more returns ODIT_EWORKSPACE and enqueues nothing.
- * Two launches: a fill kernel puts the counters to zero (a kernel, not a memset, so the call can be captured),
- * then the reduction. Every call on a GPU shares that GPU's array: calls that may overlap on one GPU
+ * Two launches: a fill kernel puts the ticket words to zero (a kernel, not a memset, so the call can be
+ * captured; whatever an earlier call left in the array, also one that never finished, is gone), then the reduction. Every call on a GPU shares that GPU's array: calls that may overlap on one GPU
  * (different streams without ordering, or several host threads) race and must be serialised by the caller.
  * The first call on each device looks the array's address up (hipGetSymbolAddress); make that call outside
  * graph capture.
  */
 int odit_rel_l1_static(const void* cur, const void* prev, double* sums, int B, int64_t n, int64_t cur_stride,
                        int64_t prev_stride, int dtype, unsigned flags, void* stream);
+
+/* Device address of that built-in array on the current device and its size (*bytes, may be NULL); NULL with
+ * an error string when it cannot be looked up. No counterpart in the reference. For diagnostics and tests (a
+ * test dirties the array to check that odit_rel_l1_static does not depend on what it holds); no caller of
+ * odit_rel_l1_static needs it.
+ */
+void* odit_rel_l1_static_scratch(size_t* bytes);
 
 /* ---------------------------------------------------------------------------------------------
  * Pointwise helpers on the block path.
@@ -288,12 +299,13 @@ int odit_silu(const void* x, void* out, int64_t n, int dtype, void* stream);
  *                                                          flux_transformer.py:30-45, wan2_2_transformer.py:92-109
  *   RowParallelLinear followed by `h + gate * y`           qwen_image_transformer.py:794-795, 801, 806,
  *                                                          flux_transformer.py:288-309, wan2_2_transformer.py:661, 673
- * Two engines. Problems with many rows run on hipBLASLt's MFMA kernels (a plain dense GEMM), set up so
- * that bias, activation, gate and residual ride in that kernel's epilogue. bf16 problems with
- * 64 <= M <= 1024 rows, K a multiple of 64, N a multiple of 8 and 16-byte aligned rows can also run on a
- * hand-written stream-K MFMA kernel (csrc/gemm_bf16.hip) that keeps all CUs busy on few output tiles and
- * takes one gate vector per group of rows in a single launch (odit_linear_rows); it is used where a
- * tuning call found it faster or, untuned, where K >= 2 N.
+ * Engines. hipBLASLt's MFMA kernels (a plain dense GEMM), set up so that bias, activation, gate and
+ * residual ride in that kernel's epilogue, and two hand-written bf16 MFMA kernels (K a multiple of 64, N a
+ * multiple of 8, 16-byte aligned rows): a stream-K kernel for 64 <= M <= 1024 rows (csrc/gemm_bf16.hip) that
+ * keeps all CUs busy on few output tiles, and a tile kernel for more rows (csrc/gemm_bf16_tile.hip: 256 x 256
+ * or 256 x 192 output tiles, one per workgroup). Both take one gate vector per group of rows in a single
+ * launch (odit_linear_rows). A hand-written kernel runs where a tuning call found it faster or, untuned,
+ * where its default rule says so (stream-K: K >= 2 N); the `flags` of odit_linear_rows can force either side.
  *
  * x [M,K] (row stride ldx), W [N,K] (row stride ldw: torch's nn.Linear weight, or a column range of
  * one), bias [N] or NULL, out [M,N] (row stride ldo). Gated form: residual [M,N] (row stride ldr; may be
@@ -302,17 +314,18 @@ int odit_silu(const void* x, void* out, int64_t n, int dtype, void* stream);
  * workspace: device scratch, 256-byte aligned, for the library's split-K kernels, in the gated form two
  * float[N] vectors, and the hand-written kernel's tile counters and partial tiles;
  * odit_linear_workspace_bytes() is a size that suits every kernel. A workspace of that size must be
- * ZERO-FILLED ONCE before its first use and not written by the caller afterwards (the first 16 KB hold
- * the tile counters, which every call leaves at zero); calls that share a workspace must not overlap
- * in time (one workspace per stream). A smaller workspace goes to the library alone and rules the
+ * ZERO-FILLED ONCE before its first use and not written by the caller afterwards (the first 32 KB hold
+ * the stream-K kernel's ticket words, stamped with the launch number like those of odit_rel_l1: every call
+ * leaves them at zero, and what a launch that did not finish left there is overridden by the next one);
+ * calls that share a workspace must not overlap in time (one workspace per stream). A smaller workspace goes to the library alone and rules the
  * hand-written kernel out; NULL restricts the choice to library kernels that need none (not allowed
  * for the gated form).
  *
  * odit_linear_tune launches every kernel the library offers for the problem, and the hand-written
  * kernel where it takes the problem, on the given buffers
- * (`out` is overwritten; this call synchronises with the stream), keeps the fastest for later
- * odit_linear calls with the same shape, strides, epilogue and dtype FROM THE SAME HOST THREAD, and
- * reports its time. `flush` (optional device buffer, ideally larger than the last-level cache) is
+ * (`out` is overwritten; this call synchronises with the stream), keeps the fastest library kernel for later
+ * odit_linear calls with the same shape, strides, epilogue and dtype FROM THE SAME HOST THREAD, records
+ * for the whole process whether the hand-written kernel beat it, and reports the winner's time. `flush` (optional device buffer, ideally larger than the last-level cache) is
  * overwritten before every timed launch so that each one starts from cold caches, as a projection
  * with its own weights does inside a model. Without tuning the library's own first choice is used.
  */
@@ -339,41 +352,33 @@ int odit_linear_tune(const void* x, const void* w, const void* bias, void* out, 
 /* odit_linear with one gate vector per group of rows_per_gate consecutive rows (the rows of one batch
  * row of a [B, S, N] activation): gate vector i, gate_stride elements after vector i - 1, scales rows
  * [i rows_per_gate, (i + 1) rows_per_gate); in the pre-scaled form `bias` is laid out the same way.
- * rows_per_gate = 0 is odit_linear. One launch when the hand-written kernel takes the problem, one
+ * rows_per_gate = 0 is odit_linear. One launch when a hand-written kernel takes the problem, one
  * library launch per group of rows otherwise.
+ * flags: 0 = choose as described above; ODIT_LINEAR_LIBRARY = hipBLASLt whatever the record says;
+ * ODIT_LINEAR_HANDWRITTEN = the hand-written kernel for this row count (ODIT_ENOTSUP when it does not take
+ * the problem). Per call: no process-wide switch exists.
  */
+#define ODIT_LINEAR_LIBRARY 1u
+#define ODIT_LINEAR_HANDWRITTEN 2u
+
 int odit_linear_rows(const void* x, const void* w, const void* bias, void* out, const void* residual,
                      const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int64_t ldr,
                      int epilogue, int gate_dtype, int dtype, int rows_per_gate, int64_t gate_stride,
-                     void* workspace, size_t workspace_bytes, void* stream);
+                     unsigned flags, void* workspace, size_t workspace_bytes, void* stream);
 
 /* What odit_linear_rows would do with these arguments, without launching anything: *handwritten = 1 when
- * the hand-written kernel would run, *launches = kernel launches the call would make. */
+ * a hand-written kernel would run, *launches = kernel launches the call would make. */
 int odit_linear_rows_plan(const void* x, const void* w, const void* bias, void* out, const void* residual,
                           const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int64_t ldr,
                           int epilogue, int gate_dtype, int dtype, int rows_per_gate, int64_t gate_stride,
-                          void* workspace, size_t workspace_bytes, int* handwritten, int* launches);
+                          unsigned flags, void* workspace, size_t workspace_bytes, int* handwritten, int* launches);
 
+/* odit_linear_tune for the per-row-group form; *handwritten (may be NULL) = 1 when the hand-written kernel won. */
 int odit_linear_rows_tune(const void* x, const void* w, const void* bias, void* out, const void* residual,
                           const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int64_t ldr,
                           int epilogue, int gate_dtype, int dtype, int rows_per_gate, int64_t gate_stride,
                           void* workspace, size_t workspace_bytes, void* stream, int iters, void* flush,
-                          size_t flush_bytes, float* best_us);
-
-/* Which kernel odit_linear / odit_linear_rows run (process-wide; for measurements and tests):
- * 0 = the hand-written kernel where it takes the problem and the library elsewhere (the default),
- * 1 = the library always, 2 = the hand-written kernel always (ODIT_ENOTSUP for problems it does not take).
- */
-int odit_linear_set_engine(int engine);
-
-/* ---------------------------------------------------------------------------------------------
- * Roofline calibration (no counterpart in the reference): launches `workgroups` workgroups of 8
- * wavefronts that issue nothing but v_mfma_f32_32x32x16_bf16 (iters x 8 per wavefront) on register
- * operands holding constant (random_operands = 0) or pseudo-random data, writes one float per thread to
- * `sink` (workgroups * 512 floats) and returns the flop count of the launch in *flop. Timed by the
- * caller with events on `stream`: the sustained matrix rate of the device for that kind of data.
- */
-int odit_probe_mfma(int random_operands, int iters, int workgroups, float* sink, double* flop, void* stream);
+                          size_t flush_bytes, float* best_us, int* handwritten);
 
 #ifdef __cplusplus
 }

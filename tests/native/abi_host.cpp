@@ -291,19 +291,18 @@ static int check_linear_rows(hipStream_t st) {
   HIP_OK(hipMemcpy(d_r.p, res.data(), res.size() * 2, hipMemcpyHostToDevice));
   HIP_OK(hipMemcpy(d_g.p, gate.data(), gate.size() * 4, hipMemcpyHostToDevice));
   HIP_OK(hipMemcpy(d_b.p, gbias.data(), gbias.size() * 4, hipMemcpyHostToDevice));
-  ODIT_OK_OR_FAIL(odit_linear_set_engine(2));
   int handwritten = 0, launches = 0;
   ODIT_OK_OR_FAIL(odit_linear_rows_plan(d_x.p, d_w.p, d_b.p, d_o.p, d_r.p, d_g.p, M, N, K, K, K, N, N,
-                                        ODIT_EPI_GATED_RESIDUAL_PRE, ODIT_F32, ODIT_BF16, S, N, d_ws.p, ws, &handwritten,
-                                        &launches));
+                                        ODIT_EPI_GATED_RESIDUAL_PRE, ODIT_F32, ODIT_BF16, S, N, ODIT_LINEAR_HANDWRITTEN,
+                                        d_ws.p, ws, &handwritten, &launches));
   if (handwritten != 1 || launches != 1) {
     std::fprintf(stderr, "linear_rows plan: handwritten %d launches %d, want 1 and 1\n", handwritten, launches);
     return 1;
   }
   for (int rep = 0; rep < 2; ++rep)  // twice: the second call finds the counters as the first left them
     ODIT_OK_OR_FAIL(odit_linear_rows(d_x.p, d_w.p, d_b.p, d_o.p, d_r.p, d_g.p, M, N, K, K, K, N, N,
-                                     ODIT_EPI_GATED_RESIDUAL_PRE, ODIT_F32, ODIT_BF16, S, N, d_ws.p, ws, st));
-  ODIT_OK_OR_FAIL(odit_linear_set_engine(0));
+                                     ODIT_EPI_GATED_RESIDUAL_PRE, ODIT_F32, ODIT_BF16, S, N, ODIT_LINEAR_HANDWRITTEN,
+                                     d_ws.p, ws, st));
   HIP_OK(hipStreamSynchronize(st));
   HIP_OK(hipMemcpy(out.data(), d_o.p, out.size() * 2, hipMemcpyDeviceToHost));
   double worst = 0.0;

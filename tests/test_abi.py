@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     for name in _declared_functions():
         assert hasattr(lib, name), name
-    assert lib.odit_version() == 102
+    assert lib.odit_version() == 200
 
 
 def _strides(*v):
@@ -65,7 +65,8 @@ def test_argument_errors_are_caught_before_launch():
                               _strides(256, 64), 2, 4, 1e-6, 1, 0, 0, 0, None)
     assert rc == -1 and b"do not fit" in lib.odit_last_error()
     # workspace too small
-    assert lib.odit_rel_l1_workspace_bytes(2, 1 << 20) == 256 + 2 * 32 * 8  # counters + 32 workgroups per row of 2^20 elements
+    # a ticket word for each of the 65536 rows a call may have, then 32 workgroups per row of 2^20 elements
+    assert lib.odit_rel_l1_workspace_bytes(2, 1 << 20) == 65536 * 8 + 2 * 32 * 8
     rc = lib.odit_rel_l1(p16, p16, p16, p16, 8, 2, 1 << 20, 1 << 20, 1 << 20, 0, 0, None)
     assert rc == -4
     # empty problems succeed without touching the device

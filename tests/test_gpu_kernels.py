@@ -242,6 +242,46 @@ def test_rel_l1_one_workspace_serves_changing_shapes(gpu):
         assert torch.allclose(fresh[i][:, 0], want, rtol=5e-6)
 
 
+def test_rel_l1_workspace_rows_grow_and_stale_ticket_words(gpu):
+    """One workspace through the C ABI: a call with few rows and many workgroups per row (its partials fill the
+    bytes behind the ticket words), then a call with many rows (whose ticket words must not be those bytes), then
+    ticket words left as by a launch that never finished (an older launch number, some tickets drawn): each call
+    equals the same call on a fresh zeroed workspace."""
+    from vllm_omni_amd import _lib
+
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    few = (2, 4096 * 3072)
+    many = (100, 3000)
+    need = max(int(lib.odit_rel_l1_workspace_bytes(*few)), int(lib.odit_rel_l1_workspace_bytes(*many)))
+    ws = torch.zeros(need, dtype=torch.uint8, device=gpu)
+
+    def run(cur, prev, workspace):
+        B, n = cur.shape
+        sums = torch.full((B, 2), -1.0, dtype=torch.float64, device=gpu)
+        rc = lib.odit_rel_l1(cur.data_ptr(), prev.data_ptr(), sums.data_ptr(), workspace.data_ptr(), workspace.numel(),
+                             B, n, n, n, 0, 1, st)
+        assert rc == 0, lib.odit_last_error()
+        return sums
+
+    data = {}
+    for B, n in (few, many):
+        prev = _rand(B, n, seed=B)
+        data[(B, n)] = ((prev.float() * 1.1 + 0.01).bfloat16().to(gpu), prev.to(gpu))
+    fresh = {k: run(*v, torch.zeros(need, dtype=torch.uint8, device=gpu)) for k, v in data.items()}
+    got_few = run(*data[few], ws)
+    got_many = run(*data[many], ws)
+    torch.cuda.synchronize()
+    assert torch.equal(got_few, fresh[few]) and torch.equal(got_many, fresh[many])
+    # stale words: launch number 0 with 1..99 tickets drawn in every row's word
+    words = ws[:8 * 100].view(torch.int64)   # the words of the rows these calls use
+    words.copy_(torch.randint(1, 100, words.shape, device=gpu))
+    assert torch.equal(run(*data[many], ws), fresh[many])
+    assert torch.equal(run(*data[few], ws), fresh[few])
+    torch.cuda.synchronize()
+    assert int(ws[:8 * 100].view(torch.int64).abs().max().item()) == 0   # handed back at zero
+
+
 def test_rel_l1_closed_forms(gpu):
     from vllm_omni_amd import kernels
 

@@ -179,7 +179,7 @@ def handwritten(gpu):
 
 
 def _counters_are_zero(kernels):
-    return all(int(ws[:16384].view(torch.int32).abs().max().item()) == 0 for ws in kernels._LINEAR_SCRATCH.values())
+    return all(int(ws[:32768].view(torch.int32).abs().max().item()) == 0 for ws in kernels._LINEAR_SCRATCH.values())
 
 
 @pytest.mark.parametrize("M,N,K", [
@@ -188,6 +188,7 @@ def _counters_are_zero(kernels):
     (64, 192, 64),       # one tile, one step
     (1024, 200, 4096),   # 8 row tiles, 2 feature tiles, every tile shared by 16 workgroups
     (512, 3072, 3072),   # text-stream output projection of the headline workload
+    (512, 3072, 12288),  # text-stream MLP down-projection of the headline workload: where the kernel runs in the step
 ])
 def test_streamk_gemm_matches_fp64_product(handwritten, gpu, M, N, K):
     x, w, b = _mk(M, N, K, torch.bfloat16, seed=M + N)
@@ -238,12 +239,121 @@ def test_streamk_gemm_refuses_what_it_does_not_take(handwritten, gpu):
     x, w, b = _mk(77, 200, 136, torch.bfloat16)      # K not a multiple of 64
     with pytest.raises(OmniDitKernelError):
         handwritten.linear(x.to(gpu), w.to(gpu), b.to(gpu))
-    x, w, b = _mk(4096, 256, 256, torch.bfloat16)    # too many rows: the library's large tiles win there
+    x, w, b = _mk(4096, 250, 256, torch.bfloat16)    # N not a multiple of 8: neither hand-written kernel
     with pytest.raises(OmniDitKernelError):
         handwritten.linear(x.to(gpu), w.to(gpu), b.to(gpu))
     handwritten.set_linear_engine("auto")
     got = handwritten.linear(x.to(gpu), w.to(gpu), b.to(gpu))
     torch.testing.assert_close(got.double().cpu(), _ref(x, w, b), atol=2e-2, rtol=2e-2)
+
+
+def test_streamk_gemm_headline_problem_with_row_group_gates(handwritten, gpu):
+    """The launch the Qwen step makes once per block: M = 2 x 256 text rows, N = 3072, K = 12288, float32
+    gate and gate * bias rows per batch entry, accumulated onto the residual in place."""
+    B, S, N, K = 2, 256, 3072, 12288
+    x, w, b = _mk(S, N, K, torch.bfloat16, seed=41, lead=(B,))
+    g = torch.Generator().manual_seed(42)
+    h = torch.randn(B, S, N, generator=g).bfloat16()
+    gate = torch.randn(B, N, generator=g)
+    want = h.double() + gate.double()[:, None, :] * _ref(x, w, b)
+    xg, wg, hg, gg = (t.to(gpu) for t in (x, w, h, gate))
+    gb = gg * b.to(gpu).float()
+    assert handwritten.linear(xg, wg, None, residual=hg, gate=gg, gate_bias=gb, prescaled=True, plan_only=True) == (True, 1)
+    got = handwritten.linear(xg, wg, None, residual=hg, gate=gg, gate_bias=gb, prescaled=True)
+    torch.testing.assert_close(got.double().cpu(), want, atol=4e-2, rtol=2e-2)
+    assert _counters_are_zero(handwritten)
+
+
+def test_streamk_gemm_overrides_stale_ticket_words(handwritten, gpu):
+    """Ticket words that an earlier launch left behind (as one that never finished would) carry an older launch
+    number: the next launch raises them to its own and still reduces every tile."""
+    x, w, b = _mk(1024, 200, 4096, torch.bfloat16, seed=43)   # every tile shared by 16 workgroups
+    xg, wg, bg = x.to(gpu), w.to(gpu), b.to(gpu)
+    want = handwritten.linear(xg, wg, bg)
+    torch.cuda.synchronize()
+    ws = handwritten._LINEAR_SCRATCH[(gpu.index or 0, torch.cuda.current_stream().cuda_stream)]
+    words = ws[:16 * 8].view(torch.int64)   # the ticket words of this problem's 8 x 2 output tiles
+    words.copy_(torch.randint(1, 14, words.shape, device=gpu))   # launch number 0, 1..13 tickets drawn
+    got = handwritten.linear(xg, wg, bg)
+    assert torch.equal(got, want)
+    assert _counters_are_zero(handwritten)
+
+
+@pytest.mark.parametrize("B,S", [(3, 96), (2, 160)])
+@pytest.mark.parametrize("engine", ["handwritten", "library"])
+def test_gated_rows_that_straddle_tiles_and_a_ragged_group(gpu, B, S, engine):
+    """Groups of rows whose ends fall inside a 128-row tile, and B * S not a multiple of the tile: the
+    hand-written kernel picks the gate row per output row, the library runs one launch per group."""
+    from vllm_omni_amd import kernels
+
+    N, K = 192, 256
+    x, w, b = _mk(S, N, K, torch.bfloat16, seed=51 + B, lead=(B,))
+    g = torch.Generator().manual_seed(52)
+    h = torch.randn(B, S, N, generator=g).bfloat16()
+    gate = torch.randn(B, N, generator=g).bfloat16()
+    want = h.double() + gate.double()[:, None, :] * _ref(x, w, b)
+    got = kernels.linear(x.to(gpu), w.to(gpu), b.to(gpu), residual=h.to(gpu), gate=gate.to(gpu), engine=engine)
+    torch.testing.assert_close(got.double().cpu(), want, atol=4e-2, rtol=2e-2)
+
+
+# ---------------------------------------------------------------------------- hand-written tile kernel (many rows)
+@pytest.mark.parametrize("M,N,K", [
+    (2048, 512, 256),     # 8 x 2 tiles of 256 x 256, four steps
+    (1280, 384, 64),      # 192-wide tiles, one step
+    (1100, 200, 192),     # ragged last row tile and last feature tile (N a multiple of 8 only), three steps
+    (4096, 768, 3072),    # 16 x 4 tiles of 256 x 192, the headline reduction length
+])
+def test_tile_gemm_matches_fp64_product(handwritten, gpu, M, N, K):
+    x, w, b = _mk(M, N, K, torch.bfloat16, seed=M + N + 1)
+    print(f"tile kernel {M}x{N}x{K}", flush=True)
+    xg, wg, bg = x.to(gpu), w.to(gpu), b.to(gpu)
+    assert handwritten.linear(xg, wg, bg, plan_only=True) == (True, 1)
+    got = handwritten.linear(xg, wg, bg)
+    torch.testing.assert_close(got.double().cpu(), _ref(x, w, b), atol=2e-2, rtol=2e-2)
+    assert torch.equal(got, handwritten.linear(xg, wg, bg))
+    got = handwritten.linear(xg, wg, None)
+    torch.testing.assert_close(got.double().cpu(), _ref(x, w, None), atol=2e-2, rtol=2e-2)
+    got = handwritten.linear(xg, wg, bg, activation="gelu_tanh")
+    torch.testing.assert_close(got.double().cpu(), ops.gelu_tanh(_ref(x, w, b)), atol=2e-2, rtol=2e-2)
+    lib = handwritten.linear(xg, wg, bg, engine="library")
+    torch.testing.assert_close(handwritten.linear(xg, wg, bg).float(), lib.float(), atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("gate_dtype", [torch.bfloat16, torch.float32])
+def test_tile_gemm_gates_per_batch_row_in_one_launch(handwritten, gpu, gate_dtype):
+    B, S, N, K = 2, 1152, 384, 512     # groups of 1152 rows: the second starts inside row tile 4
+    x, w, b = _mk(S, N, K, torch.bfloat16, seed=61, lead=(B,))
+    g = torch.Generator().manual_seed(62)
+    h = torch.randn(B, S, N, generator=g).bfloat16()
+    mod = torch.randn(B, 6 * N, generator=g).to(gate_dtype)
+    gate = mod[:, 2 * N:3 * N]
+    want = h.double() + gate.double()[:, None, :] * _ref(x, w, b)
+    xg, wg, bg, hg, mg = (t.to(gpu) for t in (x, w, b, h, mod))
+    assert handwritten.linear(xg, wg, bg, residual=hg, gate=mg[:, 2 * N:3 * N], plan_only=True) == (True, 1)
+    got = handwritten.linear(xg, wg, bg, residual=hg, gate=mg[:, 2 * N:3 * N])
+    torch.testing.assert_close(got.double().cpu(), want, atol=4e-2, rtol=2e-2)
+    assert torch.equal(hg.cpu(), h)
+    h2 = hg.clone()
+    inplace = handwritten.linear(xg, wg, bg, residual=h2, gate=mg[:, 2 * N:3 * N], out=h2)
+    assert inplace.data_ptr() == h2.data_ptr() and torch.equal(inplace, got)
+    if gate_dtype == torch.float32:
+        g32 = mg[:, 2 * N:3 * N]
+        gb = torch.zeros_like(mg)
+        gb[:, 2 * N:3 * N] = g32 * bg.float()
+        pre = handwritten.linear(xg, wg, None, residual=hg, gate=g32, gate_bias=gb[:, 2 * N:3 * N], prescaled=True)
+        torch.testing.assert_close(pre.double().cpu(), want, atol=4e-2, rtol=2e-2)
+
+
+def test_tile_gemm_on_a_column_range_of_the_weight(handwritten, gpu):
+    """W as a column range of a wider weight (row stride > K), x and out as column ranges too."""
+    M, N, K = 1536, 256, 128
+    g = torch.Generator().manual_seed(71)
+    wide_w = (torch.randn(N, 3 * K, generator=g) * 0.05).bfloat16()
+    wide_x = torch.randn(M, 2 * K, generator=g).bfloat16()
+    x, w = wide_x[:, K:], wide_w[:, K:2 * K]
+    xg, wg = wide_x.to(gpu)[:, K:], wide_w.to(gpu)[:, K:2 * K]
+    got = handwritten.linear(xg, wg, None)
+    torch.testing.assert_close(got.double().cpu(), _ref(x, w, None), atol=2e-2, rtol=2e-2)
 
 
 def test_linear_tune_compares_both_engines(gpu):

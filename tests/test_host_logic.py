@@ -201,10 +201,21 @@ def test_backend_registry_and_selector(monkeypatch):
     assert get_attn_backend(-1).get_name() == "SDPA"
     get_attn_backend.cache_clear()
     cls = get_attn_backend.__wrapped__(-1).get_impl_cls()
-    with pytest.raises(NotImplementedError):
-        from vllm_omni_amd.attention.backends.hip_flash import HipFlashAttentionImpl
+    from vllm_omni_amd.attention.backends.hip_flash import HipFlashAttentionImpl
 
-        HipFlashAttentionImpl(4, 64, 0.125, causal=True)
+    # what the kernel does not take is routed to SDPA, as the backends this one replaces take it
+    # (vllm_omni/diffusion/attention/backends/sdpa.py:73-92); on the CPU that route runs as it is
+    causal = HipFlashAttentionImpl(4, 64, 0.125, causal=True)
+    assert not causal.kernel_takes_layer and not HipFlashAttentionImpl(2, 96, 0.1).kernel_takes_layer
+    assert HipFlashAttentionImpl(4, 64, 0.125).kernel_takes_layer
+    q = torch.randn(1, 6, 4, 64)
+    want = torch.nn.functional.scaled_dot_product_attention(q.transpose(1, 2), q.transpose(1, 2), q.transpose(1, 2),
+                                                            is_causal=True, scale=0.125).transpose(1, 2)
+    assert torch.allclose(causal.forward(q, q, q), want, atol=1e-6)
+    takes = HipFlashAttentionImpl.kernel_takes_mask
+    assert takes(None, 2, 8) and takes(torch.ones(2, 8, dtype=torch.bool), 2, 8)
+    assert not takes(torch.zeros(2, 8), 2, 8) and not takes(torch.ones(2, 1, 1, 8, dtype=torch.bool), 2, 8)
+    assert not takes(torch.ones(8, 8, dtype=torch.bool), 2, 8)
     assert cls is not None
 
 

@@ -77,6 +77,35 @@ def test_rel_l1_static_equals_the_workspace_entry_point(gpu):
     assert torch.equal(got, want_small)
 
 
+def test_rel_l1_static_clears_what_an_earlier_call_left(gpu):
+    """The built-in array holds whatever the last launch on it left. Filled with garbage through a plain host-to-
+    device copy (ticket words with huge launch numbers, which no atomic maximum of a later launch would override),
+    the next calls still match the workspace entry point: each clears its ticket words first."""
+    import ctypes as C
+
+    from vllm_omni_amd import _lib
+
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    nbytes = C.c_size_t(0)
+    lib.odit_rel_l1_static_scratch.restype = C.c_void_p
+    lib.odit_rel_l1_static_scratch.argtypes = [C.POINTER(C.c_size_t)]
+    ptr = lib.odit_rel_l1_static_scratch(C.byref(nbytes))
+    assert ptr and nbytes.value == 2560, lib.odit_last_error()
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+    hip.hipMemcpy.restype = C.c_int
+    torch.cuda.synchronize()
+    dirt = (C.c_uint8 * nbytes.value)(*([0xEE] * nbytes.value))
+    assert hip.hipMemcpy(ptr, dirt, nbytes.value, 1) == 0   # hipMemcpyHostToDevice
+    for B, n, dtype, flags in ((64, 3000, torch.float32, 0), (2, 4096 * 3072, torch.bfloat16, 1)):
+        print(f"odit_rel_l1_static on a dirtied array: B={B} n={n}", flush=True)
+        pair = _pair(B, n, 9 + B, dtype, gpu)
+        got = _static(lib, *pair, flags, stream)
+        torch.cuda.synchronize()
+        assert torch.equal(got, _with_workspace(lib, *pair, flags, stream))
+
+
 def test_rel_l1_static_limits_and_errors(gpu):
     from vllm_omni_amd import _lib
 

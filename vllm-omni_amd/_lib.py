@@ -20,6 +20,7 @@ ODIT_FLAG_NEOX = 2
 ODIT_NORM_NONE, ODIT_NORM_HEAD, ODIT_NORM_ROW = 0, 1, 2
 ODIT_EPI_NONE, ODIT_EPI_BIAS, ODIT_EPI_GELU_TANH, ODIT_EPI_BIAS_GELU_TANH, ODIT_EPI_GATED_RESIDUAL = 0, 1, 2, 3, 4
 ODIT_EPI_GATED_RESIDUAL_PRE = 5
+ODIT_LINEAR_LIBRARY, ODIT_LINEAR_HANDWRITTEN = 1, 2
 
 # every symbol include/omni_dit.h declares: (name, restype, argtypes)
 _i64p = C.POINTER(C.c_int64)
@@ -84,6 +85,7 @@ _SIGNATURES = {
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_uint, C.c_void_p],
     ),
+    "odit_rel_l1_static_scratch": (C.c_void_p, [C.POINTER(C.c_size_t)]),
     "odit_linear_workspace_bytes": (C.c_size_t, []),
     "odit_linear": (
         C.c_int,
@@ -93,29 +95,27 @@ _SIGNATURES = {
     "odit_linear_rows": (
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
-         C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_void_p,
-         C.c_size_t, C.c_void_p],
+         C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_uint,
+         C.c_void_p, C.c_size_t, C.c_void_p],
     ),
     "odit_linear_rows_plan": (
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
-         C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_void_p,
-         C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_int)],
+         C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_uint,
+         C.c_void_p, C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_int)],
     ),
     "odit_linear_rows_tune": (
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
          C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_void_p,
-         C.c_size_t, C.c_void_p, C.c_int, C.c_void_p, C.c_size_t, C.POINTER(C.c_float)],
+         C.c_size_t, C.c_void_p, C.c_int, C.c_void_p, C.c_size_t, C.POINTER(C.c_float), C.POINTER(C.c_int)],
     ),
-    "odit_linear_set_engine": (C.c_int, [C.c_int]),
     "odit_linear_tune": (
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
          C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p,
          C.c_int, C.c_void_p, C.c_size_t, C.POINTER(C.c_float)],
     ),
-    "odit_probe_mfma": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double), C.c_void_p]),
     "odit_gelu_tanh": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p]),
     "odit_silu": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p]),
 }

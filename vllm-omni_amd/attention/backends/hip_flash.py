@@ -1,6 +1,12 @@
 """The MI355X attention backend: AttentionImpl.forward_hip -> odit_attn_fwd (hand-written gfx950
 flash attention). Takes the place of FlashAttentionBackend (aiter / flash-attn,
-vllm_omni/diffusion/attention/backends/flash_attn.py:25-115) and of SDPABackend for 16-bit inputs."""
+vllm_omni/diffusion/attention/backends/flash_attn.py:25-115) and of SDPABackend for 16-bit inputs.
+
+The kernel is the non-causal joint attention of the DiT blocks: head sizes 64 and 128, an optional [B,Sk]
+key-padding mask. What the backends it replaces also take (vllm_omni/diffusion/attention/backends/sdpa.py:73-92:
+causal attention, any head size, masks of any shape that broadcasts against [B,H,Sq,Sk], boolean or additive)
+goes to this package's SDPA backend, the way float32 inputs already do (attention/layer.py), so a model outside
+the DiT families keeps running when this backend is installed under the names FLASH_ATTN and TORCH_SDPA."""
 
 from __future__ import annotations
 
@@ -8,6 +14,9 @@ import torch
 
 from ... import kernels
 from .abstract import AttentionBackend, AttentionImpl, AttentionMetadata
+from .sdpa import SDPAImpl
+
+KERNEL_HEAD_SIZES = (64, 128)
 
 
 class HipFlashAttentionBackend(AttentionBackend):
@@ -27,21 +36,28 @@ class HipFlashAttentionBackend(AttentionBackend):
 
     @staticmethod
     def get_supported_head_sizes() -> list[int]:
-        return [64, 128]
+        """Head sizes the kernel takes; other sizes are served through the SDPA route of the impl."""
+        return list(KERNEL_HEAD_SIZES)
 
 
 class HipFlashAttentionImpl(AttentionImpl):
     def __init__(self, num_heads: int, head_size: int, softmax_scale: float, causal: bool = False,
                  num_kv_heads: int | None = None, prefix: str = "", **extra_impl_args) -> None:
-        if causal:
-            raise NotImplementedError("HipFlashAttentionImpl is non-causal (DiT joint attention)")
-        if head_size not in HipFlashAttentionBackend.get_supported_head_sizes():
-            raise ValueError(f"head_size {head_size} not supported; supported: 64, 128")
         self.num_heads = num_heads
         self.num_kv_heads = num_kv_heads or num_heads
         self.head_size = head_size
         self.softmax_scale = float(softmax_scale)
-        self.causal = False
+        self.causal = bool(causal)
+        # the route for what the kernel does not take, chosen here (causal, head size) or per call (mask shape)
+        self.sdpa = SDPAImpl(num_heads=num_heads, head_size=head_size, softmax_scale=softmax_scale, causal=causal,
+                             num_kv_heads=num_kv_heads, prefix=prefix, **extra_impl_args)
+        self.kernel_takes_layer = not self.causal and head_size in KERNEL_HEAD_SIZES
+
+    @staticmethod
+    def kernel_takes_mask(mask: torch.Tensor | None, batch: int, keys: int) -> bool:
+        """None, or a [B,Sk] key-padding mask (boolean or 0/1 integers). Everything else (additive float masks,
+        [B,1,1,Sk], [B,H,Sq,Sk], [Sq,Sk]) is SDPA's."""
+        return mask is None or (mask.dim() == 2 and tuple(mask.shape) == (batch, keys) and not mask.is_floating_point())
 
     def forward_hip(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                     attn_metadata: AttentionMetadata | None = None) -> torch.Tensor:
@@ -51,9 +67,9 @@ class HipFlashAttentionImpl(AttentionImpl):
         ``attn_metadata.output_split`` = s the result is the pair (out[:, :s], out[:, s:]), both dense;
         with ``attn_metadata.value_tail`` the values are [value; value_tail] along the keys, read in place."""
         mask = attn_metadata.attn_mask if attn_metadata is not None else None
+        if not self.kernel_takes_layer or not self.kernel_takes_mask(mask, query.shape[0], key.shape[1]):
+            return self.sdpa.forward_hip(query, key, value, attn_metadata)
         if mask is not None:
-            if mask.dim() != 2:
-                raise ValueError("HipFlashAttentionImpl takes a [B,Sk] key-padding mask")
             if not attn_metadata.attn_mask_checked and bool(torch.all(mask != 0)):
                 mask = None
         split = attn_metadata.output_split if attn_metadata is not None else None

@@ -100,6 +100,16 @@ class FeedForward(nn.Module):
                                 fused=self.fused, ref_rounding=ref_rounding, pre=pre)
 
 
+def project(lin: nn.Linear, x: torch.Tensor) -> torch.Tensor:
+    """lin(x). A bf16 projection that a hand-written GEMM kernel would run (the engine asked for, or the one
+    a tuning call found faster for this problem) goes through ``kernels.linear``; everything else through
+    torch's linear (hipBLASLt with the solution table tuned offline)."""
+    if (x.dtype == torch.bfloat16 and x.is_cuda and x.is_contiguous()
+            and kernels.linear(x, lin.weight, lin.bias, plan_only=True)[0]):
+        return kernels.linear(x, lin.weight, lin.bias)
+    return lin(x)
+
+
 # The gate differs per batch entry. The hand-written GEMM takes one gate vector per batch entry in one
 # launch; the library needs one GEMM per entry, and below this many rows per entry (the 256-token text
 # stream of a CFG batch: two GEMMs of 256 rows) one library GEMM over all entries plus the
@@ -255,8 +265,8 @@ class QwenImageCrossAttention(nn.Module):
         B, S_img, _ = hidden_states.shape
         S_txt = encoder_hidden_states.shape[1]
         H, D = self.total_num_heads, self.head_dim
-        img_qkv = self.to_qkv(hidden_states).view(B, S_img, 3, H, D)
-        txt_qkv = self.add_kv_proj(encoder_hidden_states).view(B, S_txt, 3, H, D)
+        img_qkv = project(self.to_qkv, hidden_states).view(B, S_img, 3, H, D)
+        txt_qkv = project(self.add_kv_proj, encoder_hidden_states).view(B, S_txt, 3, H, D)
         S = S_txt + S_img
         jq = torch.empty((B, S, H, D), dtype=img_qkv.dtype, device=img_qkv.device)
         jk = torch.empty_like(jq)

@@ -40,7 +40,9 @@ __device__ __forceinline__ void load_params(const TP* p, float fill, float (&dst
 // waves through 2*W floats of LDS.
 // PLAIN = the per-block call of the DiT step (shift and scale given, no per-token index, no LayerNorm
 // affine): the optional operands cost registers and address arithmetic even when absent, and this
-// pass lives on how many rows a CU keeps in flight.
+// pass lives on how many rows a CU keeps in flight. (A one-wavefront-per-row form with two rows per
+// wavefront streams 5 % faster from cold buffers and 25 % slower on rows a GEMM has just written, which is
+// what every call inside a block sees: 32.5 against 25.6 us per image + text pair launch in the step.)
 //
 // One launch can carry TWO problems of the same width (the image rows and the text rows of a dual-stream
 // block): workgroups [0, rows0) belong to the first, the rest to the second; the choice is
@@ -160,96 +162,6 @@ __global__ __launch_bounds__(W * 64) void adaln_rows_kernel(
   }
 }
 
-// The per-block call at widths up to 64 * NVL vectors (C <= 3072 for 16-bit elements): ONE wavefront per row,
-// NR rows per wavefront, every load of all NR rows issued before the first is used (NR * NVL 16-byte loads in
-// flight per lane), no LDS, no barrier. A read-once / write-once pass is paid by the bytes it keeps in flight:
-// at 8192 rows of 3072 two rows per wavefront on 4096 wavefronts stream 5 % faster than three wavefronts
-// per row (18.5 against 19.6 us on rotating buffers); more rows per wavefront leave too few wavefronts.
-// Wavefront g of the launch takes rows g, g + waves, ... of the two problems laid end to end (rows0 of the
-// first, then the second's). The arithmetic of a row does not depend on NR or on the grid.
-template <typename T, typename TM, int NVL, int NR, bool REF_ROUND>
-__global__ __launch_bounds__(256) void adaln_wave_rows_kernel(
-    const AdalnProblem<T, TM> p0, const AdalnProblem<T, TM> p1, unsigned rows0, unsigned rows, int C, float eps) {
-  constexpr int EPV = Vec16<T>::N;
-  const int lane = threadIdx.x & 63;
-  const unsigned waves = gridDim.x * 4u;
-  const unsigned g = blockIdx.x * 4u + static_cast<unsigned>(__builtin_amdgcn_readfirstlane(threadIdx.x >> 6));
-  u32x4 raw[NR][NVL];
-  float k0[NR];
-#pragma unroll
-  for (int r = 0; r < NR; ++r) {
-    unsigned row = g + static_cast<unsigned>(r) * waves;
-    row = row < rows ? row : rows - 1;  // a wavefront past the end re-reads the last row and stores nothing
-    const bool second = row >= rows0;   // wave-uniform
-    const AdalnProblem<T, TM>& p = second ? p1 : p0;
-    const unsigned local = row - (second ? rows0 : 0u);
-    const int b = static_cast<int>(local / static_cast<unsigned>(p.S));
-    const int s = static_cast<int>(local - static_cast<unsigned>(b) * static_cast<unsigned>(p.S));
-    const T* xr = p.x + b * p.xs_b + s * p.xs_s;
-#pragma unroll
-    for (int i = 0; i < NVL; ++i) {
-      const int c0 = (i * 64 + lane) * EPV;
-      raw[r][i] = c0 < C ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xr + c0)) : u32x4{0u, 0u, 0u, 0u};
-    }
-    k0[r] = to_float(xr[0]);
-  }
-#pragma unroll
-  for (int r = 0; r < NR; ++r) {
-    const unsigned row = g + static_cast<unsigned>(r) * waves;
-    if (row >= rows) break;  // wave-uniform
-    const bool second = row >= rows0;
-    const AdalnProblem<T, TM>& p = second ? p1 : p0;
-    const unsigned local = row - (second ? rows0 : 0u);
-    const int b = static_cast<int>(local / static_cast<unsigned>(p.S));
-    const int s = static_cast<int>(local - static_cast<unsigned>(b) * static_cast<unsigned>(p.S));
-    float s1 = 0.f, s2 = 0.f;
-#pragma unroll
-    for (int i = 0; i < NVL; ++i) {
-      const int c0 = (i * 64 + lane) * EPV;
-      if (c0 < C) {
-#pragma unroll
-        for (int j = 0; j < EPV; ++j) {
-          const float d = Raw<T>::get(raw[r][i], j) - k0[r];
-          s1 += d;
-          s2 = fmaf(d, d, s2);
-        }
-      }
-    }
-    s1 = wave_sum(s1);
-    s2 = wave_sum(s2);
-    const float inv_c = 1.f / static_cast<float>(C);
-    const float m1 = s1 * inv_c;
-    const float mean = k0[r] + m1;
-    const float rstd = rsqrtf(fmaxf(s2 * inv_c - m1 * m1, 0.f) + eps);
-    const TM* sh = p.shift + b * p.mod_stride_b;
-    const TM* sc = p.scale + b * p.mod_stride_b;
-    T* orow = p.out + b * p.os_b + s * p.os_s;
-#pragma unroll
-    for (int i = 0; i < NVL; ++i) {
-      const int c0 = (i * 64 + lane) * EPV;
-      if (c0 < C) {
-        float scl_v[EPV], shf_v[EPV];
-        load_params<TM, EPV>(sc + c0, 0.f, scl_v);
-        load_params<TM, EPV>(sh + c0, 0.f, shf_v);
-        float o_f[EPV];
-#pragma unroll
-        for (int j = 0; j < EPV; ++j) {
-          const float y = (Raw<T>::get(raw[r][i], j) - mean) * rstd;
-          if (REF_ROUND) {
-            o_f[j] = round_to<T>(round_to<T>(y) * round_to<T>(1.f + scl_v[j])) + shf_v[j];
-          } else {
-            o_f[j] = fmaf(y, 1.f + scl_v[j], shf_v[j]);
-          }
-        }
-        u32x4 o;
-#pragma unroll
-        for (int j = 0; j < EPV / 2; ++j) Raw<T>::set2(o, j, o_f[2 * j], o_f[2 * j + 1]);
-        __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(orow + c0));
-      }
-    }
-  }
-}
-
 // Any C (no vector-width or register-cache constraint): the row is read three times through L2.
 template <typename T, typename TM, bool REF_ROUND>
 __global__ __launch_bounds__(256) void adaln_rows_generic_kernel(
@@ -338,26 +250,7 @@ static int launch_adaln(const AdalnRows& r0, const AdalnRows* r1,
                      C, mod_stride_s, eps)
 #define ODIT_ADALN_CASE(WW, NVLL)                                                                  \
   do { if (plain) ODIT_ADALN_LAUNCH(WW, NVLL, true); else ODIT_ADALN_LAUNCH(WW, NVLL, false); } while (0)
-  // the per-block form at up to 6 x 64 vectors per row: one wavefront per row, two rows per wavefront once
-  // that still leaves about 16 wavefronts per CU
-  if (vec_ok && plain && nvec > 128 && nvec <= 6 * 64 && rows <= 0x7fffffffll) {
-    const bool two = rows >= 6144;
-    const unsigned nwaves = static_cast<unsigned>(two ? (rows + 1) / 2 : rows);
-    const dim3 grid((nwaves + 3) / 4);
-#define ODIT_ADALN_WAVE(NVLL)                                                                          \
-  do {                                                                                                 \
-    if (two)                                                                                           \
-      hipLaunchKernelGGL((adaln_wave_rows_kernel<T, TM, NVLL, 2, REF_ROUND>), grid, dim3(256), 0, stream, p0, p1, \
-                         static_cast<unsigned>(rows0), static_cast<unsigned>(rows), C, eps);            \
-    else                                                                                               \
-      hipLaunchKernelGGL((adaln_wave_rows_kernel<T, TM, NVLL, 1, REF_ROUND>), grid, dim3(256), 0, stream, p0, p1, \
-                         static_cast<unsigned>(rows0), static_cast<unsigned>(rows), C, eps);            \
-  } while (0)
-    if (nvec <= 3 * 64) ODIT_ADALN_WAVE(3);
-    else if (nvec <= 4 * 64) ODIT_ADALN_WAVE(4);
-    else ODIT_ADALN_WAVE(6);
-#undef ODIT_ADALN_WAVE
-  } else if (vec_ok && nvec <= 8 * 64 * 2 && rows <= 0x7fffffffll) {
+  if (vec_ok && nvec <= 8 * 64 * 2 && rows <= 0x7fffffffll) {
     if (nvec <= 64) ODIT_ADALN_CASE(1, 1);
     else if (nvec <= 128) ODIT_ADALN_CASE(2, 1);
     else if (nvec <= 256) ODIT_ADALN_CASE(4, 1);

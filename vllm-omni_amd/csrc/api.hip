@@ -1,6 +1,8 @@
 // Version and error-string entry points of libomni_dit_hip.so.
 #include <stdarg.h>
 
+#include <atomic>
+
 #include "odit_common.h"
 
 namespace odit {
@@ -11,6 +13,11 @@ void set_error(const char* fmt, ...) {
   va_start(ap, fmt);
   vsnprintf(g_err, sizeof(g_err), fmt, ap);
   va_end(ap);
+}
+
+uint64_t next_ticket_epoch() {
+  static std::atomic<uint64_t> epoch{0};
+  return (epoch.fetch_add(1, std::memory_order_relaxed) + 1) & ((1ull << 47) - 1);
 }
 }  // namespace odit
 

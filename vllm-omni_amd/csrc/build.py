@@ -20,8 +20,11 @@ CSRC = Path(__file__).resolve().parent
 PKG = CSRC.parent
 LIB_NAME = "libomni_dit_hip.so"
 LIB_PATH = PKG / LIB_NAME
+# bench.py's calibration probe (a bare MFMA loop): a library of its own, not part of the product's C ABI
+PROBE_LIB_PATH = PKG / "libomni_dit_probe.so"
 OBJ_DIR = CSRC / "build"
-HEADERS = [CSRC / "odit_common.h", CSRC / "attn_common.h", CSRC / "attn_tail.h", CSRC / "gemm_bf16.h", PKG.parent / "include" / "omni_dit.h"]
+HEADERS = [CSRC / "odit_common.h", CSRC / "attn_common.h", CSRC / "attn_tail.h", CSRC / "gemm_bf16.h",
+           CSRC / "gemm_epilogue.h", PKG.parent / "include" / "omni_dit.h"]
 
 # (source file, extra defines, object stem)
 UNITS: list[tuple[str, list[str], str]] = [
@@ -36,8 +39,9 @@ UNITS: list[tuple[str, list[str], str]] = [
     ("attn_fwd_dma.hip", [], "attn_fwd_dma"),
     ("linear.hip", [], "linear"),
     ("gemm_bf16.hip", [], "gemm_bf16"),
-    ("probe.hip", [], "probe"),
+    ("gemm_bf16_tile.hip", [], "gemm_bf16_tile"),
 ]
+PROBE_UNITS: list[tuple[str, list[str], str]] = [("probe.hip", [], "probe")]
 
 # the dense projections call hipBLASLt (its MFMA GEMM kernels); everything else is self-contained
 LINK_LIBS = ["-L/opt/rocm/lib", "-lhipblaslt"]
@@ -82,25 +86,27 @@ def build(force: bool = False, jobs: int | None = None, verbose: bool = True) ->
     OBJ_DIR.mkdir(exist_ok=True)
     jobs = jobs or min(8, os.cpu_count() or 1)
     work = []
-    objs = []
-    for src, defines, stem in UNITS:
-        src_path = CSRC / src
-        if not src_path.exists():
-            raise RuntimeError(f"missing source {src_path}")
-        obj = OBJ_DIR / f"{stem}.o"
-        objs.append(obj)
-        if force or _stale(obj, [src_path, *HEADERS, Path(__file__)]):
-            work.append([hipcc, *HIPCC_FLAGS, *defines, "-c", str(src_path), "-o", str(obj)])
+    objs: dict[Path, list[Path]] = {LIB_PATH: [], PROBE_LIB_PATH: []}
+    for lib, units in ((LIB_PATH, UNITS), (PROBE_LIB_PATH, PROBE_UNITS)):
+        for src, defines, stem in units:
+            src_path = CSRC / src
+            if not src_path.exists():
+                raise RuntimeError(f"missing source {src_path}")
+            obj = OBJ_DIR / f"{stem}.o"
+            objs[lib].append(obj)
+            if force or _stale(obj, [src_path, *HEADERS, Path(__file__)]):
+                work.append([hipcc, *HIPCC_FLAGS, *defines, "-c", str(src_path), "-o", str(obj)])
     if verbose:
-        print(f"[omni_dit build] compiling {len(work)}/{len(UNITS)} units with {jobs} jobs", flush=True)
+        print(f"[omni_dit build] compiling {len(work)}/{len(UNITS) + len(PROBE_UNITS)} units with {jobs} jobs", flush=True)
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         list(ex.map(_run, work))
-    if work or force or not LIB_PATH.exists():
-        tmp = LIB_PATH.with_suffix(".so.tmp")
-        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs), *LINK_LIBS])
-        os.replace(tmp, LIB_PATH)
-    if verbose:
-        print(f"[omni_dit build] {LIB_PATH} ({LIB_PATH.stat().st_size} bytes)", flush=True)
+    for lib, link in ((LIB_PATH, LINK_LIBS), (PROBE_LIB_PATH, [])):
+        if work or force or not lib.exists():
+            tmp = lib.with_suffix(".so.tmp")
+            _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs[lib]), *link])
+            os.replace(tmp, lib)
+        if verbose:
+            print(f"[omni_dit build] {lib} ({lib.stat().st_size} bytes)", flush=True)
     return LIB_PATH
 
 

@@ -11,7 +11,9 @@
 // contributor that finds the tile's counter short of full leaves its fp32 partial tile in a scratch slot
 // (write-through stores) and takes a ticket; the last arriver adds the partial tiles in workgroup order
 // (its own, still in registers, in its place: the sum does not depend on who arrives last), runs the
-// epilogue and resets the counter. Nobody waits for anybody.
+// epilogue and resets the counter. Nobody waits for anybody. A ticket word is (epoch << 16 | tickets): a
+// contributor first raises the word to this launch's epoch with an atomic maximum, so what an earlier
+// launch left there (one that never finished, say) cannot be mistaken for this launch's tickets.
 //
 // Workgroup: 8 wavefronts = 2 halves of each step's reduction x 4 corners (64 x 96) of the tile; a wave
 // holds 3 x 2 accumulators of v_mfma_f32_32x32x16_bf16 (W rows as the A operand, x rows as B: a lane
@@ -33,8 +35,7 @@
 // but leave a 512-row problem with too few tiles to balance without far more partial-tile traffic.
 // Measured at M=512 (cold weights): 0.84 us per step; N=3072, K=12288 in 58 us against 72 us for the
 // library's best kernel, N=9216, K=3072 in 52 us against 43 us.
-#include "attn_common.h"
-#include "gemm_bf16.h"
+#include "gemm_epilogue.h"
 
 namespace odit {
 
@@ -52,24 +53,19 @@ constexpr int kSlotFloats = kGemmBM * kGemmBN;
 static_assert(kInstPerStage % kWaves == 0, "tile loads must divide evenly over the wavefronts");
 
 struct GemmParams {
-  const void *x, *w, *bias, *residual, *gate;
-  void* out;
+  const void *x, *w;
   int M, N, K;
-  int64_t ldx, ldw, ldo, ldr, ldg;
-  int epilogue, gate_f32, rows_per_gate;
+  int64_t ldx, ldw;
+  GemmEpilogue ep;
   uint32_t x_bytes, w_bytes;
   int m_tiles, k_steps, workers, groups;
   int64_t total_steps;  // per group: feature tiles x reduction steps
-  unsigned* counters;
+  unsigned long long* counters;  // one ticket word per output tile: (epoch << 16 | tickets drawn), zero between launches
+  unsigned long long epoch;      // larger than that of any earlier launch of the process
   float* slots;
 };
 
 typedef __attribute__((address_space(3))) void* lds_void_p;
-
-__device__ __forceinline__ float gelu_tanh_f(float x) {
-  const float u = 0.7978845608028654f * x * fmaf(0.044715f * x, x, 1.f);
-  return x / (1.f + __expf(-2.f * u));
-}
 
 // worker whose range [v S / W, (v + 1) S / W) holds `step`
 __device__ __forceinline__ int worker_of(int64_t step, int64_t S, int W) {
@@ -261,19 +257,19 @@ __global__ __launch_bounds__(kWaves * 64, 1) void gemm_bf16_streamk_kernel(const
         return p.slots + (static_cast<size_t>(2 * (j * p.m_tiles + mt) + (first_tile == t ? 0 : 1))) * kSlotFloats;
       };
       const int lane_off = (w4 * 6 + kh * 3) * (16 * 64) + lane;
-      unsigned* ctr = p.counters + t * p.m_tiles + mt;
-      const unsigned others = static_cast<unsigned>(v_last - v_first);
+      unsigned long long* ctr = p.counters + t * p.m_tiles + mt;
+      const unsigned long long full = (p.epoch << 16) + static_cast<unsigned>(v_last - v_first);
       // When every other contributor has already taken its ticket this workgroup is the last arriver
       // and keeps its partial tile in registers; otherwise the tile goes to the slot first and the
       // ticket is taken after it (whoever then holds the last ticket reduces).
       if (tid == 0)
         *reinterpret_cast<volatile int*>(flag) =
-            __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == others ? 1 : 0;
+            __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == full ? 1 : 0;
       __syncthreads();
       const bool known_last = *reinterpret_cast<volatile int*>(flag) != 0;
       __syncthreads();  // the flag is read before it is written again
       if (known_last) {
-        if (tid == 0) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0) __hip_atomic_store(ctr, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       } else {
         float* mine = slot_of(group) + lane_off;
 #pragma unroll
@@ -284,9 +280,11 @@ __global__ __launch_bounds__(kWaves * 64, 1) void gemm_bf16_streamk_kernel(const
         __builtin_amdgcn_s_waitcnt(0);  // the partial tile has reached memory before the ticket is taken
         __syncthreads();
         if (tid == 0) {
-          const unsigned ticket = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          const int last = ticket == others;
-          if (last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          // two atomics of one thread on one address: applied in program order
+          __hip_atomic_fetch_max(ctr, p.epoch << 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const unsigned long long ticket = __hip_atomic_fetch_add(ctr, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const int last = ticket == full;
+          if (last) __hip_atomic_store(ctr, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           *reinterpret_cast<volatile int*>(flag) = last;
         }
         __syncthreads();
@@ -342,11 +340,6 @@ __global__ __launch_bounds__(kWaves * 64, 1) void gemm_bf16_streamk_kernel(const
         }
       }
       __syncthreads();  // a corner is written by two waves and read by the same two
-      const bf16_t* bias_h = static_cast<const bf16_t*>(p.bias);
-      const float* bias_f = static_cast<const float*>(p.bias);
-      const bool gelu = p.epilogue == ODIT_EPI_GELU_TANH || p.epilogue == ODIT_EPI_BIAS_GELU_TANH;
-      const bool gated = p.epilogue == ODIT_EPI_GATED_RESIDUAL || p.epilogue == ODIT_EPI_GATED_RESIDUAL_PRE;
-      const bool pre = p.epilogue == ODIT_EPI_GATED_RESIDUAL_PRE;
 #pragma unroll 3
       for (int it = 0; it < 6; ++it) {
         const int idx = (kh * 6 + it) * 64 + lane;
@@ -359,57 +352,13 @@ __global__ __launch_bounds__(kWaves * 64, 1) void gemm_bf16_streamk_kernel(const
         float y[8];
 #pragma unroll
         for (int u = 0; u < 4; ++u) { y[u] = lo[u]; y[4 + u] = hi[u]; }
-        if (gated) {
-          const int64_t grow = p.rows_per_gate > 0 ? static_cast<int64_t>(m / p.rows_per_gate) * p.ldg : 0;
-          float gt[8], bs[8];
-#pragma unroll
-          for (int u = 0; u < 8; ++u) { gt[u] = 1.f; bs[u] = 0.f; }
-          if (p.gate != nullptr) {
-            if (p.gate_f32) {
-              const float* gp = static_cast<const float*>(p.gate) + grow + n;
-              const f32x4_v g0 = *reinterpret_cast<const f32x4_v*>(gp), g1 = *reinterpret_cast<const f32x4_v*>(gp + 4);
-#pragma unroll
-              for (int u = 0; u < 4; ++u) { gt[u] = g0[u]; gt[4 + u] = g1[u]; }
-            } else {
-              const u32x4 gv = load_raw(static_cast<const bf16_t*>(p.gate) + grow + n);
-#pragma unroll
-              for (int u = 0; u < 8; ++u) gt[u] = Raw<bf16_t>::get(gv, u);
-            }
-          }
-          if (p.bias != nullptr) {
-            if (pre) {  // float32, already multiplied by the gate, one vector per gate vector
-              const float* bp = bias_f + grow + n;
-              const f32x4_v b0 = *reinterpret_cast<const f32x4_v*>(bp), b1 = *reinterpret_cast<const f32x4_v*>(bp + 4);
-#pragma unroll
-              for (int u = 0; u < 4; ++u) { bs[u] = b0[u]; bs[4 + u] = b1[u]; }
-            } else {
-              const u32x4 bv = load_raw(bias_h + n);
-#pragma unroll
-              for (int u = 0; u < 8; ++u) bs[u] = gt[u] * Raw<bf16_t>::get(bv, u);
-            }
-          }
-          const u32x4 rv = load_raw(static_cast<const bf16_t*>(p.residual) + m * p.ldr + n);
-#pragma unroll
-          for (int u = 0; u < 8; ++u) y[u] = fmaf(gt[u], y[u], bs[u]) + Raw<bf16_t>::get(rv, u);
-        } else {
-          if (p.bias != nullptr) {
-            const u32x4 bv = load_raw(bias_h + n);
-#pragma unroll
-            for (int u = 0; u < 8; ++u) y[u] += Raw<bf16_t>::get(bv, u);
-          }
-          if (gelu) {
-#pragma unroll
-            for (int u = 0; u < 8; ++u) y[u] = gelu_tanh_f(y[u]);
-          }
-        }
-        u32x4 o;
-#pragma unroll
-        for (int u = 0; u < 4; ++u) Raw<bf16_t>::set2(o, u, y[2 * u], y[2 * u + 1]);
-        store_raw(static_cast<bf16_t*>(p.out) + m * p.ldo + n, o);
+        gemm_epilogue_store8(p.ep, m, n, y);
       }
     }
   }
 }
+
+}  // namespace
 
 int device_cus() {
   static int cus[64] = {0};
@@ -422,8 +371,6 @@ int device_cus() {
   }
   return cus[dev];
 }
-
-}  // namespace
 
 void gemm_streamk_shape(int M, int N, int K, int cus, int* workers, int* steps_per_worker, int* tiles) {
   const int m_tiles = (M + kGemmBM - 1) / kGemmBM, n_tiles = (N + kGemmBN - 1) / kGemmBN;
@@ -451,17 +398,17 @@ bool gemm_streamk_takes(const GemmCall& c, int dtype) {
   const uint64_t xb = (static_cast<uint64_t>(c.M - 1) * c.ldx + c.K) * 2, wb = (static_cast<uint64_t>(c.N - 1) * c.ldw + c.K) * 2;
   if (xb >= (1ull << 32) || wb >= (1ull << 32)) return false;
   const int64_t tiles = static_cast<int64_t>((c.M + kGemmBM - 1) / kGemmBM) * ((c.N + kGemmBN - 1) / kGemmBN);
-  return tiles * sizeof(unsigned) <= kGemmCounterBytes;
+  return tiles * sizeof(unsigned long long) <= kGemmCounterBytes;
 }
 
 int launch_gemm_streamk(const GemmCall& c, void* scratch, hipStream_t stream) {
   const int cus = device_cus();
   if (cus <= 0) { set_error("odit_linear: cannot read the device's compute-unit count"); return ODIT_ELAUNCH; }
   GemmParams p;
-  p.x = c.x; p.w = c.w; p.bias = c.bias; p.residual = c.residual; p.gate = c.gate; p.out = c.out;
+  p.x = c.x; p.w = c.w;
   p.M = c.M; p.N = c.N; p.K = c.K;
-  p.ldx = c.ldx; p.ldw = c.ldw; p.ldo = c.ldo; p.ldr = c.ldr; p.ldg = c.ldg;
-  p.epilogue = c.epilogue; p.gate_f32 = c.gate_f32; p.rows_per_gate = c.rows_per_gate;
+  p.ldx = c.ldx; p.ldw = c.ldw;
+  p.ep = gemm_epilogue_of(c);
   p.x_bytes = static_cast<uint32_t>((static_cast<uint64_t>(c.M - 1) * c.ldx + c.K) * 2);
   p.w_bytes = static_cast<uint32_t>((static_cast<uint64_t>(c.N - 1) * c.ldw + c.K) * 2);
   p.m_tiles = (c.M + kGemmBM - 1) / kGemmBM;
@@ -470,7 +417,8 @@ int launch_gemm_streamk(const GemmCall& c, void* scratch, hipStream_t stream) {
   gemm_streamk_shape(c.M, c.N, c.K, cus, &p.workers, &spw, &tiles);
   p.groups = p.workers / p.m_tiles;
   p.total_steps = static_cast<int64_t>(tiles / p.m_tiles) * p.k_steps;
-  p.counters = static_cast<unsigned*>(scratch);
+  p.counters = static_cast<unsigned long long*>(scratch);
+  p.epoch = next_ticket_epoch();
   p.slots = reinterpret_cast<float*>(static_cast<char*>(scratch) + kGemmCounterBytes);
   hipLaunchKernelGGL(gemm_bf16_streamk_kernel, dim3(p.workers), dim3(kWaves * 64), 0, stream, p);
   return check_launch("odit_linear (stream-K kernel)");

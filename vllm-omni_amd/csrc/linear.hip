@@ -18,7 +18,7 @@
 #include <hipblaslt/hipblaslt-ext.hpp>
 
 #include <algorithm>
-#include <atomic>
+#include <mutex>
 #include <unordered_map>
 #include <vector>
 
@@ -69,11 +69,15 @@ struct LinPlan {
 struct LinState {
   hipblasLtHandle_t handle[64] = {nullptr};
   std::unordered_map<LinKey, LinPlan, LinKeyHash> plans;
-  // problems for which a tuning call has compared the hand-written kernel with the library:
-  // true = the hand-written kernel won (key: the whole problem, rows_per_gate in the lda field)
-  std::unordered_map<LinKey, bool, LinKeyHash> handwritten_wins;
 };
 static thread_local LinState g_lin;
+
+// Problems for which a tuning call has compared the hand-written kernel with the library: true = the
+// hand-written kernel won (key: the whole problem, rows_per_gate in the lda field). Process-wide and kept
+// for the life of the process: every host thread sees what any thread has measured, and the record
+// outlives the per-thread descriptor cache.
+static std::mutex g_engine_mu;
+static std::unordered_map<LinKey, bool, LinKeyHash> g_handwritten_wins;
 
 #define ODIT_LT(call)                                                                      \
   do {                                                                                     \
@@ -142,7 +146,6 @@ static int lin_plan(const LinKey& key, LinPlan** out) {
   if (g_lin.plans.size() >= kMaxPlans) {
     for (auto& kv : g_lin.plans) lin_plan_release(kv.second);
     g_lin.plans.clear();
-    g_lin.handwritten_wins.clear();
   }
   LinPlan p;
   const int rc = lin_plan_build(key, p);
@@ -155,9 +158,11 @@ static int lin_plan(const LinKey& key, LinPlan** out) {
   return ODIT_OK;
 }
 
-// 0 = the hand-written kernel where it takes the problem, else the library; 1 = library only;
-// 2 = hand-written only (problems it does not take fail with ODIT_ENOTSUP)
-static std::atomic<int> g_engine{0};
+// engine bits of the `flags` argument: neither = the hand-written kernel where it takes the problem and is
+// expected (or was measured) to win, else the library
+static int lin_engine_of(unsigned flags) {
+  return (flags & ODIT_LINEAR_LIBRARY) ? 1 : ((flags & ODIT_LINEAR_HANDWRITTEN) ? 2 : 0);
+}
 
 struct LinCall {
   const void *x, *w, *bias, *residual, *gate;
@@ -334,12 +339,32 @@ static odit::LinKey lin_engine_key(int dev, const odit::LinCall& c, int rows_per
                       c.dtype, rows_per_gate, c.ldx, c.ldw, c.ldo};
 }
 
-// Without a tuning record the hand-written kernel is used where the reduction is long against the
-// number of output tiles (K >= 2 N: the library's choices split K badly there, measured 58 vs 72 us at
-// M=512, N=3072, K=12288) and the library elsewhere.
-static bool lin_prefers_handwritten(int dev, const odit::LinCall& c, int rows_per_gate) {
-  const auto it = odit::g_lin.handwritten_wins.find(lin_engine_key(dev, c, rows_per_gate));
-  if (it != odit::g_lin.handwritten_wins.end()) return it->second;
+// Which hand-written kernel takes a problem: 1 = the stream-K kernel (few rows; needs its scratch), 2 = the
+// tile kernel (many rows), 0 = neither.
+constexpr int kTileMinRows = 1025;
+static int lin_handwritten_kind(const odit::GemmCall& g, int dtype, const void* sk) {
+  if (g.M >= kTileMinRows) return odit::gemm_tile_takes(g, dtype) ? 2 : 0;
+  return sk != nullptr && odit::gemm_streamk_takes(g, dtype) ? 1 : 0;
+}
+
+static int lin_launch_handwritten(int kind, const odit::GemmCall& g, void* sk, hipStream_t stream) {
+  if (kind == 1) return odit::launch_gemm_streamk(g, sk, stream);
+  const int cus = odit::device_cus();
+  if (cus <= 0) { odit::set_error("odit_linear: cannot read the device's compute-unit count"); return ODIT_ELAUNCH; }
+  return odit::launch_gemm_tile(g, cus, stream);
+}
+
+// Without a tuning record: the stream-K kernel where the reduction is long against the number of output
+// tiles (K >= 2 N: the library's choices split K badly there, measured 58 vs 72 us at M=512, N=3072,
+// K=12288); the tile kernel for the gated form with one gate vector per group of rows, where the library
+// needs a launch per group, and for the other forms where measured faster (ODIT_TILE_DEFAULT_ALL).
+static bool lin_prefers_handwritten(int dev, int kind, const odit::LinCall& c, int rows_per_gate) {
+  {
+    std::lock_guard<std::mutex> lock(odit::g_engine_mu);
+    const auto it = odit::g_handwritten_wins.find(lin_engine_key(dev, c, rows_per_gate));
+    if (it != odit::g_handwritten_wins.end()) return it->second;
+  }
+  if (kind == 2) return false;
   return c.K >= 2 * c.N;
 }
 
@@ -347,17 +372,15 @@ extern "C" size_t odit_linear_workspace_bytes(void) {
   return odit::kGemmScratchBytes + (static_cast<size_t>(64) << 20);
 }
 
-extern "C" int odit_linear_set_engine(int engine) {
-  if (engine < 0 || engine > 2) { odit::set_error("odit_linear_set_engine: engine must be 0, 1 or 2"); return ODIT_EINVAL; }
-  odit::g_engine.store(engine);
-  return ODIT_OK;
-}
-
 extern "C" int odit_linear_rows(const void* x, const void* w, const void* bias, void* out, const void* residual,
                                 const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
                                 int64_t ldr, int epilogue, int gate_dtype, int dtype, int rows_per_gate,
-                                int64_t gate_stride, void* workspace, size_t workspace_bytes, void* stream) {
+                                int64_t gate_stride, unsigned flags, void* workspace, size_t workspace_bytes,
+                                void* stream) {
   using namespace odit;
+  ODIT_CHECK_ARG((flags & ~(ODIT_LINEAR_LIBRARY | ODIT_LINEAR_HANDWRITTEN)) == 0 &&
+                     (flags & (ODIT_LINEAR_LIBRARY | ODIT_LINEAR_HANDWRITTEN)) != (ODIT_LINEAR_LIBRARY | ODIT_LINEAR_HANDWRITTEN),
+                 "odit_linear_rows: flags may name one engine (ODIT_LINEAR_LIBRARY or ODIT_LINEAR_HANDWRITTEN), got %#x", flags);
   void *sk, *lib;
   size_t lib_bytes;
   lin_split_ws(workspace, workspace_bytes, &sk, &lib, &lib_bytes);
@@ -368,18 +391,18 @@ extern "C" int odit_linear_rows(const void* x, const void* w, const void* bias, 
   ODIT_CHECK_ARG(rows_per_gate >= 0 && (rows_per_gate == 0 || gate_stride >= 0),
                  "odit_linear_rows: rows_per_gate and gate_stride must not be negative");
   const bool per_rows = lin_is_residual(c) && gate != nullptr && rows_per_gate > 0 && rows_per_gate < M;
-  const int engine = g_engine.load();
+  const int engine = lin_engine_of(flags);
   const GemmCall g = lin_gemm_call(c, per_rows ? rows_per_gate : 0, per_rows ? gate_stride : 0);
-  const bool takes = sk != nullptr && gemm_streamk_takes(g, dtype);
-  if (engine == 2 && !takes) {
-    set_error("odit_linear: the hand-written kernel does not take this problem (M=%d N=%d K=%d, workspace %zu bytes)",
+  const int kind = lin_handwritten_kind(g, dtype, sk);
+  if (engine == 2 && kind == 0) {
+    set_error("odit_linear: no hand-written kernel takes this problem (M=%d N=%d K=%d, workspace %zu bytes)",
               M, N, K, workspace_bytes);
     return ODIT_ENOTSUP;
   }
-  if (takes && engine != 1) {
+  if (kind != 0 && engine != 1) {
     int dev = 0;
-    if (engine == 2 || (hipGetDevice(&dev) == hipSuccess && lin_prefers_handwritten(dev, c, g.rows_per_gate)))
-      return launch_gemm_streamk(g, sk, c.stream);
+    if (engine == 2 || (hipGetDevice(&dev) == hipSuccess && lin_prefers_handwritten(dev, kind, c, g.rows_per_gate)))
+      return lin_launch_handwritten(kind, g, sk, c.stream);
   }
   if (!per_rows) return lin_run_library(c);
   // the library's epilogue takes one gate vector per launch: one launch per group of rows
@@ -403,8 +426,8 @@ extern "C" int odit_linear_rows(const void* x, const void* w, const void* bias, 
 extern "C" int odit_linear_rows_plan(const void* x, const void* w, const void* bias, void* out, const void* residual,
                                      const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
                                      int64_t ldr, int epilogue, int gate_dtype, int dtype, int rows_per_gate,
-                                     int64_t gate_stride, void* workspace, size_t workspace_bytes, int* handwritten,
-                                     int* launches) {
+                                     int64_t gate_stride, unsigned flags, void* workspace, size_t workspace_bytes,
+                                     int* handwritten, int* launches) {
   using namespace odit;
   void *sk, *lib;
   size_t lib_bytes;
@@ -415,12 +438,12 @@ extern "C" int odit_linear_rows_plan(const void* x, const void* w, const void* b
   if (rc != ODIT_OK) return rc;
   ODIT_CHECK_ARG(handwritten != nullptr && launches != nullptr, "odit_linear_rows_plan: null result pointers");
   const bool per_rows = lin_is_residual(c) && gate != nullptr && rows_per_gate > 0 && rows_per_gate < M;
-  const int engine = g_engine.load();
+  const int engine = lin_engine_of(flags);
   const GemmCall g = lin_gemm_call(c, per_rows ? rows_per_gate : 0, per_rows ? gate_stride : 0);
   int dev = 0;
   (void)hipGetDevice(&dev);
-  const bool takes = M > 0 && sk != nullptr && gemm_streamk_takes(g, dtype);
-  const bool own = takes && engine != 1 && (engine == 2 || lin_prefers_handwritten(dev, c, g.rows_per_gate));
+  const int kind = M > 0 ? lin_handwritten_kind(g, dtype, sk) : 0;
+  const bool own = kind != 0 && engine != 1 && (engine == 2 || lin_prefers_handwritten(dev, kind, c, g.rows_per_gate));
   *handwritten = own ? 1 : 0;
   *launches = M == 0 ? 0 : (own || !per_rows ? 1 : (M + rows_per_gate - 1) / rows_per_gate);
   if (!own && lin_needs_prep(c)) *launches *= 2;  // plus the [N]-sized gate-vector launch of the library form
@@ -432,7 +455,7 @@ extern "C" int odit_linear(const void* x, const void* w, const void* bias, void*
                            int64_t ldr, int epilogue, int gate_dtype, int dtype, void* workspace,
                            size_t workspace_bytes, void* stream) {
   return odit_linear_rows(x, w, bias, out, residual, gate, M, N, K, ldx, ldw, ldo, ldr, epilogue, gate_dtype, dtype, 0,
-                          0, workspace, workspace_bytes, stream);
+                          0, 0u, workspace, workspace_bytes, stream);
 }
 
 // Times the library's kernels for problem c (cold caches before every timed launch when a flush buffer
@@ -512,7 +535,7 @@ static int lin_tune_library(const odit::LinCall& c, int iters, void* flush, size
   return ODIT_OK;
 }
 
-static int lin_time_handwritten(const odit::GemmCall& g, void* sk, hipStream_t stream, int iters, void* flush,
+static int lin_time_handwritten(int kind, const odit::GemmCall& g, void* sk, hipStream_t stream, int iters, void* flush,
                                 size_t flush_bytes, float* us) {
   using namespace odit;
   hipEvent_t e0, e1;
@@ -520,12 +543,12 @@ static int lin_time_handwritten(const odit::GemmCall& g, void* sk, hipStream_t s
     set_error("odit_linear_tune: hipEventCreate failed");
     return ODIT_ELAUNCH;
   }
-  int rc = launch_gemm_streamk(g, sk, stream);
+  int rc = lin_launch_handwritten(kind, g, sk, stream);
   float total = 0.f;
   for (int i = 0; i < iters && rc == ODIT_OK; ++i) {
     if (flush != nullptr && flush_bytes > 0) (void)hipMemsetAsync(flush, i & 0xff, flush_bytes, stream);
     (void)hipEventRecord(e0, stream);
-    rc = launch_gemm_streamk(g, sk, stream);
+    rc = lin_launch_handwritten(kind, g, sk, stream);
     (void)hipEventRecord(e1, stream);
     if (hipEventSynchronize(e1) != hipSuccess) { set_error("odit_linear_tune: hipEventSynchronize failed"); rc = ODIT_ELAUNCH; }
     float ms = 0.f;
@@ -542,8 +565,9 @@ extern "C" int odit_linear_rows_tune(const void* x, const void* w, const void* b
                                      const void* gate, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
                                      int64_t ldr, int epilogue, int gate_dtype, int dtype, int rows_per_gate,
                                      int64_t gate_stride, void* workspace, size_t workspace_bytes, void* stream,
-                                     int iters, void* flush, size_t flush_bytes, float* best_us) {
+                                     int iters, void* flush, size_t flush_bytes, float* best_us, int* handwritten) {
   using namespace odit;
+  if (handwritten) *handwritten = 0;
   void *sk, *lib;
   size_t lib_bytes;
   lin_split_ws(workspace, workspace_bytes, &sk, &lib, &lib_bytes);
@@ -567,13 +591,17 @@ extern "C" int odit_linear_rows_tune(const void* x, const void* w, const void* b
   lib_us *= static_cast<float>(launches);
   float best = lib_us;
   const GemmCall g = lin_gemm_call(c, per_rows ? rows_per_gate : 0, per_rows ? gate_stride : 0);
-  if (sk != nullptr && gemm_streamk_takes(g, dtype)) {
+  if (const int kind = lin_handwritten_kind(g, dtype, sk)) {
     float own_us = 0.f;
-    rc = lin_time_handwritten(g, sk, c.stream, iters, flush, flush_bytes, &own_us);
+    rc = lin_time_handwritten(kind, g, sk, c.stream, iters, flush, flush_bytes, &own_us);
     if (rc != ODIT_OK) return rc;
     int dev = 0;
     (void)hipGetDevice(&dev);
-    g_lin.handwritten_wins[lin_engine_key(dev, c, per_rows ? rows_per_gate : 0)] = own_us < lib_us;
+    {
+      std::lock_guard<std::mutex> lock(g_engine_mu);
+      g_handwritten_wins[lin_engine_key(dev, c, per_rows ? rows_per_gate : 0)] = own_us < lib_us;
+    }
+    if (handwritten) *handwritten = own_us < lib_us ? 1 : 0;
     if (own_us < best) best = own_us;
   }
   if (best_us) *best_us = best;
@@ -586,5 +614,5 @@ extern "C" int odit_linear_tune(const void* x, const void* w, const void* bias, 
                                 size_t workspace_bytes, void* stream, int iters, void* flush,
                                 size_t flush_bytes, float* best_us) {
   return odit_linear_rows_tune(x, w, bias, out, residual, gate, M, N, K, ldx, ldw, ldo, ldr, epilogue, gate_dtype, dtype,
-                               0, 0, workspace, workspace_bytes, stream, iters, flush, flush_bytes, best_us);
+                               0, 0, workspace, workspace_bytes, stream, iters, flush, flush_bytes, best_us, nullptr);
 }

@@ -31,6 +31,10 @@ inline int check_launch(const char* what) {
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// A number larger than any this function has returned before in this process (never 0, below 2^47): the
+// epoch of the ticket words that rel_l1.hip and gemm_bf16.hip keep in caller scratch.
+uint64_t next_ticket_epoch();
+
 // ---- element types -----------------------------------------------------------------------------
 // Storage structs are raw bit containers; all arithmetic goes through float.
 struct bf16_t { uint16_t bits; };
@@ -63,6 +67,7 @@ template <typename T> __device__ __forceinline__ float round_to(float f) {
 }
 
 // ---- 16-byte vectors ---------------------------------------------------------------------------
+typedef uint32_t u32x4_nt __attribute__((ext_vector_type(4)));
 template <typename T> struct Vec16 {
   static constexpr int N = 16 / sizeof(T);
   T e[N];
@@ -71,6 +76,13 @@ template <typename T> __device__ __forceinline__ Vec16<T> load16(const T* p) {
   static_assert(sizeof(Vec16<T>) == 16, "Vec16 must be 16 bytes");
   Vec16<T> v;
   *reinterpret_cast<uint4*>(&v) = *reinterpret_cast<const uint4*>(p);
+  return v;
+}
+// the same for data that is read once: the load is marked non-temporal, so the lines do not push reusable
+// data out of the caches
+template <typename T> __device__ __forceinline__ Vec16<T> load16_stream(const T* p) {
+  Vec16<T> v;
+  *reinterpret_cast<u32x4_nt*>(&v) = __builtin_nontemporal_load(reinterpret_cast<const u32x4_nt*>(p));
   return v;
 }
 template <typename T> __device__ __forceinline__ void store16(T* p, const Vec16<T>& v) {

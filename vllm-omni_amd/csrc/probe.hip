@@ -4,7 +4,11 @@
 // 2.2 PFLOP/s, with random operands (what activations look like) about 1.6 PFLOP/s, against the
 // 2.5 PFLOP/s that 256 CUs x 4 SIMDs x one 32-cycle MFMA at 2.4 GHz would give. A kernel's fraction
 // of the nominal peak has to be read against these.
-#include "odit_common.h"
+//
+// Built into a library of its own (libomni_dit_probe.so): a measurement aid for bench.py, not part of the
+// product's C ABI.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
 namespace odit {
 
@@ -59,9 +63,13 @@ __global__ __launch_bounds__(512) void probe_mfma_kernel(float* __restrict__ sin
 
 }  // namespace odit
 
+// Launches `workgroups` workgroups of 8 wavefronts that issue nothing but v_mfma_f32_32x32x16_bf16
+// (iters x 8 per wavefront) on register operands holding constant (random_operands = 0) or pseudo-random
+// data, writes one float per thread to `sink` (workgroups * 512 floats) and returns the flop count of the
+// launch in *flop. Timed by the caller with events on `stream`. Returns 0, -1 (bad argument) or -3 (launch).
 extern "C" int odit_probe_mfma(int random_operands, int iters, int workgroups, float* sink, double* flop, void* stream) {
   using namespace odit;
-  ODIT_CHECK_ARG(iters > 0 && workgroups > 0 && sink != nullptr, "odit_probe_mfma: needs iters, workgroups > 0 and a sink");
+  if (iters <= 0 || workgroups <= 0 || sink == nullptr) return -1;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (random_operands) {
     hipLaunchKernelGGL(probe_mfma_kernel<true>, dim3(workgroups), dim3(512), 0, st, sink, iters);
@@ -69,5 +77,5 @@ extern "C" int odit_probe_mfma(int random_operands, int iters, int workgroups, f
     hipLaunchKernelGGL(probe_mfma_kernel<false>, dim3(workgroups), dim3(512), 0, st, sink, iters);
   }
   if (flop) *flop = static_cast<double>(workgroups) * 8 /*waves*/ * iters * 8 /*MFMAs*/ * 32768.0;
-  return check_launch("odit_probe_mfma");
+  return hipGetLastError() == hipSuccess ? 0 : -3;
 }

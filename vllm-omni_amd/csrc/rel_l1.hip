@@ -6,9 +6,14 @@
 // Which workgroup comes last depends on timing, what it computes does not: the tree depends only on
 // (B, n), so repeated calls give bit-identical sums.
 //
-// Scratch layout: kRelL1CounterBytes of ticket counters (one uint32 per row), then the partials
-// (B * nblk float pairs). The counters must be zero when the kernel starts; the last workgroup of every
-// row puts its counter back to zero, so scratch that was zeroed once stays usable.
+// Scratch layout: a counter region of fixed size (one 64-bit ticket word per row, room for the largest row
+// count the entry point accepts, so that no byte of it is ever used for anything else), then the partials
+// (B * nblk float pairs). A ticket word is (epoch << 16 | tickets drawn): every launch has an epoch larger
+// than any earlier one of the process, a workgroup first raises its row's word to (epoch << 16) with an
+// atomic maximum and then draws its ticket with an atomic add, so whatever an earlier launch left in the
+// word (one that never finished, say) is overridden. The last workgroup of a row puts the word back to zero
+// (a launch replayed from a HIP graph carries the same epoch every time). The region only has to be zero
+// ONCE, when the scratch is allocated.
 #include "odit_common.h"
 
 #include <mutex>
@@ -25,9 +30,10 @@ constexpr int kRelL1MaxRows = 65535;  // grid.y limit
 // rows of the no-allocation entry point, whose scratch is a fixed array in device memory
 constexpr int kRelL1StaticRows = 64;
 
-static inline size_t rel_l1_counter_bytes(int B) {
-  return (static_cast<size_t>(B) * sizeof(uint32_t) + 255) / 256 * 256;
-}
+// counter region of a caller's workspace: one word for each of the kRelL1MaxRows rows a call may have,
+// whatever B a particular call has (a region sized by B would let one call's partials be a later call's
+// counters)
+constexpr size_t kRelL1CounterBytes = (static_cast<size_t>(kRelL1MaxRows) + 1) * sizeof(uint64_t);
 
 static inline int rel_l1_blocks_per_row(int B, int64_t n) {
   // at least one pass of four 16-byte vectors per thread (sized on 8-element vectors; fp32 rows get twice the
@@ -45,7 +51,7 @@ static inline int rel_l1_blocks_per_row(int B, int64_t n) {
 
 template <typename T, bool REF_ROUND>
 __global__ __launch_bounds__(kRelL1Threads) void rel_l1_kernel(const T* __restrict__ cur, const T* __restrict__ prev,
-                                                     float* partials, uint32_t* counters,
+                                                     float* partials, uint64_t* counters, uint64_t epoch,
                                                      double* __restrict__ sums, int64_t n, int64_t n_vec,
                                                      int64_t cur_stride, int64_t prev_stride) {
   constexpr int EPV = Vec16<T>::N;
@@ -76,13 +82,13 @@ __global__ __launch_bounds__(kRelL1Threads) void rel_l1_kernel(const T* __restri
     Vec16<T> cv[U], pv[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      cv[u] = load16(c + (i + u * NT) * EPV);
-      pv[u] = load16(p + (i + u * NT) * EPV);
+      cv[u] = load16_stream(c + (i + u * NT) * EPV);
+      pv[u] = load16_stream(p + (i + u * NT) * EPV);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) accumulate(cv[u], pv[u]);
   }
-  for (; i < v_end; i += NT) accumulate(load16(c + i * EPV), load16(p + i * EPV));
+  for (; i < v_end; i += NT) accumulate(load16_stream(c + i * EPV), load16_stream(p + i * EPV));
   if (blockIdx.x == 0) {  // scalar tail (also the whole row when vector loads are not possible)
     for (int64_t i = n_vec * EPV + threadIdx.x; i < n; i += NT) {
       const float pf = to_float(p[i]);
@@ -111,9 +117,17 @@ __global__ __launch_bounds__(kRelL1Threads) void rel_l1_kernel(const T* __restri
     // invalidation of the whole L2 per workgroup: measured 25.3 us against 21.9 us.
     __hip_atomic_store(out, o0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __hip_atomic_store(out + 1, o1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // the compiler may move nothing across the wait: the stores stay above it, the ticket below
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
     __builtin_amdgcn_s_waitcnt(0);
-    const uint32_t ticket = __hip_atomic_fetch_add(counters + b, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    last_of_row = ticket == static_cast<uint32_t>(nblk) - 1u;
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    // the row's word is raised to this launch's epoch (a no-op for all but the row's first workgroup), then
+    // the ticket is drawn: two atomics of one thread on one address, applied in program order
+    const uint64_t base = epoch << 16;
+    __hip_atomic_fetch_max(counters + b, base, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint64_t ticket = __hip_atomic_fetch_add(counters + b, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    last_of_row = ticket == base + static_cast<uint64_t>(nblk) - 1u;
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);  // the reader's loads below stay below the ticket
   }
   __syncthreads();
   if (!last_of_row) return;  // uniform over the workgroup
@@ -140,19 +154,20 @@ __global__ __launch_bounds__(kRelL1Threads) void rel_l1_kernel(const T* __restri
     for (int w = 0; w < NWAVE; ++w) { t0 += red2[0][w]; t1 += red2[1][w]; }
     sums[2 * b] = t0;
     sums[2 * b + 1] = t1;
-    // hand the counter back at zero for the next call on this scratch
-    __hip_atomic_store(counters + b, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // back to zero: a launch recorded in a HIP graph is replayed with the same epoch, and finds its word as
+    // the first launch did
+    __hip_atomic_store(counters + b, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
-// Puts n ticket counters to zero (a kernel, not a memset: safe to record into a HIP graph).
-__global__ __launch_bounds__(256) void rel_l1_clear_kernel(uint32_t* counters, int n) {
+// Puts n ticket words to zero (a kernel, not a memset: safe to record into a HIP graph).
+__global__ __launch_bounds__(256) void rel_l1_clear_kernel(uint64_t* counters, int n) {
   const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i < n) counters[i] = 0u;
+  if (i < n) counters[i] = 0ull;
 }
 
 template <typename T>
-static int launch_rel_l1(const void* cur, const void* prev, double* sums, void* scratch, int B,
+static int launch_rel_l1(const void* cur, const void* prev, double* sums, uint64_t* counters, float* partials, int B,
                          int64_t n, int64_t cur_stride, int64_t prev_stride, bool ref_round,
                          hipStream_t stream) {
   constexpr int EPV = Vec16<T>::N;
@@ -160,28 +175,27 @@ static int launch_rel_l1(const void* cur, const void* prev, double* sums, void* 
                       prev_stride % EPV == 0;
   const int64_t n_vec = vec_ok ? n / EPV : 0;
   const int nblk = rel_l1_blocks_per_row(B, n);
-  uint32_t* counters = static_cast<uint32_t*>(scratch);
-  float* partials = reinterpret_cast<float*>(static_cast<char*>(scratch) + rel_l1_counter_bytes(B));
+  const uint64_t epoch = next_ticket_epoch();
   const dim3 grid(nblk, B);
   if (ref_round) {
     hipLaunchKernelGGL((rel_l1_kernel<T, true>), grid, dim3(kRelL1Threads), 0, stream, static_cast<const T*>(cur),
-                       static_cast<const T*>(prev), partials, counters, sums, n, n_vec, cur_stride, prev_stride);
+                       static_cast<const T*>(prev), partials, counters, epoch, sums, n, n_vec, cur_stride, prev_stride);
   } else {
     hipLaunchKernelGGL((rel_l1_kernel<T, false>), grid, dim3(kRelL1Threads), 0, stream, static_cast<const T*>(cur),
-                       static_cast<const T*>(prev), partials, counters, sums, n, n_vec, cur_stride, prev_stride);
+                       static_cast<const T*>(prev), partials, counters, epoch, sums, n, n_vec, cur_stride, prev_stride);
   }
   return check_launch("odit_rel_l1");
 }
 
-static size_t rel_l1_scratch_bytes(int B, int64_t n) {
-  return rel_l1_counter_bytes(B) + static_cast<size_t>(B) * rel_l1_blocks_per_row(B, n) * 2 * sizeof(float);
+static size_t rel_l1_partial_bytes(int B, int64_t n) {
+  return static_cast<size_t>(B) * rel_l1_blocks_per_row(B, n) * 2 * sizeof(float);
 }
 
 }  // namespace odit
 
 extern "C" size_t odit_rel_l1_workspace_bytes(int B, int64_t n) {
   if (B <= 0 || n < 0) return 0;
-  return odit::rel_l1_scratch_bytes(B, n);
+  return odit::kRelL1CounterBytes + odit::rel_l1_partial_bytes(B, n);
 }
 
 extern "C" int odit_rel_l1(const void* cur, const void* prev, double* sums, void* workspace,
@@ -198,8 +212,10 @@ extern "C" int odit_rel_l1(const void* cur, const void* prev, double* sums, void
     return ODIT_EWORKSPACE;
   }
   const bool rr = (flags & ODIT_FLAG_REF_ROUNDING) && dtype != ODIT_F32;
+  uint64_t* counters = static_cast<uint64_t*>(workspace);
+  float* partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + kRelL1CounterBytes);
   ODIT_DISPATCH_DTYPE(dtype, T,
-                      return launch_rel_l1<T>(cur, prev, sums, workspace, B, n, cur_stride, prev_stride, rr,
+                      return launch_rel_l1<T>(cur, prev, sums, counters, partials, B, n, cur_stride, prev_stride, rr,
                                               static_cast<hipStream_t>(stream)));
   return ODIT_OK;
 }
@@ -209,10 +225,11 @@ extern "C" int odit_rel_l1(const void* cur, const void* prev, double* sums, void
 // (one copy per GPU the library runs on, held until the process ends).
 namespace odit {
 
-// 256 bytes of counters + one float pair per workgroup: a launch over at most kRelL1StaticRows rows has at most
-// kRelL1TotalBlocks workgroups (rel_l1_blocks_per_row), so 2304 bytes hold any call this entry point accepts
-constexpr size_t kRelL1StaticBytes = 256 + static_cast<size_t>(kRelL1TotalBlocks) * 2 * sizeof(float);
-static_assert(kRelL1StaticRows * sizeof(uint32_t) <= 256, "the counters of the static rows fit their 256 bytes");
+// 512 bytes of ticket words + one float pair per workgroup: a launch over at most kRelL1StaticRows rows has at most
+// kRelL1TotalBlocks workgroups (rel_l1_blocks_per_row), so 2560 bytes hold any call this entry point accepts
+constexpr size_t kRelL1StaticCounterBytes = kRelL1StaticRows * sizeof(uint64_t);
+constexpr size_t kRelL1StaticBytes = kRelL1StaticCounterBytes + static_cast<size_t>(kRelL1TotalBlocks) * 2 * sizeof(float);
+static_assert(kRelL1StaticCounterBytes % 256 == 0, "the partials start on a 256-byte boundary");
 static_assert(kRelL1StaticRows <= kRelL1TotalBlocks, "one workgroup per row at least");
 
 static __device__ __align__(256) unsigned char scratch[kRelL1StaticBytes];
@@ -247,6 +264,13 @@ static void* static_scratch_ptr(int* status) {
 
 }  // namespace odit
 
+extern "C" void* odit_rel_l1_static_scratch(size_t* bytes) {
+  int rc = ODIT_OK;
+  void* ptr = odit::static_scratch_ptr(&rc);
+  if (bytes != nullptr) *bytes = ptr != nullptr ? odit::kRelL1StaticBytes : 0;
+  return ptr;
+}
+
 extern "C" int odit_rel_l1_static(const void* cur, const void* prev, double* sums, int B, int64_t n,
                                   int64_t cur_stride, int64_t prev_stride, int dtype, unsigned flags,
                                   void* stream) {
@@ -258,22 +282,24 @@ extern "C" int odit_rel_l1_static(const void* cur, const void* prev, double* sum
               "a workspace", B, kRelL1StaticRows);
     return ODIT_EWORKSPACE;
   }
-  if (rel_l1_scratch_bytes(B, n) > kRelL1StaticBytes) {  // cannot happen while the row limit holds; kept as the guard
-    set_error("odit_rel_l1_static: %zu bytes of scratch needed, %zu built in", rel_l1_scratch_bytes(B, n),
-              kRelL1StaticBytes);
+  if (kRelL1StaticCounterBytes + rel_l1_partial_bytes(B, n) > kRelL1StaticBytes) {  // cannot happen while the row limit holds
+    set_error("odit_rel_l1_static: %zu bytes of scratch needed, %zu built in",
+              kRelL1StaticCounterBytes + rel_l1_partial_bytes(B, n), kRelL1StaticBytes);
     return ODIT_EWORKSPACE;
   }
   int rc = ODIT_OK;
   void* ptr = static_scratch_ptr(&rc);
   if (ptr == nullptr) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  // The array keeps whatever the last call left (normally counters back at zero; not if that call's kernel never
-  // finished): clear this call's counters first. A fill kernel, not a memset, so the pair may be captured in a graph.
-  hipLaunchKernelGGL(rel_l1_clear_kernel, dim3(1), dim3(256), 0, st, static_cast<uint32_t*>(ptr), kRelL1StaticRows);
+  // The array keeps whatever the last call left (normally ticket words back at zero; not if that call's kernel
+  // never finished): clear this call's ticket words first. A fill kernel, not a memset, so the pair may be captured in a graph.
+  hipLaunchKernelGGL(rel_l1_clear_kernel, dim3(1), dim3(256), 0, st, static_cast<uint64_t*>(ptr), kRelL1StaticRows);
   rc = check_launch("odit_rel_l1_static (clear)");
   if (rc != ODIT_OK) return rc;
   const bool rr = (flags & ODIT_FLAG_REF_ROUNDING) && dtype != ODIT_F32;
+  uint64_t* counters = static_cast<uint64_t*>(ptr);
+  float* partials = reinterpret_cast<float*>(static_cast<char*>(ptr) + kRelL1StaticCounterBytes);
   ODIT_DISPATCH_DTYPE(dtype, T,
-                      return launch_rel_l1<T>(cur, prev, sums, ptr, B, n, cur_stride, prev_stride, rr, st));
+                      return launch_rel_l1<T>(cur, prev, sums, counters, partials, B, n, cur_stride, prev_stride, rr, st));
   return ODIT_OK;
 }

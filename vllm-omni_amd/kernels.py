@@ -23,6 +23,8 @@ from ._lib import (
     ODIT_F32,
     ODIT_FLAG_NEOX,
     ODIT_FLAG_REF_ROUNDING,
+    ODIT_LINEAR_HANDWRITTEN,
+    ODIT_LINEAR_LIBRARY,
     ODIT_NORM_HEAD,
     ODIT_NORM_NONE,
     ODIT_NORM_ROW,
@@ -509,7 +511,7 @@ def rel_l1_sums(cur: torch.Tensor, prev: torch.Tensor, *, ref_rounding: bool = T
     key = (cur.device.index or 0, _stream())  # launches on one stream are ordered and can share it
     ws = _REL_L1_SCRATCH.get(key)
     if ws is None or ws.numel() < need:
-        # zeroed once: the kernel needs its ticket counters at zero and hands them back at zero
+        # zero-filled once: the ticket words live in a region of fixed size at the start
         ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=cur.device)
         _REL_L1_SCRATCH[key] = ws
     sums = torch.empty((B, 2), dtype=torch.float64, device=cur.device)
@@ -575,17 +577,20 @@ def set_linear_autotune(iters: int) -> None:
         _FLUSH.clear()
 
 
-_LINEAR_ENGINES = {"auto": 0, "library": 1, "handwritten": 2}
+_LINEAR_ENGINES = {"auto": 0, "library": ODIT_LINEAR_LIBRARY, "handwritten": ODIT_LINEAR_HANDWRITTEN}
+_LINEAR_ENGINE_FLAGS = 0
 
 
 def set_linear_engine(engine: str) -> None:
-    """Which kernel ``linear`` runs, process-wide: "auto" (the hand-written stream-K kernel where a tuning
-    run found it faster or, untuned, where K >= 2 N and it takes the problem; the library elsewhere),
-    "library" (hipBLASLt always) or "handwritten" (the stream-K kernel always; problems it does not take
-    raise). For measurements and tests."""
+    """Which kernel later ``linear`` calls of this process ask for when they name none themselves: "auto" (a
+    hand-written kernel where a tuning run found it faster or its default rule says so, the library
+    elsewhere), "library" (hipBLASLt always) or "handwritten" (the hand-written kernel for the row count
+    always; problems it does not take raise). The choice travels with every call as a flag of
+    ``odit_linear_rows``; the library keeps no switch. For measurements and tests."""
+    global _LINEAR_ENGINE_FLAGS
     if engine not in _LINEAR_ENGINES:
         raise ValueError(f"engine must be one of {sorted(_LINEAR_ENGINES)}")
-    _lib.check(_lib.load().odit_linear_set_engine(_LINEAR_ENGINES[engine]), "odit_linear_set_engine")
+    _LINEAR_ENGINE_FLAGS = _LINEAR_ENGINES[engine]
 
 
 def linear_tuning_report() -> dict[tuple, float]:
@@ -597,7 +602,7 @@ def _linear_workspace(lib, device: torch.device) -> torch.Tensor:
     key = (device.index or 0, _stream())
     ws = _LINEAR_SCRATCH.get(key)
     if ws is None:
-        # zero-filled: the hand-written kernel keeps tile counters at the start, zero between calls
+        # zero-filled once: the stream-K kernel keeps its ticket words at the start
         ws = torch.zeros(int(lib.odit_linear_workspace_bytes()), dtype=torch.uint8, device=device)
         _LINEAR_SCRATCH[key] = ws
     return ws
@@ -616,7 +621,7 @@ def _rows2d(t: torch.Tensor, name: str) -> tuple[torch.Tensor, int]:
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *, activation: str | None = None,
            residual: torch.Tensor | None = None, gate: torch.Tensor | None = None, out: torch.Tensor | None = None,
            gate_bias: torch.Tensor | None = None, prescaled: bool = False, tune_iters: int = 0,
-           plan_only: bool = False):
+           plan_only: bool = False, engine: str | None = None):
     """x W^T (+ bias) with the elementwise tail inside the GEMM's epilogue.
 
     activation="gelu_tanh": GELU(tanh) of the result. residual (same shape as the result) with optional
@@ -627,8 +632,12 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
     ``tune_iters`` > 0 first times the library's kernels and the hand-written kernel for this problem
     (overwrites ``out``), keeps the faster for later calls and returns its time in microseconds instead
     of the result. ``plan_only`` launches nothing and returns (the hand-written kernel would run, number of
-    kernel launches the call would make).
+    kernel launches the call would make). ``engine``: "auto", "library" or "handwritten" for this call
+    (default: what ``set_linear_engine`` chose).
     """
+    if engine is not None and engine not in _LINEAR_ENGINES:
+        raise ValueError(f"engine must be one of {sorted(_LINEAR_ENGINES)}")
+    eflags = _LINEAR_ENGINE_FLAGS if engine is None else _LINEAR_ENGINES[engine]
     _dev(x, weight, bias, residual, gate, out)
     if weight.dim() != 2 or weight.stride(1) != 1 or x.shape[-1] != weight.shape[1]:
         raise ValueError(f"weight must be [N,K] rows with K = {x.shape[-1]}, got {tuple(weight.shape)}")
@@ -658,7 +667,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
                 None if rp is None else rp + row0 * ldr * esz, gp, M, N, K, ldx, ldw, ldo, ldr, epi, gate_code,
                 _code(x), rows_per_gate, gate_stride)
         if plan_only:
-            _lib.check(lib.odit_linear_rows_plan(*prob, ws.data_ptr(), ws.numel(), _lib.C.byref(plan[0]),
+            _lib.check(lib.odit_linear_rows_plan(*prob, eflags, ws.data_ptr(), ws.numel(), _lib.C.byref(plan[0]),
                                                  _lib.C.byref(plan[1])), "odit_linear_rows_plan")
             return
         if _LINEAR_AUTOTUNE_ITERS > 0 and tune_iters == 0:
@@ -673,14 +682,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
                 t_prob = prob[:3] + (t_out.data_ptr(), _ptr(t_res)) + prob[5:]
                 _lib.check(lib.odit_linear_rows_tune(*t_prob, ws.data_ptr(), ws.numel(), _stream(),
                                                      _LINEAR_AUTOTUNE_ITERS, _flush_buffer(x.device), _FLUSH_BYTES,
-                                                     _lib.C.byref(t_best)), "odit_linear_rows_tune")
+                                                     _lib.C.byref(t_best), None), "odit_linear_rows_tune")
                 _LINEAR_TUNED[key] = t_best.value
         if tune_iters > 0:
             _lib.check(lib.odit_linear_rows_tune(*prob, ws.data_ptr(), ws.numel(), _stream(), int(tune_iters),
-                                                 _flush_buffer(x.device), _FLUSH_BYTES, _lib.C.byref(best)),
+                                                 _flush_buffer(x.device), _FLUSH_BYTES, _lib.C.byref(best), None),
                        "odit_linear_rows_tune")
         else:
-            _lib.check(lib.odit_linear_rows(*prob, ws.data_ptr(), ws.numel(), _stream()), "odit_linear_rows")
+            _lib.check(lib.odit_linear_rows(*prob, eflags, ws.data_ptr(), ws.numel(), _stream()), "odit_linear_rows")
 
     ldr = 0
     if residual is None:

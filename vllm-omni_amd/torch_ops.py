@@ -93,6 +93,6 @@ def attention_forward_hip(self, query: torch.Tensor, key: torch.Tensor, value: t
     mask is handed to the kernel as it is: testing it for all-true would need a device-to-host copy,
     which a traced region cannot hold."""
     mask = getattr(attn_metadata, "attn_mask", None) if attn_metadata is not None else None
-    if mask is not None and mask.dim() != 2:
-        raise ValueError("the HIP attention backend takes a [B,Sk] key-padding mask")
+    if not self.kernel_takes_layer or not self.kernel_takes_mask(mask, query.shape[0], key.shape[1]):
+        return self.sdpa.forward_hip(query, key, value, attn_metadata)  # torch's own op: traceable as it is
     return torch.ops.omni_dit.attention(query, key, value, float(self.softmax_scale), mask)
