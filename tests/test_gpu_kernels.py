@@ -771,6 +771,52 @@ def test_attention_key_split_tail(gpu, shape):
     _close(lsep, torch.logsumexp(sp, dim=-1).float(), atol=2e-2, rtol=1e-3, what="key-split, peaked logits, lse")
 
 
+_PERSISTENT_CHILD = """
+import sys, torch
+from vllm_omni_amd import kernels
+d = torch.load(sys.argv[1])
+q, k, v, m = (d[n].cuda() for n in ("q", "k", "v", "m"))
+assert "persistent workgroups" in kernels.attn_plan(q.shape[0], q.shape[1], k.shape[1], q.shape[2], q.shape[3])
+out = {}
+for rep in range(3):            # the ticket words are back at zero after every launch
+    out[f"plain{rep}"], out[f"lse{rep}"] = (t.cpu() for t in kernels.attn_fwd(q, k, v, d["scale"], return_lse=True))
+out["masked"] = kernels.attn_fwd(q, k, v, d["scale"], key_mask=m).cpu()
+torch.save(out, sys.argv[2])
+"""
+
+
+def test_attention_persistent_form_matches_the_default_form(gpu, tmp_path):
+    """The measurement mode ODIT_ATTN_PERSISTENT=1 (resident workgroups that draw unit after unit from ticket words
+    in the scratch) gives the default form's results bit for bit, also on repeated launches over the same ticket
+    words, with a key mask, and with a last round that is cut along the keys. The variable is read once per
+    process, so the persistent form runs in a child process."""
+    import os
+    import subprocess
+    import sys
+
+    from vllm_omni_amd import kernels
+
+    B, Sq, S, H, D = 2, 2816, 1408, 24, 128  # 22 query blocks x 48 = 1056 units on 512 slots (two rounds + 32), 22 key tiles
+    q, k, v = _attn_inputs(B, Sq, S, H, H, D, seed=91)
+    m = torch.rand(B, S, generator=torch.Generator().manual_seed(3)) > 0.2
+    scale = 1.0 / math.sqrt(D)
+    plan = kernels.attn_plan(B, Sq, S, H, D)
+    assert "persistent" not in plan and "attn_merge_kernel" in plan
+    want, want_lse = kernels.attn_fwd(q.to(gpu), k.to(gpu), v.to(gpu), scale, return_lse=True)
+    want_m = kernels.attn_fwd(q.to(gpu), k.to(gpu), v.to(gpu), scale, key_mask=m.to(gpu))
+    torch.save({"q": q, "k": k, "v": v, "m": m, "scale": scale}, tmp_path / "in.pt")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, ODIT_ATTN_PERSISTENT="1", PYTHONPATH=root + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    proc = subprocess.run([sys.executable, "-c", _PERSISTENT_CHILD, str(tmp_path / "in.pt"), str(tmp_path / "out.pt")],
+                          env=env, capture_output=True, text=True, timeout=100)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got = torch.load(tmp_path / "out.pt")
+    for rep in range(3):
+        assert torch.equal(got[f"plain{rep}"], want.cpu()), rep
+        assert torch.equal(got[f"lse{rep}"], want_lse.cpu()), rep
+    assert torch.equal(got["masked"], want_m.cpu())
+
+
 @pytest.mark.parametrize("shape,cut", [((2, 300, 300, 4, 4, 128), 64), ((1, 1100, 1100, 3, 3, 64), 256),
                                        ((2, 130, 2048, 4, 2, 128), 1024), ((1, 300, 1100, 3, 3, 128), 192),
                                        ((2, 200, 200, 2, 2, 128), 70)])

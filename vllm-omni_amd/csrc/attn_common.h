@@ -56,7 +56,14 @@ struct AttnParams {
   // workgroup per range, which leave unnormalised partial results in `ws` for the merge kernel
   int n_full, key_chunks, tiles_per_chunk;
   float* ws;
+  // persistent form (attn_fwd_dma.hip): one ticket word per XCD, 64 bytes apart, from which its workgroups draw
+  // their next unit: (epoch << 24 | tickets drawn), zero between launches; epoch = number of this launch,
+  // larger than that of any earlier launch of the process
+  unsigned long long* queue;
+  unsigned long long epoch;
 };
+
+constexpr size_t kAttnQueueBytes = 1024;  // head of the workspace: the ticket words of the persistent form
 
 // address of output row `row` of (batch b, head h): head of the joint sequence in `o`, tail in `o_tail`
 template <typename T>
@@ -87,8 +94,8 @@ int launch_attn_dma(AttnParams& p, int dtype, int D, hipStream_t stream, void* w
 size_t attn_dma_workspace_bytes(int B, int Sq, int Sk, int H, int D);
 
 
-// whether launch_attn_dma takes a problem with these key/value row strides (elements)
-bool attn_dma_addressable(int Sk, int64_t k_seq_stride, int64_t v_seq_stride);
+// whether launch_attn_dma takes a problem of head size D with these key/value row strides (elements)
+bool attn_dma_addressable(int Sk, int D, int64_t k_seq_stride, int64_t v_seq_stride);
 
 // text description of the launches launch_attn_dma makes for a shape; returns their number
 int attn_dma_plan(int B, int Sq, int Sk, int H, int D, bool with_workspace, char* text, size_t text_bytes);

@@ -340,7 +340,7 @@ extern "C" int odit_attn_fwd_plan(int B, int Sq, int Sk, int H, int D, int64_t k
   using namespace odit;
   ODIT_CHECK_ARG(text != nullptr && text_bytes > 0, "odit_attn_fwd_plan: no text buffer");
   ODIT_CHECK_ARG(B > 0 && Sq > 0 && Sk > 0 && H > 0 && (D == 64 || D == 128), "odit_attn_fwd_plan: bad shape");
-  if (attn_dma_addressable(Sk, k_seq_stride, v_seq_stride))
+  if (attn_dma_addressable(Sk, D, k_seq_stride, v_seq_stride))
     return attn_dma_plan(B, Sq, Sk, H, D, with_workspace != 0, text, text_bytes);
   const int64_t units = static_cast<int64_t>((Sq + 255) / 256) * H * B;
   snprintf(text, text_bytes, "attn_fwd_pipe_kernel<T, %d, 8> units=%lld", D, static_cast<long long>(units));

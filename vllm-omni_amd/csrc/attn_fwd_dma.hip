@@ -18,6 +18,32 @@
 // Everything else (transposed S^T = K Q^T / O^T = V^T P^T formulation, one query per lane, lazy
 // rescale, stage A = next-tile QK^T MFMAs interleaved with this tile's exp2 work, stage B = PV, one
 // barrier per tile, XCD-aware workgroup order) is as in attn_fwd_pipe_kernel.
+//
+// Persistent form (MODE 2), a measurement aid that no default launch uses (ODIT_ATTN_PERSISTENT=1 in the
+// environment turns it on). With more units than workgroup slots the launch has as many workgroups as run at
+// once, and each runs unit after unit as ONE stream of key tiles: the tile pipeline runs across the unit
+// boundary. Units are handed out dynamically: every XCD owns a contiguous eighth of the units (neighbours in
+// (q block, head) order share keys and values in its L2), its workgroups start on the first ones and draw the
+// next from the XCD's ticket word in scratch whenever they begin a unit, one unit ahead of need, so the draw's
+// latency hides behind that unit's first tile. While a unit's last tiles are multiplied, the K and V tiles of
+// the next unit's first keys are already on their way into LDS; the last tile's stage A computes the next
+// unit's first scores from that unit's queries (fetched a tile earlier into the fragment registers the finished
+// unit no longer needs); after the last tile's stage B the finished unit is normalised and stored and the
+// running maximum, sum and accumulators start again. A unit then costs its key tiles and one fetch of its
+// queries, not a workgroup dispatch, a cold prologue and a drained pipeline at its end.
+// What it measured (bf16, D = 128, us, one workgroup per unit / persistent, same process, same box):
+//   B=2 S=4352 H=24 (3.19 rounds)  506 / 532      B=2 S=4096 H=24 (3.00 rounds)  433 / 447
+//   B=1 S=4608 H=24 (1.69 rounds)  306 / 316      B=2 S=32760 H=40 (40 rounds)   39709 / 41187
+// i.e. 3 to 5 % slower everywhere, also at 40 units per workgroup where the boundaries no longer matter: the
+// steady-state tile loop itself is slower (it carries the next unit's state and the boundary's branches, and
+// needs all 256 vector registers where MODE 0 needs 235), and that costs more than the boundaries save. With a
+// fixed assignment of units (w, w + W, ...) instead of the ticket words it was 6 % slower: compute units do
+// not all run at one speed, and the dispatcher (or the tickets) gives the faster ones more work. Neither form
+// removes the cost of a last round that is partly filled: that needs units cut along the keys (MODE 1).
+#include <stddef.h>
+
+#include <cstdlib>
+
 #include "attn_common.h"
 #include "attn_tail.h"
 
@@ -32,18 +58,32 @@
 
 namespace odit {
 
+// A kernel argument fetched again from the argument segment at the point of use (a scalar load the compiler can
+// neither hoist nor merge with others). The persistent form reads what it needs at a unit boundary this way:
+// taken from the by-value argument struct, those fields would be held in scalar registers across the whole tile
+// loop, which has none to spare.
+template <typename V> __device__ __forceinline__ V kernel_arg(size_t offset) {
+  typedef __attribute__((address_space(4))) const char* arg_ptr;
+  arg_ptr base = (arg_ptr)__builtin_amdgcn_kernarg_segment_ptr();
+  return *(const volatile __attribute__((address_space(4))) V*)(base + offset);
+}
+#define ODIT_ARG(field) (PERSIST ? kernel_arg<decltype(AttnParams::field)>(offsetof(AttnParams, field)) : p.field)
+
 typedef short s16x4_d __attribute__((ext_vector_type(4)));
 typedef short s16x8_d __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) s16x4_d* lds_s16x4_p;
 typedef __attribute__((address_space(3))) void* lds_void_p;
 
-// TAIL = false: workgroup i owns unit i (a q block of one head of one batch row), all keys.
-// TAIL = true:  launched after the full rounds for the units that are left over: workgroup i owns key
-//               tiles [jt0, n_tiles) of unit n_full + i / key_chunks and leaves an unnormalised partial
-//               result in scratch for attn_merge_kernel. A separate instantiation, so the extra
-//               bookkeeping cannot disturb the register allocation of the main kernel.
-template <typename T, int D, int NW, bool TAIL>
+// MODE 0: workgroup i owns unit i (a q block of one head of one batch row), all keys.
+// MODE 1: launched after the full rounds for the units that are left over: workgroup i owns key
+//         tiles [jt0, n_tiles) of unit n_full + i / key_chunks and leaves an unnormalised partial
+//         result in scratch for attn_merge_kernel.
+// MODE 2: persistent, see above.
+// Separate instantiations, so the extra bookkeeping of one cannot disturb the register allocation of another.
+template <typename T, int D, int NW, int MODE>
 __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const AttnParams p) {
+  constexpr bool TAIL = MODE == 1;
+  constexpr bool PERSIST = MODE == 2;
   using M = Mma<T>;
   using frag = typename M::frag;
   constexpr int BN = 64;
@@ -61,30 +101,36 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   __shared__ __attribute__((aligned(1024))) char lds[4 * TILEB];  // K0 K1 V0 V1
   char* const Kb = lds;
   char* const Vb = lds + 2 * TILEB;
+  constexpr int kKoff = 0, kVoff = 2 * TILEB;  // the same as byte offsets, for the tile loads' LDS destinations
 
   const int n_tiles_all = (p.Sk + BN - 1) / BN;
   int pid, jt0 = 0, n_tiles = n_tiles_all;
   const int part = blockIdx.x;
-  if constexpr (!TAIL) {
+  // persistent form: the unit after the current one (-1: none, or not drawn yet)
+  int next_pid = -1;
+  __shared__ int next_unit_box;  // thread 0's draw, handed to the workgroup across a tile's barrier
+  if constexpr (MODE == 0) {
     pid = xcd_remap(blockIdx.x, p.n_full);
-  } else {  // this workgroup covers key tiles [jt0, n_tiles) of unit pid (jt0 is even)
+  } else if constexpr (TAIL) {  // this workgroup covers key tiles [jt0, n_tiles) of unit pid (jt0 is even)
     pid = p.n_full + part / p.key_chunks;
     jt0 = (part % p.key_chunks) * p.tiles_per_chunk;
     n_tiles = jt0 + p.tiles_per_chunk < n_tiles_all ? jt0 + p.tiles_per_chunk : n_tiles_all;
+  } else {
+    // gridDim.x = W workgroups, a multiple of the XCD count, all resident; hardware puts workgroup w on XCD
+    // w % 8. XCD x owns units [x_lo, x_hi); its W / 8 workgroups start on the first W / 8 of them.
+    const int xcd = part % kNumXcd;
+    const int x_lo = static_cast<int>(static_cast<int64_t>(p.n_full) * xcd / kNumXcd);
+    const int x_hi = static_cast<int>(static_cast<int64_t>(p.n_full) * (xcd + 1) / kNumXcd);
+    pid = x_lo + part / kNumXcd;
+    if (pid >= x_hi) return;  // fewer units than workgroups on this XCD (before any barrier: the whole workgroup leaves)
   }
-  const int qb = pid % p.n_qblocks;
-  const int bh = pid / p.n_qblocks;
-  const int h = bh % p.H;
-  const int b = bh / p.H;
-  const int hkv = h / (p.H / p.Hkv);
-
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hh = lane >> 5;
-  const int q0 = qb * BM + wave * 32;
 
-  const T* qbase = static_cast<const T*>(p.q) + b * p.qs_b + h * p.qs_h;
-  const T* kbase = static_cast<const T*>(p.k) + b * p.ks_b + hkv * p.ks_h;
-  const T* vbase = static_cast<const T*>(p.v) + b * p.vs_b + hkv * p.vs_h;
+  // ---- the current unit (fixed for MODE 0 and 1, advanced unit by unit in the persistent form) ----
+  int h = (pid / p.n_qblocks) % p.H;
+  int b = (pid / p.n_qblocks) / p.H;
+  int q0 = (pid % p.n_qblocks) * BM + wave * 32;
 
   // buffer descriptors end right after the last valid key row: later rows read as zeros
   const uint32_t k_bytes = static_cast<uint32_t>(((p.Sk - 1) * p.ks_s + D) * 2);
@@ -93,6 +139,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   const int v_split_tiles = p.v_tail != nullptr ? p.k_split / BN : n_tiles_all;
   const int v_rows = p.v_tail != nullptr ? p.k_split : p.Sk;
   const uint32_t v_bytes = static_cast<uint32_t>(((v_rows - 1) * p.vs_s + D) * 2);
+  const uint32_t v2_bytes = p.v_tail != nullptr ? static_cast<uint32_t>(((p.Sk - p.k_split - 1) * p.vs_s + D) * 2) : v_bytes;
   // raw buffer descriptors {base[31:0], base[47:32] (stride 0), bytes, dword3 = 0x00020000}
   auto make_rsrc = [](const void* base, uint32_t bytes) {
     const uint64_t a = reinterpret_cast<uint64_t>(base);
@@ -100,23 +147,66 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
     r.x = static_cast<uint32_t>(a); r.y = static_cast<uint32_t>(a >> 32) & 0xffffu; r.z = bytes; r.w = 0x00020000u;
     return r;
   };
-  const u32x4_v krsrc = make_rsrc(kbase, k_bytes);
-  const u32x4_v vrsrc = make_rsrc(vbase, v_bytes);
-  u32x4_v vrsrc2 = vrsrc;
-  if (p.v_tail != nullptr) {
-    const T* vbase2 = static_cast<const T*>(p.v_tail) + b * p.vt_b + hkv * p.vt_h;
-    vrsrc2 = make_rsrc(vbase2, static_cast<uint32_t>(((p.Sk - p.k_split - 1) * p.vs_s + D) * 2));
-  }
+  // descriptors of the keys / values / second value tensor of (batch b_, head h_)
+  auto k_rsrc_of = [&](int b_, int h_) {
+    const int hkv_ = h_ / (ODIT_ARG(H) / ODIT_ARG(Hkv));
+    return make_rsrc(static_cast<const T*>(ODIT_ARG(k)) + b_ * ODIT_ARG(ks_b) + hkv_ * ODIT_ARG(ks_h), k_bytes);
+  };
+  auto v_rsrc_of = [&](int b_, int h_) {
+    const int hkv_ = h_ / (ODIT_ARG(H) / ODIT_ARG(Hkv));
+    return make_rsrc(static_cast<const T*>(ODIT_ARG(v)) + b_ * ODIT_ARG(vs_b) + hkv_ * ODIT_ARG(vs_h), v_bytes);
+  };
+  auto v2_rsrc_of = [&](int b_, int h_) {
+    const int hkv_ = h_ / (ODIT_ARG(H) / ODIT_ARG(Hkv));
+    return make_rsrc(static_cast<const T*>(ODIT_ARG(v_tail)) + b_ * ODIT_ARG(vt_b) + hkv_ * ODIT_ARG(vt_h), v2_bytes);
+  };
+  u32x4_v krsrc = k_rsrc_of(b, h);
+  u32x4_v vrsrc = v_rsrc_of(b, h);
+  u32x4_v vrsrc2 = p.v_tail != nullptr ? v2_rsrc_of(b, h) : vrsrc;
+  const uint8_t* mrow = p.mask ? p.mask + static_cast<int64_t>(b) * p.Sk : nullptr;
+  // persistent form: where the next unit is (valid while next_pid >= 0)
+  int n_h = 0, n_b = 0;
+  // Thread 0 draws the unit after the current one: the XCD's word is raised to this launch's epoch (a no-op but
+  // for the XCD's first draw of the launch), then ticket t names unit x_first + t. Every unit that is run draws
+  // once, so the draw with the ticket of the XCD's last unit is the launch's last on this word and puts it back
+  // to zero (a launch replayed from a HIP graph carries the same epoch).
+  auto draw_next = [&]() {
+    if (tid == 0) {
+      // the XCD's unit range, worked out again here rather than held in scalar registers for the whole unit
+      int xcd = part % kNumXcd;
+      asm volatile("" : "+s"(xcd));  // (so that the word's address is formed here, not held in vector registers)
+      const int per = static_cast<int>(gridDim.x) / kNumXcd;
+      const int x_lo = static_cast<int>(static_cast<int64_t>(p.n_full) * xcd / kNumXcd);
+      const int x_hi = static_cast<int>(static_cast<int64_t>(p.n_full) * (xcd + 1) / kNumXcd);
+      const int x_first = x_lo + per < x_hi ? x_lo + per : x_hi;  // first unit handed out by ticket
+      unsigned long long* word = ODIT_ARG(queue) + xcd * 8;
+      __hip_atomic_fetch_max(word, ODIT_ARG(epoch) << 24, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned t = static_cast<unsigned>(__hip_atomic_fetch_add(word, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) & 0xffffffu;
+      if (static_cast<int>(t) == x_hi - x_lo - 1) __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int cand = x_first + static_cast<int>(t);
+      next_unit_box = cand < x_hi ? cand : -1;
+    }
+  };
+  auto take_next = [&]() {  // behind the barrier that follows draw_next
+    next_pid = __builtin_amdgcn_readfirstlane(next_unit_box);
+    if (next_pid >= 0) {
+      const int bh = next_pid / ODIT_ARG(n_qblocks), heads = ODIT_ARG(H);
+      n_h = bh % heads;
+      n_b = bh / heads;
+    }
+  };
 
-  // per-lane global byte offsets of the chunks this lane moves, relative to the tile's first row
-  uint32_t kvoff[IPW], vvoff[IPW];
-#pragma unroll
-  for (int i = 0; i < IPW; ++i) {
-    const int r = (wave * IPW + i) * RPI + lane / CPR;  // tile row
-    const int pc = lane % CPR;
-    kvoff[i] = static_cast<uint32_t>(r * p.ks_s * 2) + static_cast<uint32_t>(((pc ^ (r % 16)) % CPR) * 16);
-    vvoff[i] = static_cast<uint32_t>(r * p.vs_s * 2) + static_cast<uint32_t>(((pc ^ (4 * (r % 4))) % CPR) * 16);
-  }
+  // Per-lane global byte offset of the chunk this lane moves with its wave's FIRST instruction of a tile,
+  // relative to the tile's first row; instruction i moves the rows RPI * i further down, which is a scalar
+  // term (it goes into the load's scalar offset), and its swizzle differs from the first one's by a constant:
+  // for K, row % 16 = (row0 % 16) + (RPI * i) % 16 without a carry (row0 % 16 < RPI), so the chunk index is that
+  // of instruction 0 XOR ((RPI * i) % 16 % CPR) - for V (4 * (row % 4), RPI a multiple of 4) it is the same. The
+  // XOR is done on the byte offset, which needs row strides that are multiples of the row's own 2 D bytes.
+  const int r0 = wave * IPW * RPI + lane / CPR, pc0 = lane % CPR;
+  const uint32_t kvoff0 = static_cast<uint32_t>(r0 * p.ks_s * 2) + static_cast<uint32_t>(((pc0 ^ (r0 % 16)) % CPR) * 16);
+  const uint32_t vvoff0 = static_cast<uint32_t>(r0 * p.vs_s * 2) + static_cast<uint32_t>(((pc0 ^ (4 * (r0 % 4))) % CPR) * 16);
+  const uint32_t k_inst_step = static_cast<uint32_t>(RPI * p.ks_s * 2);
+  const uint32_t v_inst_step = static_cast<uint32_t>(RPI * p.vs_s * 2);
   const uint32_t k_tile_step = static_cast<uint32_t>(BN * p.ks_s * 2);
   const uint32_t v_tile_step = static_cast<uint32_t>(BN * p.vs_s * 2);
 
@@ -126,40 +216,70 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   // being filled): the loads issued at the top of a tile, meant to land a whole tile later, were waited
   // for half a tile after issue. Here the ordering is explicit instead: one `s_waitcnt vmcnt(0)` and one
   // barrier at the end of each tile, before any wave reads the buffers those loads filled.
-  auto dma_tile = [&](const u32x4_v& rsrc, const uint32_t(&voff)[IPW], uint32_t soff, char* dst) {
+  // `dst_off` is the tile's byte offset inside the kernel's LDS block: a literal at every call
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_p)lds));
+  auto dma_tile = [&](const u32x4_v& rsrc, const bool is_k, uint32_t soff, const int dst_off) {
 #if defined(__HIP_DEVICE_COMPILE__)
-    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_p)(dst + wave * IPW * 1024)));
+    const uint32_t lds0 = lds_base + static_cast<uint32_t>(dst_off) + static_cast<uint32_t>(wave * IPW * 1024);
+    // (the empty asm makes the offset opaque here: otherwise the compiler forms the IPW swizzled offsets once,
+    // outside the tile loop, and holds them in registers the loop does not have)
+    uint32_t voff0 = is_k ? kvoff0 : vvoff0;
+    asm volatile("" : "+v"(voff0));
 #pragma unroll
     for (int i = 0; i < IPW; ++i) {
       const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds0 + i * 1024);
+      const uint32_t voff_i = is_k ? (voff0 ^ static_cast<uint32_t>((((RPI * i) % 16) % CPR) * 16)) : voff0;
+      const uint32_t soff_i = soff + static_cast<uint32_t>(i) * (is_k ? k_inst_step : v_inst_step);
       // m0 (the LDS destination of the load) is a reserved register: naming it as clobbered draws a
       // warning per expansion, and leaving it out would hide the write from the compiler
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                    :
-                   : "s"(m0v), "v"(voff[i]), "s"(rsrc), "s"(soff)
+                   : "s"(m0v), "v"(voff_i), "s"(rsrc), "s"(soff_i)
                    : "memory", "m0");
 #pragma clang diagnostic pop
     }
 #endif
   };
 
-  auto dma_v = [&](int jt, char* dst) {
+  auto dma_v = [&](int jt, const int dst) {
     const bool second = jt >= v_split_tiles;
-    dma_tile(second ? vrsrc2 : vrsrc, vvoff, static_cast<uint32_t>(second ? jt - v_split_tiles : jt) * v_tile_step, dst);
+    dma_tile(second ? vrsrc2 : vrsrc, false, static_cast<uint32_t>(second ? jt - v_split_tiles : jt) * v_tile_step, dst);
+  };
+  // the same for tiles of the NEXT unit (persistent form): descriptors made on the spot from (n_b, n_h), a few
+  // scalar instructions per tile instead of a dozen scalar registers held for the whole unit
+  auto dma_k_next = [&](int jt, const int dst) {
+    dma_tile(k_rsrc_of(n_b, n_h), true, static_cast<uint32_t>(jt) * k_tile_step, dst);
+  };
+  auto dma_v_next = [&](int jt, const int dst) {
+    const bool second = jt >= v_split_tiles;
+    dma_tile(second ? v2_rsrc_of(n_b, n_h) : v_rsrc_of(n_b, n_h), false,
+             static_cast<uint32_t>(second ? jt - v_split_tiles : jt) * v_tile_step, dst);
   };
 
   // ---- Q fragments stay in registers ----
   frag qf[KS];
-  {
-    int row = q0 + l32;
-    row = row < p.Sq ? row : p.Sq - 1;
-    const T* qp = qbase + row * p.qs_s + hh * 8;
+  // (the persistent form calls these two inside the tile loop: they take the lane's position from the thread
+  // index again, so that nothing of theirs is carried through the loop)
+  auto lane_again = [&](int& l32_, int& hh_) {
+    int t = tid;
+    if constexpr (PERSIST) asm volatile("" : "+v"(t));
+    l32_ = t & 31;
+    hh_ = (t >> 5) & 1;
+  };
+  auto load_q = [&](int b_, int h_, int q0_) {
+    int l32, hh;
+    lane_again(l32, hh);
+    int row = q0_ + l32;
+    const int rows = ODIT_ARG(Sq);
+    row = row < rows ? row : rows - 1;
+    const T* qp = static_cast<const T*>(ODIT_ARG(q)) + b_ * ODIT_ARG(qs_b) + h_ * ODIT_ARG(qs_h) + row * ODIT_ARG(qs_s) + hh * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
       qf[ks] = __builtin_bit_cast(frag, *reinterpret_cast<const u32x4_v*>(qp + ks * 16));
-  }
+  };
+  load_q(b, h, q0);
 
   f32x16_v o[DT];
 #pragma unroll
@@ -169,7 +289,6 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   float m_run = -INFINITY, l_run = 0.f;
 
   const float c = p.scale_log2;
-  const uint8_t* mrow = p.mask ? p.mask + static_cast<int64_t>(b) * p.Sk : nullptr;
 
   // K fragment (kt, ks): row kt*32 + l32, logical chunk 2*ks + hh  ->  chunk (2*ks) ^ (hh ^ l32 % 16)
   const int k_lane = l32 * ROWB + ((((hh ^ (l32 % 16)) % CPR)) << 4);
@@ -195,7 +314,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
       }
   };
 
-  auto mask_and_max = [&](int j, f32x16_v(&s)[2]) -> float {
+  auto mask_and_max = [&](int j, const uint8_t* mrow, f32x16_v(&s)[2]) -> float {
     // branch-free selects: every lane rewrites all its scores, excluded ones with -inf
     if (mrow != nullptr) {
 #pragma unroll
@@ -245,14 +364,72 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
     }
   };
 
-  auto tile = [&](int j, f32x16_v(&s_cur)[2], f32x16_v(&s_next)[2]) {
-    const int buf = j & 1;
-    const bool has_next = j + 1 < n_tiles;
+  // normalises and stores the finished unit (b, h, q0): the tail of MODE 0 and of every unit of the persistent form
+  auto finish_unit = [&]() {
+    int l32, hh;
+    lane_again(l32, hh);
+    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    const int row = q0 + l32;
+    if (row < ODIT_ARG(Sq)) {
+      // head of the joint sequence in `o`, tail in `o_tail` (out_row_ptr, with the arguments fetched here)
+      T* op;
+      void* const o_tail = ODIT_ARG(o_tail);
+      const int q_split = ODIT_ARG(q_split);
+      if (o_tail != nullptr && row >= q_split) {
+        op = static_cast<T*>(o_tail) + b * ODIT_ARG(ts_b) + h * ODIT_ARG(ts_h) + static_cast<int64_t>(row - q_split) * ODIT_ARG(ts_s);
+      } else {
+        op = static_cast<T*>(ODIT_ARG(o)) + b * ODIT_ARG(os_b) + h * ODIT_ARG(os_h) + static_cast<int64_t>(row) * ODIT_ARG(os_s);
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          u32x2_v w;
+          w.x = M::pack2(o[dt][g * 4 + 0] * inv, o[dt][g * 4 + 1] * inv);
+          w.y = M::pack2(o[dt][g * 4 + 2] * inv, o[dt][g * 4 + 3] * inv);
+          *reinterpret_cast<u32x2_v*>(op + dt * 32 + g * 8 + hh * 4) = w;
+          // (in the persistent form this runs inside the tile loop, with the next unit's queries and first scores
+          // live: the values go out one store at a time instead of being formed all at once)
+          if constexpr (PERSIST) __builtin_amdgcn_sched_barrier(0);
+        }
+      float* const lse_out = ODIT_ARG(lse);
+      if (lse_out != nullptr && hh == 0) {
+        const float lse = l_tot > 0.f ? m_run * ODIT_ARG(scale) + __logf(l_tot) : -INFINITY;
+        lse_out[(static_cast<int64_t>(b) * ODIT_ARG(H) + h) * ODIT_ARG(Sq) + row] = lse;
+      }
+    }
+  };
+
+  // Tile j of the current unit. In the persistent form the tile after a unit's last one is tile 0 of the
+  // workgroup's next unit (`cross`), and the tile after that its tile 1.
+  // `buf` (the LDS buffer pair of this tile: the parity of its running index) is a literal at every call, so the
+  // LDS addresses below are compile-time offsets.
+  auto tile = [&](int j, const int buf, f32x16_v(&s_cur)[2], f32x16_v(&s_next)[2]) {
+    const bool last = j + 1 == n_tiles;
+    const bool cross = PERSIST && last && next_pid >= 0;
+    const bool has_next = !last || cross;
     // buffers K[buf] (held K(j), consumed last tile) and V[buf^1] (held V(j-1)) are free now
-    if (j + 2 < n_tiles) dma_tile(krsrc, kvoff, static_cast<uint32_t>(j + 2) * k_tile_step, Kb + buf * TILEB);
-    if (has_next) dma_v(j + 1, Vb + (buf ^ 1) * TILEB);
+    if (j + 2 < n_tiles) {
+      dma_tile(krsrc, true, static_cast<uint32_t>(j + 2) * k_tile_step, kKoff + buf * TILEB);
+    } else if (PERSIST && next_pid >= 0) {
+      dma_k_next(j + 2 - n_tiles, kKoff + buf * TILEB);
+    }
+    if constexpr (PERSIST) {
+      if (j == 0) draw_next();  // the answer is in the box when this tile's barrier has been passed
+    }
+    if (!last) {
+      dma_v(j + 1, kVoff + (buf ^ 1) * TILEB);
+    } else if (cross) {
+      dma_v_next(0, kVoff + (buf ^ 1) * TILEB);
+    }
+    // the tile whose scores stage A computes, and the mask row of its unit
+    const int jn = last ? 0 : j + 1;
+    const uint8_t* mrow_n = cross ? (p.mask ? p.mask + static_cast<int64_t>(n_b) * p.Sk : nullptr) : mrow;  // (p.mask and p.Sk are live in the tile loop anyway)
 
     const float mc = (m_run == -INFINITY) ? 0.f : m_run * c;
+    // (Row sums in fp32 from the unrounded probabilities. Summing the packed pairs with v_dot2c_f32_bf16, one
+    // instruction per pair instead of two adds, measured 4 % slower at D = 128, with one chain or four.)
     uint32_t pf[2][2][4];
     float psum = 0.f;
     // Stage A mixes this wave's MFMAs with its exp2 work; giving it issue priority over the SIMD's other
@@ -262,6 +439,10 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
     // ---- stage A ----
     if (has_next) {
       const char* kt_base = Kb + (buf ^ 1) * TILEB;
+      // (opaque copy: the KS swizzled variants of the lane offset are formed again in every tile, one XOR each,
+      // instead of being carried through the loop in KS registers)
+      int k_lane_t = k_lane;
+      if constexpr (PERSIST) asm volatile("" : "+v"(k_lane_t));
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
@@ -270,7 +451,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
       u32x4_v kfr[KPF + 1];
       auto k_fetch = [&](int i) {
         const int ks = i >> 1, kt = i & 1;
-        kfr[i % (KPF + 1)] = *reinterpret_cast<const u32x4_v*>(kt_base + kt * 32 * ROWB + (k_lane ^ (ks * 32)));
+        kfr[i % (KPF + 1)] = *reinterpret_cast<const u32x4_v*>(kt_base + kt * 32 * ROWB + (k_lane_t ^ (ks * 32)));
       };
 #pragma unroll
       for (int i = 0; i < KPF; ++i) k_fetch(i);
@@ -294,16 +475,28 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
         __builtin_amdgcn_sched_barrier(0);  // pin: fetch(i+KPF), MFMA(i), this step's exp2 work
       }
     } else {
+      // (an opaque copy of the offset: were the two branches' exponent arguments the same expressions, the
+      // compiler would form all 32 ahead of the branch, out of the MFMAs' shadow and in 32 more registers)
+      float mc_t = mc;
+      asm volatile("" : "+v"(mc_t));
 #pragma unroll
       for (int pi = 0; pi < 16; ++pi) {
         const int pkt = pi >> 3, e0 = (pi & 7) * 2;
-        const float p0 = __builtin_amdgcn_exp2f(fmaf(s_cur[pkt][e0], c, -mc));
-        const float p1 = __builtin_amdgcn_exp2f(fmaf(s_cur[pkt][e0 + 1], c, -mc));
+        const float p0 = __builtin_amdgcn_exp2f(fmaf(s_cur[pkt][e0], c, -mc_t));
+        const float p1 = __builtin_amdgcn_exp2f(fmaf(s_cur[pkt][e0 + 1], c, -mc_t));
         psum += p0 + p1;
         pf[pkt][(pi & 7) >> 2][pi & 3] = M::pack2(p0, p1);
       }
     }
     l_run += psum;
+    if constexpr (PERSIST) {
+      // The next unit's queries replace this unit's once its last scores have been formed, a tile before they are
+      // used: they land behind this tile's closing wait. (Loaded at the top of the tile that uses them, the
+      // compiler's own wait for them, which it has to place on every trip through the loop, also waits for the
+      // tile loads it does not know of.)
+      if (j + 2 == n_tiles && next_pid >= 0)
+        load_q(n_b, n_h, (next_pid - (n_b * ODIT_ARG(H) + n_h) * ODIT_ARG(n_qblocks)) * BM + wave * 32);
+    }
 
     __builtin_amdgcn_s_setprio(0);
     // ---- stage B: O^T += V(j)^T P(j)^T ----
@@ -312,16 +505,18 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
     // of step n, so LDS latency is covered by PF matrix instructions. The in-lane row maximum of
     // S(j+1) — vector work with nothing to wait for — is placed in the shadow of these MFMAs.
     const char* vt_base = Vb + buf * TILEB;
+    int v_lane_t = v_lane;  // (opaque copy, as for the key fragments)
+    if constexpr (PERSIST) asm volatile("" : "+v"(v_lane_t));
     constexpr int NSTEP = 4 * DT;
     constexpr int PF = ODIT_ATTN_VPF;
     s16x4_d vlo[PF + 1], vhi[PF + 1];
     auto v_fetch = [&](int step) {
       const int dt = step % DT, kt = (step / DT) >> 1, g2 = (step / DT) & 1;
-      const char* vp = vt_base + (kt * 32 + g2 * 16) * ROWB + (v_lane ^ ((dt * 64) % ROWB));
+      const char* vp = vt_base + (kt * 32 + g2 * 16) * ROWB + (v_lane_t ^ ((dt * 64) % ROWB));
       vlo[step % (PF + 1)] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_p)(vp));
       vhi[step % (PF + 1)] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_p)(vp + 8 * ROWB));
     };
-    const bool plain_next = has_next && mrow == nullptr && (j + 2) * BN <= p.Sk;  // no exclusions in S(j+1)
+    const bool plain_next = has_next && mrow_n == nullptr && (jn + 1) * BN <= p.Sk;  // no exclusions in the next scores
     float mx = -INFINITY;
 #pragma unroll
     for (int st = 0; st < PF; ++st) v_fetch(st);
@@ -344,35 +539,74 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
       __builtin_amdgcn_sched_barrier(0);  // keep the reads of step st+PF ahead of this MFMA
     }
     if (has_next && !plain_next) {
-      const float t = mask_and_max(j + 1, s_next);
+      const float t = mask_and_max(jn, mrow_n, s_next);
       mx = fmaxf(t, __shfl_xor(t, 32, 64));
     }
     __builtin_amdgcn_s_waitcnt(0);  // this wave's tile loads have landed in LDS
     __syncthreads();
+    if constexpr (PERSIST) {
+      if (j == 0) take_next();
+      if (last) {
+        finish_unit();
+        if (cross) {  // the next unit becomes the current one; its running maximum, sum and accumulators start over
+          h = n_h; b = n_b;
+          q0 = (next_pid - (n_b * ODIT_ARG(H) + n_h) * ODIT_ARG(n_qblocks)) * BM + wave * 32;
+          krsrc = k_rsrc_of(b, h);
+          vrsrc = v_rsrc_of(b, h);
+          vrsrc2 = p.v_tail != nullptr ? v2_rsrc_of(b, h) : vrsrc;
+          mrow = mrow_n;
+          pid = next_pid;
+          next_pid = -1;  // drawn during the new unit's first tile
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[dt][e] = 0.f;
+          m_run = -INFINITY;
+          l_run = 0.f;
+        }
+      }
+    }
     if (has_next) settle_max(mx);
   };
 
   // ---- prologue (jt0 is even, so tile j always lives in buffer j & 1) ----
-  dma_tile(krsrc, kvoff, static_cast<uint32_t>(jt0) * k_tile_step, Kb);
-  dma_v(jt0, Vb);
-  if (jt0 + 1 < n_tiles) dma_tile(krsrc, kvoff, static_cast<uint32_t>(jt0 + 1) * k_tile_step, Kb + TILEB);
+  dma_tile(krsrc, true, static_cast<uint32_t>(jt0) * k_tile_step, kKoff);
+  dma_v(jt0, kVoff);
+  if (jt0 + 1 < n_tiles) dma_tile(krsrc, true, static_cast<uint32_t>(jt0 + 1) * k_tile_step, kKoff + TILEB);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   f32x16_v sa[2], sb[2];
   qk_plain(Kb, sa);
   {
-    const float t = mask_and_max(jt0, sa);
+    const float t = mask_and_max(jt0, mrow, sa);
     settle_max(fmaxf(t, __shfl_xor(t, 32, 64)));
   }
 
-  for (int j = jt0; j < n_tiles; j += 2) {
-    tile(j, sa, sb);
-    if (j + 1 < n_tiles) tile(j + 1, sb, sa);
+  if constexpr (PERSIST) {
+    // one stream of tiles over all units this workgroup gets; every unit stores itself behind its last tile, and
+    // the stream ends behind a unit that found the XCD's range exhausted (every wave sees the same next_pid)
+    int j = 0;
+    for (;;) {  // a tile's buffer pair is the parity of its index in this stream
+      bool done = j + 1 == n_tiles && next_pid < 0;
+      tile(j, 0, sa, sb);
+      if (done) break;
+      j = j + 1 == n_tiles ? 0 : j + 1;
+      done = j + 1 == n_tiles && next_pid < 0;
+      tile(j, 1, sb, sa);
+      if (done) break;
+      j = j + 1 == n_tiles ? 0 : j + 1;
+    }
+    return;
+  } else {
+    for (int j = jt0; j < n_tiles; j += 2) {  // jt0 is even
+      tile(j, 0, sa, sb);
+      if (j + 1 < n_tiles) tile(j + 1, 1, sb, sa);
+    }
   }
 
   // ---- epilogue ----
-  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
   if constexpr (TAIL) {
+    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
     // partial result of a key range: unnormalised O (fp32, [BM][D] per part) and the row's (m, l)
     float* wo = p.ws + (static_cast<int64_t>(part) * BM + wave * 32 + l32) * D;
 #pragma unroll
@@ -391,24 +625,30 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
     }
     return;
   }
-  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  const int row = q0 + l32;
-  if (row < p.Sq) {
-    T* op = out_row_ptr<T>(p, b, h, row);
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2_v w;
-        w.x = M::pack2(o[dt][g * 4 + 0] * inv, o[dt][g * 4 + 1] * inv);
-        w.y = M::pack2(o[dt][g * 4 + 2] * inv, o[dt][g * 4 + 3] * inv);
-        *reinterpret_cast<u32x2_v*>(op + dt * 32 + g * 8 + hh * 4) = w;
-      }
-    if (p.lse != nullptr && hh == 0) {
-      const float lse = l_tot > 0.f ? m_run * p.scale + __logf(l_tot) : -INFINITY;
-      p.lse[(static_cast<int64_t>(b) * p.H + h) * p.Sq + row] = lse;
-    }
-  }
+  finish_unit();
+}
+
+// The persistent form is a measurement aid, off unless the environment says ODIT_ATTN_PERSISTENT=1 when the
+// library makes its first attention launch: with it every shape measured ran 3 to 6 % slower than one workgroup
+// per unit (its tile loop is slower than what it saves at the unit boundaries, see the header comment).
+#ifndef ODIT_ATTN_PERSISTENT_DEFAULT
+#define ODIT_ATTN_PERSISTENT_DEFAULT 0
+#endif
+static bool persistent_form_on() {
+  static const bool on = [] {
+    const char* e = getenv("ODIT_ATTN_PERSISTENT");
+    return e != nullptr ? e[0] == '1' : ODIT_ATTN_PERSISTENT_DEFAULT != 0;
+  }();
+  return on;
+}
+
+// Workgroups of the persistent form for `units` whole units of `n_tiles` key tiles each on `slots` workgroup
+// slots, or 0 when every unit gets a workgroup of its own (no more units than slots, or units too short for the
+// next unit to be known before its first tiles are fetched).
+static int persistent_workgroups(int units, int n_tiles, int slots) {
+  const int W = slots - slots % kNumXcd;
+  if (!persistent_form_on() || W < kNumXcd || units <= W || n_tiles < 4 || units >= (1 << 26)) return 0;  // tickets have 24 bits
+  return W;
 }
 
 template <typename T, int D, int NW>
@@ -422,31 +662,42 @@ static int launch_dma(AttnParams& p, hipStream_t stream, void* ws, size_t ws_byt
   }
   p.total_blocks = static_cast<int>(total);
   p.n_full = p.total_blocks; p.key_chunks = 1; p.tiles_per_chunk = 0; p.ws = nullptr;
+  p.queue = nullptr; p.epoch = 0;
   TailPlan t{0, 1, 0};
+  const int n_tiles = (p.Sk + 63) / 64, slots = device_slots(NW);
   if (ws != nullptr) {
-    t = plan_tail(total, (p.Sk + 63) / 64, device_slots(NW));
+    if ((reinterpret_cast<uintptr_t>(ws) & 15) != 0) {
+      set_error("odit_attn_fwd: workspace must be 16-byte aligned");
+      return ODIT_EINVAL;
+    }
+    t = plan_tail(total, n_tiles, slots);
+    const size_t need = attn_dma_workspace_bytes(p.B, p.Sq, p.Sk, p.H, D);
+    if (ws_bytes < need) {
+      set_error("odit_attn_fwd: workspace of %zu bytes given, %zu needed", ws_bytes, need);
+      return ODIT_EWORKSPACE;
+    }
     if (t.rem > 0) {
-      if (ws_bytes < tail_ws_bytes(t, BM, D)) {
-        set_error("odit_attn_fwd: workspace of %zu bytes given, %zu needed", ws_bytes, tail_ws_bytes(t, BM, D));
-        return ODIT_EWORKSPACE;
-      }
-      if ((reinterpret_cast<uintptr_t>(ws) & 15) != 0) {
-        set_error("odit_attn_fwd: workspace must be 16-byte aligned");
-        return ODIT_EINVAL;
-      }
       p.n_full = p.total_blocks - t.rem; p.key_chunks = t.key_chunks; p.tiles_per_chunk = t.tiles_per_chunk;
-      p.ws = static_cast<float*>(ws);
+      p.ws = reinterpret_cast<float*>(static_cast<char*>(ws) + kAttnQueueBytes);
     }
   }
   const int n_parts = t.rem * t.key_chunks;
   int rc = ODIT_OK;
   if (p.n_full > 0) {
-    hipLaunchKernelGGL((attn_fwd_dma_kernel<T, D, NW, false>), dim3(p.n_full), dim3(NW * 64), 0, stream, p);
+    // the persistent form draws its units from ticket words at the head of the workspace
+    const int W = ws != nullptr ? persistent_workgroups(p.n_full, n_tiles, slots) : 0;
+    if (W > 0) {
+      p.queue = static_cast<unsigned long long*>(ws);
+      p.epoch = next_ticket_epoch() & ((1ull << 40) - 1);
+      hipLaunchKernelGGL((attn_fwd_dma_kernel<T, D, NW, 2>), dim3(W), dim3(NW * 64), 0, stream, p);
+    } else {
+      hipLaunchKernelGGL((attn_fwd_dma_kernel<T, D, NW, 0>), dim3(p.n_full), dim3(NW * 64), 0, stream, p);
+    }
     rc = check_launch("odit_attn_fwd");
   }
   if (rc != ODIT_OK || n_parts == 0) return rc;
   // stream order puts these after the full rounds, when every slot is free again
-  hipLaunchKernelGGL((attn_fwd_dma_kernel<T, D, NW, true>), dim3(n_parts), dim3(NW * 64), 0, stream, p);
+  hipLaunchKernelGGL((attn_fwd_dma_kernel<T, D, NW, 1>), dim3(n_parts), dim3(NW * 64), 0, stream, p);
   rc = check_launch("odit_attn_fwd (key-split tail)");
   if (rc != ODIT_OK) return rc;
   const int64_t rows = static_cast<int64_t>(t.rem) * BM;
@@ -462,34 +713,53 @@ size_t attn_dma_workspace_bytes(int B, int Sq, int Sk, int H, int D) {
   constexpr int nw = kDmaWaves;
   const int bm = nw * 32;
   const int64_t units = static_cast<int64_t>((Sq + bm - 1) / bm) * H * B;
-  return tail_ws_bytes(plan_tail(units, (Sk + 63) / 64, device_slots(nw)), bm, D);
+  const int n_tiles = (Sk + 63) / 64, slots = device_slots(nw);
+  const TailPlan t = plan_tail(units, n_tiles, slots);
+  const int64_t main_units = units - t.rem;
+  const bool persistent = main_units <= 0x3fffffff && persistent_workgroups(static_cast<int>(main_units), n_tiles, slots) > 0;
+  if (t.rem == 0 && !persistent) return 0;
+  return kAttnQueueBytes + tail_ws_bytes(t, bm, D);  // ticket words first (zero-filled once), then the tail's partial results
 }
 
 // 32-bit buffer offsets: the whole key range of one (batch, head) must be addressable
-bool attn_dma_addressable(int Sk, int64_t k_seq_stride, int64_t v_seq_stride) {
+bool attn_dma_addressable(int Sk, int D, int64_t k_seq_stride, int64_t v_seq_stride) {
   const int64_t k_span = (static_cast<int64_t>(Sk) + 64) * k_seq_stride * 2;
   const int64_t v_span = (static_cast<int64_t>(Sk) + 64) * v_seq_stride * 2;
-  return k_span < (1ll << 31) && v_span < (1ll << 31) && k_seq_stride >= 0 && v_seq_stride >= 0;
+  // (the tile loads fold their swizzle into the byte offset by an XOR, which needs rows that start on a multiple
+  // of their own length of D elements)
+  return k_span < (1ll << 31) && v_span < (1ll << 31) && k_seq_stride >= 0 && v_seq_stride >= 0 &&
+         k_seq_stride % D == 0 && v_seq_stride % D == 0;
 }
 
 int attn_dma_plan(int B, int Sq, int Sk, int H, int D, bool with_workspace, char* text, size_t text_bytes) {
   constexpr int bm = kDmaWaves * 32;
   const int64_t units = static_cast<int64_t>((Sq + bm - 1) / bm) * H * B;
+  const int n_tiles = (Sk + 63) / 64, slots = device_slots(kDmaWaves);
   TailPlan t{0, 1, 0};
-  if (with_workspace) t = plan_tail(units, (Sk + 63) / 64, device_slots(kDmaWaves));
+  if (with_workspace) t = plan_tail(units, n_tiles, slots);
+  // kernel names as a profiler prints them, with T for the element type
+  char main_text[160];
+  const int64_t main_units = units - t.rem;
+  const int W = (!with_workspace || main_units > 0x3fffffff) ? 0 : persistent_workgroups(static_cast<int>(main_units), n_tiles, slots);
+  if (W > 0) {
+    snprintf(main_text, sizeof(main_text), "attn_fwd_dma_kernel<T, %d, %d, 2> units=%lld on %d persistent workgroups", D,
+             kDmaWaves, static_cast<long long>(main_units), W);
+  } else {
+    snprintf(main_text, sizeof(main_text), "attn_fwd_dma_kernel<T, %d, %d, 0> units=%lld", D, kDmaWaves,
+             static_cast<long long>(main_units));
+  }
   if (t.rem == 0) {
-    snprintf(text, text_bytes, "attn_fwd_dma_kernel<T, %d, %d, false> units=%lld", D, kDmaWaves, static_cast<long long>(units));
+    snprintf(text, text_bytes, "%s", main_text);
     return 1;
   }
-  // kernel names as a profiler prints them, with T for the element type
-  snprintf(text, text_bytes, "attn_fwd_dma_kernel<T, %d, %d, false> units=%lld; attn_fwd_dma_kernel<T, %d, %d, true> "
-           "units=%d x %d key ranges of %d tiles; attn_merge_kernel<T, %d, %d> rows=%d", D, kDmaWaves,
-           static_cast<long long>(units - t.rem), D, kDmaWaves, t.rem, t.key_chunks, t.tiles_per_chunk, D, bm, t.rem * bm);
-  return units - t.rem > 0 ? 3 : 2;
+  snprintf(text, text_bytes, "%s; attn_fwd_dma_kernel<T, %d, %d, 1> units=%d x %d key ranges of %d tiles; "
+           "attn_merge_kernel<T, %d, %d> rows=%d", main_text, D, kDmaWaves, t.rem, t.key_chunks, t.tiles_per_chunk, D, bm,
+           t.rem * bm);
+  return main_units > 0 ? 3 : 2;
 }
 
 int launch_attn_dma(AttnParams& p, int dtype, int D, hipStream_t stream, void* ws, size_t ws_bytes) {
-  if (!attn_dma_addressable(p.Sk, p.ks_s, p.vs_s)) return ODIT_ENOTSUP;
+  if (!attn_dma_addressable(p.Sk, D, p.ks_s, p.vs_s)) return ODIT_ENOTSUP;
 #define ODIT_DMA_GO(T)                                                                     \
   if (D == 128) return launch_dma<T, 128, kDmaWaves>(p, stream, ws, ws_bytes);                \
   return launch_dma<T, 64, kDmaWaves>(p, stream, ws, ws_bytes);

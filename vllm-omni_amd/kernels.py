@@ -200,7 +200,8 @@ def _attn_workspace(lib, device: torch.device, B: int, Sq: int, Sk: int, H: int,
     key = (device.index or 0, _stream())
     ws = _ATTN_SCRATCH.get(key)
     if ws is None or ws.numel() < need:
-        ws = torch.empty(need, dtype=torch.uint8, device=device)
+        # zero-filled once: the first kilobyte holds the ticket words the persistent kernel draws its units from
+        ws = torch.zeros(need, dtype=torch.uint8, device=device)
         _ATTN_SCRATCH[key] = ws
     return ws
 

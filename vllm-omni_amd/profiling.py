@@ -261,7 +261,7 @@ def summarise_step(directory: str, bench_stdout: str, workload: str) -> str:
     out = [f"# rocprofv3 kernel-trace summary: bench.py, {title}, MI355X",
            "# commands (from the repo root, on the GPU box):",
            f"#   export TMPDIR=/tmp OUT=<a scratch directory>; rocprofv3 --kernel-trace --stats --output-format csv -d $OUT/prof_{workload} -o bench -- "
-           f"python3 bench.py{flag} --steps {d['steps']} --warmup {d['warmup']} --no-cpu --no-kernels > $OUT/prof_{workload}.log",
+           f"python3 bench.py{flag} --steps {d['steps']} --warmup {d['warmup']} --no-cpu --no-kernels --no-in-step --no-teacache > $OUT/prof_{workload}.log",
            f"#   python3 -m vllm_omni_amd.profiling step $OUT/prof_{workload} $OUT/prof_{workload}.log {workload}",
            f"# {steps} steps recorded ({d['warmup']} warm-up + {d['steps']} timed) => per-step time = total / {steps}. Weight-initialisation kernels of the",
            "# synthetic model (at::native::distribution_* = normal_ init, FillFunctor = zero_ init, __amd_rocclr_copyBuffer = stacking the",
