@@ -243,7 +243,8 @@ int odit_gated_residual(const void* h, const void* y, const void* gate, const fl
  * cur, prev: [B, n] with row strides cur_stride / prev_stride (elements); n % 8 == 0 not required.
  * sums: double [B,2] on the device.
  * workspace: device scratch of at least odit_rel_l1_workspace_bytes(B, n) bytes, 16-byte aligned: a
- *   region of fixed size (512 KiB, whatever B is) with one 64-bit ticket word per row, then the partials.
+ *   region of fixed size (568 KiB, whatever B is) with one 64-bit ticket word per row and the group words that
+ *   rows of many workgroups draw from first, then the partials.
  *   ZERO-FILL IT ONCE after allocating it (hipMemsetAsync, or a fill kernel under graph capture) and do
  *   not write it afterwards. A ticket word is (launch number << 16 | tickets drawn); every launch first
  *   raises its rows' words to its own number, which is larger than any earlier launch's, and the last

@@ -65,8 +65,9 @@ def test_argument_errors_are_caught_before_launch():
                               _strides(256, 64), 2, 4, 1e-6, 1, 0, 0, 0, None)
     assert rc == -1 and b"do not fit" in lib.odit_last_error()
     # workspace too small
-    # a ticket word for each of the 65536 rows a call may have, then 32 workgroups per row of 2^20 elements
-    assert lib.odit_rel_l1_workspace_bytes(2, 1 << 20) == 65536 * 8 + 2 * 32 * 8
+    # a ticket word for each of the 65536 rows a call may have, 8 group words 1 KiB apart for each of the 7 rows that
+    # can have more than 32 workgroups, then 32 workgroups per row of 2^20 elements
+    assert lib.odit_rel_l1_workspace_bytes(2, 1 << 20) == 65536 * 8 + 7 * 8 * 1024 + 2 * 32 * 8
     rc = lib.odit_rel_l1(p16, p16, p16, p16, 8, 2, 1 << 20, 1 << 20, 1 << 20, 0, 0, None)
     assert rc == -4
     # empty problems succeed without touching the device

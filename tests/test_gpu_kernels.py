@@ -276,10 +276,14 @@ def test_rel_l1_workspace_rows_grow_and_stale_ticket_words(gpu):
     # stale words: launch number 0 with 1..99 tickets drawn in every row's word
     words = ws[:8 * 100].view(torch.int64)   # the words of the rows these calls use
     words.copy_(torch.randint(1, 100, words.shape, device=gpu))
+    # ... and in the group words of the two long rows (8 per row, 1 KiB apart, behind the 65536 row words)
+    groups = ws[65536 * 8:65536 * 8 + 2 * 8 * 1024].view(torch.int64).view(16, 128)[:, 0]
+    groups.copy_(torch.randint(1, 16, groups.shape, device=gpu))
     assert torch.equal(run(*data[many], ws), fresh[many])
     assert torch.equal(run(*data[few], ws), fresh[few])
     torch.cuda.synchronize()
     assert int(ws[:8 * 100].view(torch.int64).abs().max().item()) == 0   # handed back at zero
+    assert int(groups.abs().max().item()) == 0
 
 
 def test_rel_l1_closed_forms(gpu):

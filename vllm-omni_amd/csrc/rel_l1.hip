@@ -33,7 +33,22 @@ constexpr int kRelL1StaticRows = 64;
 // counter region of a caller's workspace: one word for each of the kRelL1MaxRows rows a call may have,
 // whatever B a particular call has (a region sized by B would let one call's partials be a later call's
 // counters)
-constexpr size_t kRelL1CounterBytes = (static_cast<size_t>(kRelL1MaxRows) + 1) * sizeof(uint64_t);
+constexpr size_t kRelL1RowWordBytes = (static_cast<size_t>(kRelL1MaxRows) + 1) * sizeof(uint64_t);
+// Behind the rows' words, group words: a row of more than kRelL1GroupAbove workgroups (few, long rows) draws its
+// tickets in two levels, workgroup x from the word of group x % kRelL1Groups and only each group's last arrival
+// from the row's word. Atomics on one address are applied one after the other (~20 ns each, and every workgroup
+// arrives within the kernel's last microsecond). Measured for 2 x 12.6 M bf16 elements on one box: two atomics per
+// workgroup on the row's word at the end of the kernel 24.7 us; the first of them moved to the start of the kernel
+// 23.0; 16 arrivals per group word and 8 on the row's word 21.6; one atomic per workgroup and nothing to override
+// stale words with 20.0; no tickets and no final sum at all 19.2. Group words are 1 KiB apart so that they sit in
+// different memory channels.
+constexpr int kRelL1Groups = 8;
+constexpr int kRelL1GroupAbove = 32;
+constexpr int kRelL1GroupedRows = kRelL1TotalBlocks / (kRelL1GroupAbove + 1);  // rows that can have that many workgroups
+constexpr int kRelL1GroupStrideWords = 128;
+constexpr size_t kRelL1GroupBytes =
+    static_cast<size_t>(kRelL1GroupedRows) * kRelL1Groups * kRelL1GroupStrideWords * sizeof(uint64_t);
+constexpr size_t kRelL1CounterBytes = kRelL1RowWordBytes + kRelL1GroupBytes;
 
 static inline int rel_l1_blocks_per_row(int B, int64_t n) {
   // at least one pass of four 16-byte vectors per thread (sized on 8-element vectors; fp32 rows get twice the
@@ -51,7 +66,7 @@ static inline int rel_l1_blocks_per_row(int B, int64_t n) {
 
 template <typename T, bool REF_ROUND>
 __global__ __launch_bounds__(kRelL1Threads) void rel_l1_kernel(const T* __restrict__ cur, const T* __restrict__ prev,
-                                                     float* partials, uint64_t* counters, uint64_t epoch,
+                                                     float* partials, uint64_t* counters, uint64_t* groups, uint64_t epoch,
                                                      double* __restrict__ sums, int64_t n, int64_t n_vec,
                                                      int64_t cur_stride, int64_t prev_stride) {
   constexpr int EPV = Vec16<T>::N;
@@ -63,6 +78,16 @@ __global__ __launch_bounds__(kRelL1Threads) void rel_l1_kernel(const T* __restri
   const int64_t per_blk = (n_vec + nblk - 1) / nblk;
   const int64_t v_begin = static_cast<int64_t>(blockIdx.x) * per_blk;
   const int64_t v_end = v_begin + per_blk < n_vec ? v_begin + per_blk : n_vec;
+  // Two-level tickets for rows of many workgroups (groups == nullptr: one level always)
+  const bool grouped = groups != nullptr && nblk > kRelL1GroupAbove && b < kRelL1GroupedRows;
+  const int grp = static_cast<int>(blockIdx.x) % kRelL1Groups;
+  uint64_t* const my_word = grouped ? groups + (static_cast<int64_t>(b) * kRelL1Groups + grp) * kRelL1GroupStrideWords : counters + b;
+  const uint64_t my_arrivals = grouped ? static_cast<uint64_t>((nblk - grp + kRelL1Groups - 1) / kRelL1Groups) : static_cast<uint64_t>(nblk);
+  // The word this workgroup draws from is raised to the launch's epoch here, long before the tickets are drawn (a
+  // no-op for all but the word's first arrival; no value comes back, nothing waits for it): at the end of the
+  // kernel each workgroup then waits for one atomic, not two.
+  const uint64_t base = epoch << 16;
+  if (threadIdx.x == 0) __hip_atomic_fetch_max(my_word, base, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   float sd = 0.f, sp = 0.f;
   auto accumulate = [&](const Vec16<T>& cv, const Vec16<T>& pv) {
 #pragma unroll
@@ -121,12 +146,20 @@ __global__ __launch_bounds__(kRelL1Threads) void rel_l1_kernel(const T* __restri
     __atomic_signal_fence(__ATOMIC_SEQ_CST);
     __builtin_amdgcn_s_waitcnt(0);
     __atomic_signal_fence(__ATOMIC_SEQ_CST);
-    // the row's word is raised to this launch's epoch (a no-op for all but the row's first workgroup), then
-    // the ticket is drawn: two atomics of one thread on one address, applied in program order
-    const uint64_t base = epoch << 16;
-    __hip_atomic_fetch_max(counters + b, base, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const uint64_t ticket = __hip_atomic_fetch_add(counters + b, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    last_of_row = ticket == base + static_cast<uint64_t>(nblk) - 1u;
+    // the ticket is drawn: this thread's second atomic on the word after the one that raised it to the launch's
+    // epoch, two atomics of one thread on one address, applied in program order
+    uint64_t ticket = __hip_atomic_fetch_add(my_word, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    bool last = ticket == base + my_arrivals - 1u;
+    if (grouped && last) {
+      // last of its group: the group's word goes back to zero (as the row's word below), and the group arrives at
+      // the row's word, which its first arrival raises
+      __hip_atomic_store(my_word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_fetch_max(counters + b, base, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      ticket = __hip_atomic_fetch_add(counters + b, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int n_groups = nblk < kRelL1Groups ? nblk : kRelL1Groups;
+      last = ticket == base + static_cast<uint64_t>(n_groups) - 1u;
+    }
+    last_of_row = last;
     __atomic_signal_fence(__ATOMIC_SEQ_CST);  // the reader's loads below stay below the ticket
   }
   __syncthreads();
@@ -167,7 +200,7 @@ __global__ __launch_bounds__(256) void rel_l1_clear_kernel(uint64_t* counters, i
 }
 
 template <typename T>
-static int launch_rel_l1(const void* cur, const void* prev, double* sums, uint64_t* counters, float* partials, int B,
+static int launch_rel_l1(const void* cur, const void* prev, double* sums, uint64_t* counters, uint64_t* groups, float* partials, int B,
                          int64_t n, int64_t cur_stride, int64_t prev_stride, bool ref_round,
                          hipStream_t stream) {
   constexpr int EPV = Vec16<T>::N;
@@ -179,10 +212,10 @@ static int launch_rel_l1(const void* cur, const void* prev, double* sums, uint64
   const dim3 grid(nblk, B);
   if (ref_round) {
     hipLaunchKernelGGL((rel_l1_kernel<T, true>), grid, dim3(kRelL1Threads), 0, stream, static_cast<const T*>(cur),
-                       static_cast<const T*>(prev), partials, counters, epoch, sums, n, n_vec, cur_stride, prev_stride);
+                       static_cast<const T*>(prev), partials, counters, groups, epoch, sums, n, n_vec, cur_stride, prev_stride);
   } else {
     hipLaunchKernelGGL((rel_l1_kernel<T, false>), grid, dim3(kRelL1Threads), 0, stream, static_cast<const T*>(cur),
-                       static_cast<const T*>(prev), partials, counters, epoch, sums, n, n_vec, cur_stride, prev_stride);
+                       static_cast<const T*>(prev), partials, counters, groups, epoch, sums, n, n_vec, cur_stride, prev_stride);
   }
   return check_launch("odit_rel_l1");
 }
@@ -213,9 +246,10 @@ extern "C" int odit_rel_l1(const void* cur, const void* prev, double* sums, void
   }
   const bool rr = (flags & ODIT_FLAG_REF_ROUNDING) && dtype != ODIT_F32;
   uint64_t* counters = static_cast<uint64_t*>(workspace);
+  uint64_t* groups = reinterpret_cast<uint64_t*>(static_cast<char*>(workspace) + kRelL1RowWordBytes);
   float* partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + kRelL1CounterBytes);
   ODIT_DISPATCH_DTYPE(dtype, T,
-                      return launch_rel_l1<T>(cur, prev, sums, counters, partials, B, n, cur_stride, prev_stride, rr,
+                      return launch_rel_l1<T>(cur, prev, sums, counters, groups, partials, B, n, cur_stride, prev_stride, rr,
                                               static_cast<hipStream_t>(stream)));
   return ODIT_OK;
 }
@@ -300,6 +334,6 @@ extern "C" int odit_rel_l1_static(const void* cur, const void* prev, double* sum
   uint64_t* counters = static_cast<uint64_t*>(ptr);
   float* partials = reinterpret_cast<float*>(static_cast<char*>(ptr) + kRelL1StaticCounterBytes);
   ODIT_DISPATCH_DTYPE(dtype, T,
-                      return launch_rel_l1<T>(cur, prev, sums, counters, partials, B, n, cur_stride, prev_stride, rr, st));
+                      return launch_rel_l1<T>(cur, prev, sums, counters, nullptr, partials, B, n, cur_stride, prev_stride, rr, st));
   return ODIT_OK;
 }
