@@ -94,8 +94,15 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   constexpr int RPI = 64 / CPR;               // tile rows filled by one wave instruction (4 or 8)
   constexpr int TILEB = BN * ROWB;            // bytes per tile
   constexpr int NINST = BN / RPI;             // wave instructions per tile (16 or 8)
-  constexpr int IPW = (NINST + NW - 1) / NW;  // ... per wavefront
-  static_assert(NINST % NW == 0, "tile loads must divide evenly over the wavefronts");
+  // NW = 8 is the anti-phase form: the workgroup's two wavefronts on a SIMD (w and w + 4) run the same tile loop
+  // half a tile apart, held there by a second barrier between the stages, so one's stage A (exp2 and the other
+  // vector work, with the next scores' MFMAs) always meets the other's stage B (MFMAs and LDS reads only). Wavefronts
+  // 0-3 fetch the K tiles, 4-7 the V tiles, each group at the start of its own stage A.
+  constexpr bool PP = NW == 8;
+  static_assert(!(PP && PERSIST), "the persistent form has no anti-phase variant");
+  constexpr int NWL = PP ? 4 : NW;              // wavefronts that fetch one tile
+  constexpr int IPW = (NINST + NWL - 1) / NWL;  // ... per wavefront
+  static_assert(NINST % NWL == 0, "tile loads must divide evenly over the wavefronts");
   constexpr int BM = NW * 32;
 
   __shared__ __attribute__((aligned(1024))) char lds[4 * TILEB];  // K0 K1 V0 V1
@@ -126,6 +133,8 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   }
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hh = lane >> 5;
+  const int wl = PP ? (wave & 3) : wave;     // this wavefront's share of a tile load
+  const bool grp1 = PP && wave >= 4;          // second group of the anti-phase form (wave-uniform)
 
   // ---- the current unit (fixed for MODE 0 and 1, advanced unit by unit in the persistent form) ----
   int h = (pid / p.n_qblocks) % p.H;
@@ -202,7 +211,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   // for K, row % 16 = (row0 % 16) + (RPI * i) % 16 without a carry (row0 % 16 < RPI), so the chunk index is that
   // of instruction 0 XOR ((RPI * i) % 16 % CPR) - for V (4 * (row % 4), RPI a multiple of 4) it is the same. The
   // XOR is done on the byte offset, which needs row strides that are multiples of the row's own 2 D bytes.
-  const int r0 = wave * IPW * RPI + lane / CPR, pc0 = lane % CPR;
+  const int r0 = wl * IPW * RPI + lane / CPR, pc0 = lane % CPR;
   const uint32_t kvoff0 = static_cast<uint32_t>(r0 * p.ks_s * 2) + static_cast<uint32_t>(((pc0 ^ (r0 % 16)) % CPR) * 16);
   const uint32_t vvoff0 = static_cast<uint32_t>(r0 * p.vs_s * 2) + static_cast<uint32_t>(((pc0 ^ (4 * (r0 % 4))) % CPR) * 16);
   const uint32_t k_inst_step = static_cast<uint32_t>(RPI * p.ks_s * 2);
@@ -220,7 +229,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_void_p)lds));
   auto dma_tile = [&](const u32x4_v& rsrc, const bool is_k, uint32_t soff, const int dst_off) {
 #if defined(__HIP_DEVICE_COMPILE__)
-    const uint32_t lds0 = lds_base + static_cast<uint32_t>(dst_off) + static_cast<uint32_t>(wave * IPW * 1024);
+    const uint32_t lds0 = lds_base + static_cast<uint32_t>(dst_off) + static_cast<uint32_t>(wl * IPW * 1024);
     // (the empty asm makes the offset opaque here: otherwise the compiler forms the IPW swizzled offsets once,
     // outside the tile loop, and holds them in registers the loop does not have)
     uint32_t voff0 = is_k ? kvoff0 : vvoff0;
@@ -410,18 +419,24 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
     const bool cross = PERSIST && last && next_pid >= 0;
     const bool has_next = !last || cross;
     // buffers K[buf] (held K(j), consumed last tile) and V[buf^1] (held V(j-1)) are free now
-    if (j + 2 < n_tiles) {
-      dma_tile(krsrc, true, static_cast<uint32_t>(j + 2) * k_tile_step, kKoff + buf * TILEB);
-    } else if (PERSIST && next_pid >= 0) {
-      dma_k_next(j + 2 - n_tiles, kKoff + buf * TILEB);
+    // (anti-phase form: the first group fetches K, the second V; K(j) was last read by the second group's stage A
+    // of tile j - 1, half a tile before the first group gets here, V(j-1) by the second group's own stage B)
+    if (!PP || !grp1) {
+      if (j + 2 < n_tiles) {
+        dma_tile(krsrc, true, static_cast<uint32_t>(j + 2) * k_tile_step, kKoff + buf * TILEB);
+      } else if (PERSIST && next_pid >= 0) {
+        dma_k_next(j + 2 - n_tiles, kKoff + buf * TILEB);
+      }
     }
     if constexpr (PERSIST) {
       if (j == 0) draw_next();  // the answer is in the box when this tile's barrier has been passed
     }
-    if (!last) {
-      dma_v(j + 1, kVoff + (buf ^ 1) * TILEB);
-    } else if (cross) {
-      dma_v_next(0, kVoff + (buf ^ 1) * TILEB);
+    if (!PP || grp1) {
+      if (!last) {
+        dma_v(j + 1, kVoff + (buf ^ 1) * TILEB);
+      } else if (cross) {
+        dma_v_next(0, kVoff + (buf ^ 1) * TILEB);
+      }
     }
     // the tile whose scores stage A computes, and the mask row of its unit
     const int jn = last ? 0 : j + 1;
@@ -499,6 +514,13 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
     }
 
     __builtin_amdgcn_s_setprio(0);
+    if constexpr (PP) {
+      // the stages' boundary: the two groups swap roles here. A bare barrier: no wavefront writes LDS, and the tile
+      // loads in flight are waited for at the end of the tile, not here.
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_barrier" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+    }
     // ---- stage B: O^T += V(j)^T P(j)^T ----
     // 4*DT steps, head-dim tile innermost so that consecutive MFMAs hit different accumulators and one
     // P fragment serves DT of them; the two transpose reads of step n + PF are issued before the MFMA
@@ -570,9 +592,9 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   };
 
   // ---- prologue (jt0 is even, so tile j always lives in buffer j & 1) ----
-  dma_tile(krsrc, true, static_cast<uint32_t>(jt0) * k_tile_step, kKoff);
-  dma_v(jt0, kVoff);
-  if (jt0 + 1 < n_tiles) dma_tile(krsrc, true, static_cast<uint32_t>(jt0 + 1) * k_tile_step, kKoff + TILEB);
+  if (!PP || !grp1) dma_tile(krsrc, true, static_cast<uint32_t>(jt0) * k_tile_step, kKoff);
+  if (!PP || grp1) dma_v(jt0, kVoff);
+  if ((!PP || !grp1) && jt0 + 1 < n_tiles) dma_tile(krsrc, true, static_cast<uint32_t>(jt0 + 1) * k_tile_step, kKoff + TILEB);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   f32x16_v sa[2], sb[2];
@@ -580,6 +602,13 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
   {
     const float t = mask_and_max(jt0, mrow, sa);
     settle_max(fmaxf(t, __shfl_xor(t, 32, 64)));
+  }
+  // every wavefront has read the first K tile: the loop's first tile load overwrites it
+  __syncthreads();
+  if constexpr (PP) {
+    // the second group enters the loop one barrier, i.e. half a tile, behind the first (which makes up for it
+    // behind the loop)
+    if (grp1) asm volatile("s_barrier" ::: "memory");
   }
 
   if constexpr (PERSIST) {
@@ -601,6 +630,9 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attn_fwd_dma_kernel(const Att
     for (int j = jt0; j < n_tiles; j += 2) {  // jt0 is even
       tile(j, 0, sa, sb);
       if (j + 1 < n_tiles) tile(j + 1, 1, sb, sa);
+    }
+    if constexpr (PP) {
+      if (!grp1) asm volatile("s_barrier" ::: "memory");
     }
   }
 
@@ -645,9 +677,9 @@ static bool persistent_form_on() {
 // Workgroups of the persistent form for `units` whole units of `n_tiles` key tiles each on `slots` workgroup
 // slots, or 0 when every unit gets a workgroup of its own (no more units than slots, or units too short for the
 // next unit to be known before its first tiles are fetched).
-static int persistent_workgroups(int units, int n_tiles, int slots) {
+static int persistent_workgroups(int units, int n_tiles, int slots, int nw) {
   const int W = slots - slots % kNumXcd;
-  if (!persistent_form_on() || W < kNumXcd || units <= W || n_tiles < 4 || units >= (1 << 26)) return 0;  // tickets have 24 bits
+  if (!persistent_form_on() || nw != 4 || W < kNumXcd || units <= W || n_tiles < 4 || units >= (1 << 26)) return 0;  // tickets have 24 bits
   return W;
 }
 
@@ -685,12 +717,15 @@ static int launch_dma(AttnParams& p, hipStream_t stream, void* ws, size_t ws_byt
   int rc = ODIT_OK;
   if (p.n_full > 0) {
     // the persistent form draws its units from ticket words at the head of the workspace
-    const int W = ws != nullptr ? persistent_workgroups(p.n_full, n_tiles, slots) : 0;
-    if (W > 0) {
-      p.queue = static_cast<unsigned long long*>(ws);
-      p.epoch = next_ticket_epoch() & ((1ull << 40) - 1);
-      hipLaunchKernelGGL((attn_fwd_dma_kernel<T, D, NW, 2>), dim3(W), dim3(NW * 64), 0, stream, p);
-    } else {
+    const int W = (ws != nullptr && NW == 4) ? persistent_workgroups(p.n_full, n_tiles, slots, NW) : 0;
+    if constexpr (NW == 4) {
+      if (W > 0) {
+        p.queue = static_cast<unsigned long long*>(ws);
+        p.epoch = next_ticket_epoch() & ((1ull << 40) - 1);
+        hipLaunchKernelGGL((attn_fwd_dma_kernel<T, D, NW, 2>), dim3(W), dim3(NW * 64), 0, stream, p);
+      }
+    }
+    if (W == 0) {
       hipLaunchKernelGGL((attn_fwd_dma_kernel<T, D, NW, 0>), dim3(p.n_full), dim3(NW * 64), 0, stream, p);
     }
     rc = check_launch("odit_attn_fwd");
@@ -706,17 +741,34 @@ static int launch_dma(AttnParams& p, hipStream_t stream, void* ws, size_t ws_byt
   return check_launch("odit_attn_fwd (merge)");
 }
 
-constexpr int kDmaWaves = 4;  // wavefronts per workgroup (two workgroups per compute unit)
+// Wavefronts per workgroup: 4 (two workgroups per compute unit, each on its own) or 8 (one workgroup per compute unit
+// whose two halves run in anti-phase). Side by side in one process (bf16, us, 4 / 8 wavefronts; two boxes):
+//   D=128  B=2 S=4352 H=24  514 / 491, 492 / 473     B=2 S=4096 H=24  429 / 420, 407 / 402
+//          B=1 S=4608 H=24  302 / 297, 289 / 288     B=2 S=32760 H=40  38910 / 38616, 37053 / 36483
+//   D=64   B=2 S=4352 H=24  326 / 334, 316 / 328
+// so head size 128 takes 8 and head size 64 stays at 4. (With the two halves' roles paired wrongly, wavefronts w and
+// w + 1 or w and w + 2 in anti-phase instead of w and w + 4, the same kernel is 10 to 18 % slower: two wavefronts of a
+// SIMD in the same stage is what costs, and independent workgroups already avoid it most of the time by themselves.)
+// ODIT_ATTN_WAVES in the environment, read at the first attention launch, overrides the choice (for measurements).
+static int dma_waves(int D) {
+  static const int forced = [] {
+    const char* e = getenv("ODIT_ATTN_WAVES");
+    const int v = e != nullptr ? atoi(e) : 0;
+    return (v == 4 || v == 8) ? v : 0;
+  }();
+  if (forced != 0) return forced;
+  return D == 128 ? 8 : 4;
+}
 
 size_t attn_dma_workspace_bytes(int B, int Sq, int Sk, int H, int D) {
   if (B <= 0 || Sq <= 0 || Sk <= 0 || H <= 0) return 0;
-  constexpr int nw = kDmaWaves;
+  const int nw = dma_waves(D);
   const int bm = nw * 32;
   const int64_t units = static_cast<int64_t>((Sq + bm - 1) / bm) * H * B;
   const int n_tiles = (Sk + 63) / 64, slots = device_slots(nw);
   const TailPlan t = plan_tail(units, n_tiles, slots);
   const int64_t main_units = units - t.rem;
-  const bool persistent = main_units <= 0x3fffffff && persistent_workgroups(static_cast<int>(main_units), n_tiles, slots) > 0;
+  const bool persistent = main_units <= 0x3fffffff && persistent_workgroups(static_cast<int>(main_units), n_tiles, slots, nw) > 0;
   if (t.rem == 0 && !persistent) return 0;
   return kAttnQueueBytes + tail_ws_bytes(t, bm, D);  // ticket words first (zero-filled once), then the tail's partial results
 }
@@ -732,20 +784,20 @@ bool attn_dma_addressable(int Sk, int D, int64_t k_seq_stride, int64_t v_seq_str
 }
 
 int attn_dma_plan(int B, int Sq, int Sk, int H, int D, bool with_workspace, char* text, size_t text_bytes) {
-  constexpr int bm = kDmaWaves * 32;
+  const int nw = dma_waves(D), bm = nw * 32;
   const int64_t units = static_cast<int64_t>((Sq + bm - 1) / bm) * H * B;
-  const int n_tiles = (Sk + 63) / 64, slots = device_slots(kDmaWaves);
+  const int n_tiles = (Sk + 63) / 64, slots = device_slots(nw);
   TailPlan t{0, 1, 0};
   if (with_workspace) t = plan_tail(units, n_tiles, slots);
   // kernel names as a profiler prints them, with T for the element type
   char main_text[160];
   const int64_t main_units = units - t.rem;
-  const int W = (!with_workspace || main_units > 0x3fffffff) ? 0 : persistent_workgroups(static_cast<int>(main_units), n_tiles, slots);
+  const int W = (!with_workspace || main_units > 0x3fffffff) ? 0 : persistent_workgroups(static_cast<int>(main_units), n_tiles, slots, nw);
   if (W > 0) {
     snprintf(main_text, sizeof(main_text), "attn_fwd_dma_kernel<T, %d, %d, 2> units=%lld on %d persistent workgroups", D,
-             kDmaWaves, static_cast<long long>(main_units), W);
+             nw, static_cast<long long>(main_units), W);
   } else {
-    snprintf(main_text, sizeof(main_text), "attn_fwd_dma_kernel<T, %d, %d, 0> units=%lld", D, kDmaWaves,
+    snprintf(main_text, sizeof(main_text), "attn_fwd_dma_kernel<T, %d, %d, 0> units=%lld", D, nw,
              static_cast<long long>(main_units));
   }
   if (t.rem == 0) {
@@ -753,7 +805,7 @@ int attn_dma_plan(int B, int Sq, int Sk, int H, int D, bool with_workspace, char
     return 1;
   }
   snprintf(text, text_bytes, "%s; attn_fwd_dma_kernel<T, %d, %d, 1> units=%d x %d key ranges of %d tiles; "
-           "attn_merge_kernel<T, %d, %d> rows=%d", main_text, D, kDmaWaves, t.rem, t.key_chunks, t.tiles_per_chunk, D, bm,
+           "attn_merge_kernel<T, %d, %d> rows=%d", main_text, D, nw, t.rem, t.key_chunks, t.tiles_per_chunk, D, bm,
            t.rem * bm);
   return main_units > 0 ? 3 : 2;
 }
@@ -761,8 +813,12 @@ int attn_dma_plan(int B, int Sq, int Sk, int H, int D, bool with_workspace, char
 int launch_attn_dma(AttnParams& p, int dtype, int D, hipStream_t stream, void* ws, size_t ws_bytes) {
   if (!attn_dma_addressable(p.Sk, D, p.ks_s, p.vs_s)) return ODIT_ENOTSUP;
 #define ODIT_DMA_GO(T)                                                                     \
-  if (D == 128) return launch_dma<T, 128, kDmaWaves>(p, stream, ws, ws_bytes);                \
-  return launch_dma<T, 64, kDmaWaves>(p, stream, ws, ws_bytes);
+  if (dma_waves(D) == 8) {                                                                  \
+    if (D == 128) return launch_dma<T, 128, 8>(p, stream, ws, ws_bytes);                   \
+    return launch_dma<T, 64, 8>(p, stream, ws, ws_bytes);                                  \
+  }                                                                                        \
+  if (D == 128) return launch_dma<T, 128, 4>(p, stream, ws, ws_bytes);                     \
+  return launch_dma<T, 64, 4>(p, stream, ws, ws_bytes);
   if (dtype == ODIT_BF16) { ODIT_DMA_GO(bf16_t) }
   ODIT_DMA_GO(f16_t)
 #undef ODIT_DMA_GO
