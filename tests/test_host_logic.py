@@ -674,14 +674,14 @@ def test_profile_records_name_the_launches_they_were_measured_on():
     traffic = profiling.read_record(profiling.TRAFFIC_FILE)
     counters = profiling.read_record(profiling.COUNTERS_FILE)
     plan = traffic["attention_plan"]
-    assert plan == counters["attention_plan"] and "attn_fwd_dma_kernel<T, 128, 4, 0>" in plan
+    assert plan == counters["attention_plan"] and "attn_fwd_dma_kernel<T, 128, 8, 0>" in plan
     fig = profiling.attention_figures(plan)
     assert fig["traffic_bytes"] == traffic["traffic_bytes"] > 213.9e6          # at least the algorithmic bytes
     assert 0.3 < fig["mfma_busy_frac"] < 1.0 and 1000 < fig["clock_MHz"] < 2500
     assert "attn_fwd_dma_kernel" in fig["profiled_kernel"]
     with pytest.raises(RuntimeError, match="re-run the counter passes"):
-        profiling.attention_figures(plan.replace("units=1536", "units=1537"))
-    assert profiling._plan_kernels(plan) == ["attn_fwd_dma_kernel<T, 128, 4, 0>", "attn_fwd_dma_kernel<T, 128, 4, 1>",
-                                             "attn_merge_kernel<T, 128, 128>"]
-    assert profiling._is_kernel("attn_merge_kernel<T, 128, 128>", "void odit::attn_merge_kernel<odit::bf16_t, 128, 128>(odit::AttnParams, int)")
-    assert not profiling._is_kernel("attn_fwd_dma_kernel<T, 128, 4, 1>", "void odit::attn_fwd_dma_kernel<odit::bf16_t, 128, 4, 0>(odit::AttnParams)")
+        profiling.attention_figures(plan.replace("units=768", "units=769"))
+    assert profiling._plan_kernels(plan) == ["attn_fwd_dma_kernel<T, 128, 8, 0>", "attn_fwd_dma_kernel<T, 128, 8, 1>",
+                                             "attn_merge_kernel<T, 128, 256>"]
+    assert profiling._is_kernel("attn_merge_kernel<T, 128, 256>", "void odit::attn_merge_kernel<odit::bf16_t, 128, 256>(odit::AttnParams, int)")
+    assert not profiling._is_kernel("attn_fwd_dma_kernel<T, 128, 8, 1>", "void odit::attn_fwd_dma_kernel<odit::bf16_t, 128, 8, 0>(odit::AttnParams)")
