@@ -348,6 +348,14 @@ def run_secondary(torch, kernels, args):
     ms, flop, n = timer.dominant()
     tf = flop / ms / 1e9
     attn_total = sum(timer.flops) / args.steps
+    in_step = None
+    if not args.no_in_step:   # as for the headline workload: extra steps outside the timed region, kernel by kernel
+        n_extra = 1 if args.workload == "wan" else 2
+        with torch.inference_mode(), StepKernelTimer(torch, kernels) as kt:
+            for i in range(n_extra):
+                lat = step(i, lat)
+            torch.cuda.synchronize()
+        in_step = kt.report(n_extra)
     teacache = None
     if args.teacache is not None:
         if args.workload != "flux":
@@ -364,6 +372,9 @@ def run_secondary(torch, kernels, args):
         "step_flop": {"gemm": gemm_flop, "attention": attn_total,
                       "achieved_TFLOP/s": (gemm_flop + attn_total) / (elapsed / args.steps) / 1e12},
         "teacache": teacache,
+        "kernels_in_step": None if in_step is None else {
+            "what": "per-kernel averages over extra steps run right after the timed region, each call between its own "
+                    "HIP events (not part of `value`)", "kernels": in_step},
     }))
 
 

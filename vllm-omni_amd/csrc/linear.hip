@@ -578,17 +578,27 @@ extern "C" int odit_linear_rows_tune(const void* x, const void* w, const void* b
   ODIT_CHECK_ARG(M > 0 && iters > 0, "odit_linear_tune: needs M > 0 and iters > 0");
   ODIT_CHECK_ARG(rows_per_gate >= 0 && gate_stride >= 0, "odit_linear_tune: rows_per_gate and gate_stride must not be negative");
   const bool per_rows = lin_is_residual(c) && gate != nullptr && rows_per_gate > 0 && rows_per_gate < M;
-  // the library runs one launch per group of rows: tune that launch (on the first group)
+  // the library runs one launch per group of rows: tune that launch (on the first group), and the shorter
+  // launch of a last group that is not full, which is a problem of its own to the library
   LinCall cl = c;
-  int launches = 1;
+  int launches = 1, last_rows = 0;
   if (per_rows) {
     cl.M = rows_per_gate;
-    launches = (M + rows_per_gate - 1) / rows_per_gate;
+    launches = M / rows_per_gate;
+    last_rows = M % rows_per_gate;
   }
   float lib_us = 0.f;
   rc = lin_tune_library(cl, iters, flush, flush_bytes, &lib_us);
   if (rc != ODIT_OK) return rc;
   lib_us *= static_cast<float>(launches);
+  if (last_rows > 0) {
+    LinCall cr = cl;   // (timed on the first rows: only the shape matters)
+    cr.M = last_rows;
+    float last_us = 0.f;
+    rc = lin_tune_library(cr, iters, flush, flush_bytes, &last_us);
+    if (rc != ODIT_OK) return rc;
+    lib_us += last_us;
+  }
   float best = lib_us;
   const GemmCall g = lin_gemm_call(c, per_rows ? rows_per_gate : 0, per_rows ? gate_stride : 0);
   if (const int kind = lin_handwritten_kind(g, dtype, sk)) {
