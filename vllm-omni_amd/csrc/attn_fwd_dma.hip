@@ -746,23 +746,28 @@ static int launch_dma(AttnParams& p, hipStream_t stream, void* ws, size_t ws_byt
 //   D=128  B=2 S=4352 H=24  514 / 491, 492 / 473     B=2 S=4096 H=24  429 / 420, 407 / 402
 //          B=1 S=4608 H=24  302 / 297, 289 / 288     B=2 S=32760 H=40  38910 / 38616, 37053 / 36483
 //   D=64   B=2 S=4352 H=24  326 / 334, 316 / 328
-// so head size 128 takes 8 and head size 64 stays at 4. (With the two halves' roles paired wrongly, wavefronts w and
+// so head size 128 takes 8 and head size 64 stays at 4 - from 32 key tiles per unit on: the two halves of an
+// 8-wavefront workgroup begin and end their unit together, so the unit's fixed cost (first tiles fetched cold,
+// first scores, the store) is not hidden behind another workgroup's tiles as it is with two independent workgroups
+// per compute unit, and with few tiles per unit that costs more than the anti-phase gains (B=2, 16384 queries,
+// 24 heads, 4 / 8 wavefronts: 512 keys 300 / 334 us, 1024 keys 469 / 496, 2048 keys 823 / 823; Wan's cross-attention,
+// 32760 queries x 512 keys x 40 heads, 901 / 947). (With the two halves' roles paired wrongly, wavefronts w and
 // w + 1 or w and w + 2 in anti-phase instead of w and w + 4, the same kernel is 10 to 18 % slower: two wavefronts of a
 // SIMD in the same stage is what costs, and independent workgroups already avoid it most of the time by themselves.)
 // ODIT_ATTN_WAVES in the environment, read at the first attention launch, overrides the choice (for measurements).
-static int dma_waves(int D) {
+static int dma_waves(int D, int Sk) {
   static const int forced = [] {
     const char* e = getenv("ODIT_ATTN_WAVES");
     const int v = e != nullptr ? atoi(e) : 0;
     return (v == 4 || v == 8) ? v : 0;
   }();
   if (forced != 0) return forced;
-  return D == 128 ? 8 : 4;
+  return (D == 128 && Sk >= 32 * 64) ? 8 : 4;
 }
 
 size_t attn_dma_workspace_bytes(int B, int Sq, int Sk, int H, int D) {
   if (B <= 0 || Sq <= 0 || Sk <= 0 || H <= 0) return 0;
-  const int nw = dma_waves(D);
+  const int nw = dma_waves(D, Sk);
   const int bm = nw * 32;
   const int64_t units = static_cast<int64_t>((Sq + bm - 1) / bm) * H * B;
   const int n_tiles = (Sk + 63) / 64, slots = device_slots(nw);
@@ -784,7 +789,7 @@ bool attn_dma_addressable(int Sk, int D, int64_t k_seq_stride, int64_t v_seq_str
 }
 
 int attn_dma_plan(int B, int Sq, int Sk, int H, int D, bool with_workspace, char* text, size_t text_bytes) {
-  const int nw = dma_waves(D), bm = nw * 32;
+  const int nw = dma_waves(D, Sk), bm = nw * 32;
   const int64_t units = static_cast<int64_t>((Sq + bm - 1) / bm) * H * B;
   const int n_tiles = (Sk + 63) / 64, slots = device_slots(nw);
   TailPlan t{0, 1, 0};
@@ -813,7 +818,7 @@ int attn_dma_plan(int B, int Sq, int Sk, int H, int D, bool with_workspace, char
 int launch_attn_dma(AttnParams& p, int dtype, int D, hipStream_t stream, void* ws, size_t ws_bytes) {
   if (!attn_dma_addressable(p.Sk, D, p.ks_s, p.vs_s)) return ODIT_ENOTSUP;
 #define ODIT_DMA_GO(T)                                                                     \
-  if (dma_waves(D) == 8) {                                                                  \
+  if (dma_waves(D, p.Sk) == 8) {                                                                  \
     if (D == 128) return launch_dma<T, 128, 8>(p, stream, ws, ws_bytes);                   \
     return launch_dma<T, 64, 8>(p, stream, ws, ws_bytes);                                  \
   }                                                                                        \
