@@ -17,7 +17,8 @@
 //
 // Everything else (transposed S^T = K Q^T / O^T = V^T P^T formulation, one query per lane, lazy
 // rescale, stage A = next-tile QK^T MFMAs interleaved with this tile's exp2 work, stage B = PV, one
-// barrier per tile, XCD-aware workgroup order) is as in attn_fwd_pipe_kernel.
+// barrier per tile - two in the anti-phase form of 8 wavefronts, see NW below -, XCD-aware workgroup order)
+// is as in attn_fwd_pipe_kernel.
 //
 // Persistent form (MODE 2), a measurement aid that no default launch uses (ODIT_ATTN_PERSISTENT=1 in the
 // environment turns it on). With more units than workgroup slots the launch has as many workgroups as run at
@@ -35,11 +36,16 @@
 //   B=2 S=4352 H=24 (3.19 rounds)  506 / 532      B=2 S=4096 H=24 (3.00 rounds)  433 / 447
 //   B=1 S=4608 H=24 (1.69 rounds)  306 / 316      B=2 S=32760 H=40 (40 rounds)   39709 / 41187
 // i.e. 3 to 5 % slower everywhere, also at 40 units per workgroup where the boundaries no longer matter: the
-// steady-state tile loop itself is slower (it carries the next unit's state and the boundary's branches, and
-// needs all 256 vector registers where MODE 0 needs 235), and that costs more than the boundaries save. With a
-// fixed assignment of units (w, w + W, ...) instead of the ticket words it was 6 % slower: compute units do
-// not all run at one speed, and the dispatcher (or the tickets) gives the faster ones more work. Neither form
-// removes the cost of a last round that is partly filled: that needs units cut along the keys (MODE 1).
+// steady-state tile loop itself is slower. It carries the next unit's state and the boundary's branches in 97 of
+// 102 scalar registers, so the tile loads' LDS destinations and the fragment addresses are formed again in every
+// tile instead of being held: the hardware counters show 5.77 vector instructions per MFMA against 4.82 and the
+// matrix pipe busy 50.8 % of the cycles against 57.0 %. And what it saves is little: at 8 key tiles per unit, where
+// a unit's fixed cost (8 us: dispatch, cold first tiles, first scores, store) is a third of the unit, it runs in
+// the time of one workgroup per unit (899 / 901 us at 32760 queries x 512 keys x 40 heads), so its boundary costs
+// what a dispatch and a cold start cost. With a fixed assignment of units (w, w + W, ...) instead of the ticket
+// words it was 6 % slower: compute units do not all run at one speed, and the dispatcher (or the tickets) gives
+// the faster ones more work. Neither form removes the cost of a last round that is partly filled: that needs
+// units cut along the keys (MODE 1).
 #include <stddef.h>
 
 #include <cstdlib>
