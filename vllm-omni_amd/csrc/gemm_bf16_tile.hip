@@ -39,7 +39,11 @@
 // (ODIT_TILE_ABLATE): matrix instructions alone 390, plus fragment reads 483, plus tile loads instead 517,
 // tile loads and barrier without any matrix instruction 495 - the two kinds of LDS traffic add up instead of
 // hiding behind the matrix pipe. The library's kernel for the same tile runs four waves with 128 x 128 corners
-// (128 KB of fragment reads per step) at 76 % matrix-pipe busy against 56 % here.
+// (128 KB of fragment reads per step) at 76 % matrix-pipe busy against 56 % here. That layout was also built with
+// the 256 accumulators at fixed accumulation registers named in one-instruction inline assembly (no register
+// allocation problem left: 102 vector registers, no scratch, same results): 560 us with the tile loads going
+// through registers, 610 direct to LDS, and 405 us = 1.53 PFLOP/s with no tile traffic at all - the fetches from
+// L2, not LDS and not the matrix pipe, are what separates both layouts from the library.
 #include <type_traits>
 
 #include "gemm_epilogue.h"
@@ -200,6 +204,21 @@ __global__ __launch_bounds__(WM * 2 * 64) __attribute__((amdgpu_waves_per_eu(WM 
   };
 
   const int nk = p.k_steps;
+  // The reduction starts at a different step in every row tile and wraps around: the rows of x and W are a
+  // multiple of 4 KB apart for the usual reduction lengths, so at one reduction offset every row of a tile sits in
+  // the same memory channel, and workgroups that all stand at the same offset queue up in front of it. Row tiles
+  // 256 bytes (two steps) apart spread over the channels; the feature tiles of one row tile keep the same offset,
+  // so they still find each other's x pieces in L2. Worth 0 to 5 % (M = 8192, us without / with: N=9216 K=3072
+  // 430 / 406, N=3072 K=12288 630 / 613, N=12288 K=3072 567 / 568); what such strides really cost shows when the
+  // rows are padded by 128 bytes instead: 628 -> 509 us at K=12288, 536 -> 506 at K=3072 (hipBLASLt's kernels are
+  // indifferent to it). Sums are formed in the rotated order.
+  constexpr int kStagger = 32;
+  const int stagger = ((mt % kStagger) * 2) % nk;
+  auto wrapk = [&](int j) {   // reduction step of the j-th step this workgroup runs (j < nk + 3)
+    int t = j + stagger;
+    t = t >= nk ? t - nk : t;
+    return t >= nk ? t - nk : t;
+  };
   // A step's tile loads go out in two halves, each spread over the matrix instructions of one k16 slice (the
   // texture addresser takes a wave instruction every 16 cycles: issued faster, the loads fill its queue and the
   // wave, which issues in order, stalls in front of its next matrix instruction): the first half of step i + 2
@@ -209,9 +228,9 @@ __global__ __launch_bounds__(WM * 2 * 64) __attribute__((amdgpu_waves_per_eu(WM 
     const int n = i1 - i0, a = i0 + n * part / parts, b = i0 + n * (part + 1) / parts;
     issue(kk, stage, a, b);
   };
-  issue(0, 0, 0, IPW);
+  issue(wrapk(0), 0, 0, IPW);
   if (nk > 1) {
-    issue(1, 1, 0, H0);
+    issue(wrapk(1), 1, 0, H0);
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(H0) : "memory");
   } else {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -232,7 +251,7 @@ __global__ __launch_bounds__(WM * 2 * 64) __attribute__((amdgpu_waves_per_eu(WM 
         // slice 0 carries the second half of step i + 1's tile loads, a few per group of matrix instructions
 #pragma unroll
         for (int tn = 0; tn < NT; ++tn) {
-          if (next) issue_spread(i + 1, stage ^ 1, H0, IPW, tn, NT);
+          if (next) issue_spread(wrapk(i + 1), stage ^ 1, H0, IPW, tn, NT);
           if (!(ODIT_TILE_ABLATE & 2))
 #pragma unroll
             for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = M::run(wf[0][tn], xf[0][tm], acc[tn][tm]);
@@ -263,7 +282,7 @@ __global__ __launch_bounds__(WM * 2 * 64) __attribute__((amdgpu_waves_per_eu(WM 
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int tn = 0; tn < NT; ++tn) {
-      if (more && !(ODIT_TILE_ABLATE & 1)) issue_spread(i + 2, stage, 0, H0, tn, NT);
+      if (more && !(ODIT_TILE_ABLATE & 1)) issue_spread(wrapk(i + 2), stage, 0, H0, tn, NT);
       if (!(ODIT_TILE_ABLATE & 2))
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = M::run(wf[1][tn], xf[1][tm], acc[tn][tm]);
