@@ -99,9 +99,9 @@ int odit_attn_fwd(const void* q, const void* k, const void* v, void* o, const ui
  * GPU, where the unsplit launch leaves most of the GPU idle. NULL = never split. Results with and
  * without scratch agree to rounding (the merge re-associates the key sum); for given shapes and device
  * the partition is fixed, so repeated calls are bit-identical. No counterpart in the reference.
- * The first 1024 bytes of the scratch belong to a measurement mode (ODIT_ATTN_PERSISTENT=1 in the
- * environment when the library makes its first attention launch: as many workgroups as run at once, each
- * drawing unit after unit from ticket words there). That mode alone needs those bytes zero before the first
+ * The first 1024 bytes of the scratch belong to a measurement mode (ODIT_ATTN_PERSISTENT=1 and
+ * ODIT_ATTN_WAVES=4 in the environment when the library makes its first attention launch: as many workgroups
+ * of 4 wavefronts as run at once, each drawing unit after unit from ticket words there). That mode alone needs those bytes zero before the first
  * call that uses the buffer and leaves them zero; no default launch reads or writes them.
  *
  * v_tail == NULL, o_tail == NULL and workspace == NULL behaves exactly like odit_attn_fwd.

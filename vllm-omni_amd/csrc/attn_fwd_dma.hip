@@ -21,7 +21,7 @@
 // is as in attn_fwd_pipe_kernel.
 //
 // Persistent form (MODE 2), a measurement aid that no default launch uses (ODIT_ATTN_PERSISTENT=1 in the
-// environment turns it on). With more units than workgroup slots the launch has as many workgroups as run at
+// environment turns it on for launches of 4-wavefront workgroups, i.e. with ODIT_ATTN_WAVES=4 at head size 128). With more units than workgroup slots the launch has as many workgroups as run at
 // once, and each runs unit after unit as ONE stream of key tiles: the tile pipeline runs across the unit
 // boundary. Units are handed out dynamically: every XCD owns a contiguous eighth of the units (neighbours in
 // (q block, head) order share keys and values in its L2), its workgroups start on the first ones and draw the
