@@ -613,6 +613,7 @@ def counter_probe(torch, kernels, dev):
         kernels.gated_residual(x, y, gate, out=o)
         kernels.rel_l1_sums(x, y)
         kernels.linear(x2, w_up, b_up, activation="gelu_tanh")
+        kernels.linear(x2, w_up, b_up, activation="gelu_tanh", engine="handwritten")   # the tile kernel on the same problem
         torch.nn.functional.linear(x2, w_qkv, b_qkv)
         kernels.linear(t_in, w_dn, None, residual=t_res, gate=g32, gate_bias=g32 * 0.1, prescaled=True)
     torch.cuda.synchronize()
